@@ -1,0 +1,128 @@
+/*
+ * s2attn: spherical neighborhood attention (gather direction) for AMD gfx950.
+ *
+ * Plain C ABI of libs2attn.so.  No torch types cross this boundary: device
+ * buffers are raw pointers, sizes are ints, the stream is a hipStream_t passed
+ * as void*.  Every entry point returns S2ATTN_OK (0) or a negative S2ATTN_E_*
+ * code; s2attn_last_error() returns the message of the last failure on the
+ * calling thread.  Nothing here allocates or frees device memory and nothing
+ * synchronises the stream.
+ *
+ * Tensor contract (same as the reference ops, attention_interface.cpp:85-119):
+ *   k  [B, nlat_in,  nlon_in,  num_heads*ck]   v  [B, nlat_in,  nlon_in,  num_heads*cv]
+ *   q  [B, nlat_out, nlon_out, num_heads*ck]   y, dy [B, nlat_out, nlon_out, num_heads*cv]
+ * physical NHWC, contiguous, heads packed along the channel axis, one storage
+ * dtype for all activations; quad_weights [nlat_in] fp32; q arrives already
+ * multiplied by the softmax scale.  nlon_in must be a multiple of nlon_out.
+ */
+#ifndef S2ATTN_H
+#define S2ATTN_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define S2ATTN_OK 0
+#define S2ATTN_E_INVALID (-1)     /* bad shape, dtype, null pointer, psi entry out of range */
+#define S2ATTN_E_UNSUPPORTED (-2) /* a shape the kernels are not instantiated for */
+#define S2ATTN_E_LAUNCH (-3)      /* HIP reported an error at launch */
+
+/* storage dtype of k, v, q, y, dy, dk, dv, dq */
+#define S2ATTN_F32 0
+#define S2ATTN_BF16 1
+#define S2ATTN_F16 2
+
+const char *s2attn_last_error(void);
+
+/* Library version, bumped when the ABI below changes. */
+int s2attn_abi_version(void);
+
+/*
+ * Neighborhood plan.  The reference kernels walk the CSR neighborhood
+ * (row_off[nlat_out+1], col_idx[nnz], col = hi*nlon_in + wi at output longitude 0)
+ * entry by entry and re-sort its rows by length on every call
+ * (attention_cuda_utils.cu:74-113, called from attention_cuda_fwd.cu:476 and
+ * attention_cuda_bwd.cu:792).  This library instead converts the CSR once, on the
+ * host, into runs of consecutive longitudes:
+ *
+ *   run = (lat, ws, len, 0)   four int32
+ *
+ * gather runs   grouped by output latitude ho:  lat = hi, neighbors (hi, (ws + t + pscale*wo) mod nlon_in), t in [0, len)
+ * scatter runs  the same runs grouped by input latitude hi: lat = ho
+ *
+ * plus, for each grouping, the group offsets and the groups ordered by
+ * decreasing work (longest first), which is the launch order of the kernels.
+ * Any CSR is representable (worst case every entry is its own run).
+ *
+ * s2attn_plan_count   number of runs the CSR decomposes into, or a negative error.
+ * s2attn_plan_build   fills caller-allocated host arrays:
+ *     gather_off  [nlat_out+1]   gather_runs  [4*nruns]   gather_order  [nlat_out]
+ *     scatter_off [nlat_in+1]    scatter_runs [4*nruns]   scatter_order [nlat_in]
+ * The caller copies the six arrays to the device and passes them in s2attn_plan.
+ */
+int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                          int nlat_out, int nlon_out);
+
+int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                      int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
+                      int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order);
+
+typedef struct s2attn_plan {
+    const int32_t *gather_off;    /* device, [nlat_out+1] */
+    const int32_t *gather_runs;   /* device, [4*nruns]    */
+    const int32_t *gather_order;  /* device, [nlat_out]   */
+    const int32_t *scatter_off;   /* device, [nlat_in+1]  (backward only) */
+    const int32_t *scatter_runs;  /* device, [4*nruns]    (backward only) */
+    const int32_t *scatter_order; /* device, [nlat_in]    (backward only) */
+    int64_t nruns;
+} s2attn_plan;
+
+typedef struct s2attn_shape {
+    int batch, num_heads;
+    int nlat_in, nlon_in, nlat_out, nlon_out;
+    int ck; /* per-head channels of q and k */
+    int cv; /* per-head channels of v and y */
+    int dtype;
+} s2attn_shape;
+
+/*
+ * Forward.  Replaces attention_kernels::forward (attention_interface.cpp:114-116;
+ * CUDA implementation s2_attention_fwd_cuda, attention_cuda_fwd.cu:539-633).
+ *   y = sum_j a_j v_j / sum_j a_j,  a_j = exp(q.k_j - max) * quad_weights[hi_j]
+ * y must not alias an input.
+ */
+int s2attn_forward(const void *k, const void *v, const void *q, const float *quad_weights, void *y,
+                   const s2attn_plan *plan, const s2attn_shape *shape, void *stream);
+
+/*
+ * Backward.  Replaces attention_kernels::backward (attention_interface.cpp:117-119;
+ * CUDA implementation s2_attention_bwd_dkvq_cuda, attention_cuda_bwd.cu:856-956).
+ * Writes dk, dv, dq (every element; no pre-zeroing needed, no atomics).
+ * workspace: device fp32 scratch of s2attn_backward_workspace_bytes(shape) bytes
+ * holding two softmax statistics per (batch, head, output point).
+ */
+int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape);
+
+int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, void *dk,
+                    void *dv, void *dq, void *workspace, const s2attn_plan *plan, const s2attn_shape *shape,
+                    void *stream);
+
+/*
+ * Layout conversion.  Replace attention_kernels::permute_to_nhwc / permute_to_nchw
+ * (attention_interface.cpp:85-86; CUDA kernels attention_cuda_utils.cuh:417-576).
+ * Pure element moves; elem_size is 2 or 4 bytes.  dst must not alias src.
+ *   to_nhwc: src [B, C, H, W] -> dst [B, H, W, C]
+ *   to_nchw: src [B, H, W, C] -> dst [B, C, H, W]
+ */
+int s2attn_permute_to_nhwc(const void *src, void *dst, int64_t B, int64_t C, int64_t H, int64_t W, int elem_size,
+                           void *stream);
+int s2attn_permute_to_nchw(const void *src, void *dst, int64_t B, int64_t H, int64_t W, int64_t C, int elem_size,
+                           void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* S2ATTN_H */

@@ -1,0 +1,129 @@
+"""
+GPU parity of the HIP path against the CPU oracle, called through the C ABI (ctypes) via the
+package's operators.  Tolerances: fp32 rtol = atol = 1e-5; bf16/fp16 2e-2 relative to the
+tensor's scale (fp32 accumulation inside the kernels).
+"""
+
+import math
+
+import pytest
+import torch
+
+from oracle import cpu_attention as oracle
+from oracle import geometry as ogeo
+from tests.util import assert_close, randn_inputs
+
+pytestmark = pytest.mark.gpu
+
+F32_TOL = dict(rtol=1e-5, atol=1e-5)
+
+
+def _psi(in_shape, out_shape, grid_in, grid_out, theta_cutoff):
+    col_idx, row_off = ogeo.neighborhood_csr(in_shape, out_shape, grid_in, grid_out, theta_cutoff)
+    quad = ogeo.attention_quad_weights(in_shape[0], in_shape[1], grid_in)
+    return col_idx, row_off, quad
+
+
+def _run_hip(k, v, q, dy, quad, col_idx, row_off, nh, dtype=torch.float32):
+    from torch_harmonics_amd import ops
+
+    dev = torch.device("cuda", 0)
+    kd, vd, qd, gd = [t.to(device=dev, dtype=dtype) for t in (k, v, q, dy)]
+    wd, cd, rd = quad.to(dev), col_idx.to(dev), row_off.to(dev)
+    Wi, Ho, Wo = k.shape[2], q.shape[1], q.shape[2]
+    y = ops.forward(kd, vd, qd, wd, cd, rd, nh, Wi, Ho, Wo)
+    dk, dv, dq = ops.backward(kd, vd, qd, gd, wd, cd, rd, nh, Wi, Ho, Wo)
+    torch.cuda.synchronize()
+    return y, dk, dv, dq
+
+
+# (B, nh, ck, cv, in_shape, out_shape, grid_in, grid_out, theta_cutoff): the reference's own shape matrix
+# (tests/test_attention.py:86-110, gather rows) plus head dims that exercise every kernel width
+SMALL_CASES = [
+    (4, 1, 4, 4, (6, 12), (6, 12), "equiangular", "equiangular", None),
+    (4, 2, 2, 2, (6, 12), (6, 12), "equiangular", "equiangular", None),
+    (4, 4, 1, 1, (6, 12), (6, 12), "equiangular", "equiangular", None),
+    (4, 4, 1, 2, (6, 12), (6, 12), "equiangular", "equiangular", None),
+    (4, 4, 2, 1, (6, 12), (6, 12), "equiangular", "equiangular", None),
+    (4, 1, 1, 1, (2, 4), (2, 4), "equiangular", "equiangular", None),
+    (4, 1, 1, 4, (2, 4), (2, 4), "equiangular", "equiangular", None),
+    (4, 4, 1, 1, (6, 12), (6, 12), "legendre-gauss", "legendre-gauss", None),
+    (4, 1, 4, 4, (6, 12), (6, 12), "lobatto", "lobatto", None),
+    (4, 4, 2, 1, (12, 24), (6, 12), "equiangular", "equiangular", None),
+    (4, 4, 1, 2, (12, 24), (6, 12), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (6, 12), (6, 6), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (12, 24), (6, 8), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (12, 24), (3, 6), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (12, 12), (6, 12), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (12, 24), (6, 12), "legendre-gauss", "legendre-gauss", None),
+    (4, 1, 4, 4, (7, 12), (5, 6), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (9, 12), (5, 4), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (11, 24), (7, 12), "equiangular", "equiangular", None),
+    (4, 1, 4, 4, (12, 24), (11, 24), "equiangular", "equiangular", None),
+    (2, 2, 8, 8, (12, 24), (12, 24), "equiangular", "equiangular", 0.5),
+    (2, 2, 16, 16, (16, 32), (16, 32), "equiangular", "equiangular", 0.4),
+    (1, 2, 32, 32, (16, 32), (16, 32), "legendre-gauss", "legendre-gauss", 0.4),
+    (1, 2, 32, 16, (24, 48), (12, 24), "equiangular", "legendre-gauss", 0.5),
+    (1, 1, 3, 5, (10, 20), (10, 20), "equiangular", "equiangular", 0.7),
+    (1, 3, 12, 20, (10, 20), (5, 10), "equiangular", "equiangular", 0.9),
+    (1, 1, 16, 16, (12, 160), (12, 160), "equiangular", "equiangular", 0.3),
+    (1, 1, 8, 8, (10, 200), (10, 100), "equiangular", "equiangular", 0.35),
+    (2, 1, 4, 4, (6, 12), (6, 12), "equiangular", "equiangular", 7.0),
+]
+
+
+@pytest.mark.parametrize("case", SMALL_CASES, ids=lambda c: f"B{c[0]}h{c[1]}ck{c[2]}cv{c[3]}_{c[4][0]}x{c[4][1]}to{c[5][0]}x{c[5][1]}_{c[6][:3]}")
+def test_small_shapes_fp32(case):
+    B, nh, ck, cv, ins, outs, gi, go, tc = case
+    print(f"case {case}", flush=True)
+    col_idx, row_off, quad = _psi(ins, outs, gi, go, tc)
+    k, v, q, dy = randn_inputs(B, ins[0], ins[1], outs[0], outs[1], nh, ck, cv)
+    y, dk, dv, dq = _run_hip(k, v, q, dy, quad, col_idx, row_off, nh)
+    y32 = oracle.forward_f32(k, v, q, quad, col_idx, row_off, nh)
+    dk32, dv32, dq32 = oracle.backward_f32(k, v, q, dy, quad, col_idx, row_off, nh)
+    y64 = oracle.forward_f64(k, v, q, quad, col_idx, row_off, nh)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, quad, col_idx, row_off, nh)
+    for name, got, w32, w64 in (("y", y, y32, y64), ("dk", dk, dk32, dk64), ("dv", dv, dv32, dv64), ("dq", dq, dq32, dq64)):
+        assert_close(name + " vs fp32 oracle", got, w32, **F32_TOL)
+        assert_close(name + " vs fp64 spec", got, w64, **F32_TOL)
+
+
+def test_cfg1_full():
+    """32x64 self-attention, B=1, C=16, one head, default cutoff: the CPU-runnable benchmark case, in full."""
+    ins = outs = (32, 64)
+    col_idx, row_off, quad = _psi(ins, outs, "equiangular", "equiangular", None)
+    k, v, q, dy = randn_inputs(1, 32, 64, 32, 64, 1, 16, 16)
+    y, dk, dv, dq = _run_hip(k, v, q, dy, quad, col_idx, row_off, 1)
+    y32 = oracle.forward_f32(k, v, q, quad, col_idx, row_off, 1)
+    dk32, dv32, dq32 = oracle.backward_f32(k, v, q, dy, quad, col_idx, row_off, 1)
+    for name, got, want in (("y", y, y32), ("dk", dk, dk32), ("dv", dv, dv32), ("dq", dq, dq32)):
+        assert_close(name, got, want, **F32_TOL)
+
+
+def test_cfg2_reduced_batch():
+    """128x256, 4 heads of 16, cutoff 4 spacings; batch 1 of 4 so that the reference CPU backward's scratch (1.3 GB) fits."""
+    ins = outs = (128, 256)
+    col_idx, row_off, quad = _psi(ins, outs, "equiangular", "equiangular", 4 * math.pi / 127)
+    k, v, q, dy = randn_inputs(1, 128, 256, 128, 256, 4, 16, 16)
+    y, dk, dv, dq = _run_hip(k, v, q, dy, quad, col_idx, row_off, 4)
+    y32 = oracle.forward_f32(k, v, q, quad, col_idx, row_off, 4)
+    assert_close("y", y, y32, **F32_TOL)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, quad, col_idx, row_off, 4)
+    for name, got, want in (("dk", dk, dk64), ("dv", dv, dv64), ("dq", dq, dq64)):
+        assert_close(name, got, want, **F32_TOL)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float16, 2e-2)], ids=["bf16", "fp16"])
+def test_reduced_precision_storage(dtype, tol):
+    """16-bit storage, fp32 softmax and accumulation: error relative to each tensor's RMS within 2e-2."""
+    ins, outs = (24, 48), (24, 48)
+    col_idx, row_off, quad = _psi(ins, outs, "legendre-gauss", "legendre-gauss", 0.35)
+    k, v, q, dy = randn_inputs(2, 24, 48, 24, 48, 2, 32, 32, scale=0.5)
+    k, v, q, dy = [t.to(dtype).float() for t in (k, v, q, dy)]  # the oracle sees exactly the stored values
+    y, dk, dv, dq = _run_hip(k, v, q, dy, quad, col_idx, row_off, 2, dtype=dtype)
+    assert y.dtype == dtype and dk.dtype == dtype and dv.dtype == dtype and dq.dtype == dtype
+    y64 = oracle.forward_f64(k, v, q, quad, col_idx, row_off, 2)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, quad, col_idx, row_off, 2)
+    for name, got, want in (("y", y, y64), ("dk", dk, dk64), ("dv", dv, dv64), ("dq", dq, dq64)):
+        rms = want.pow(2).mean().sqrt().item()
+        assert_close(name, got, want, rtol=tol, atol=tol * rms)

@@ -1,0 +1,112 @@
+"""
+ctypes binding of libs2attn.so (the C ABI in include/s2attn.h).
+
+The library is built in-tree by torch_harmonics_amd/csrc/Makefile.  Loading never
+falls back to anything: if the shared object is missing or a symbol is absent the
+first use raises.
+"""
+
+import ctypes
+import os
+import subprocess
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libs2attn.so")
+
+S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
+ABI_VERSION = 1
+
+_vp = ctypes.c_void_p
+_i64 = ctypes.c_int64
+_int = ctypes.c_int
+
+
+class PlanStruct(ctypes.Structure):
+    _fields_ = [
+        ("gather_off", _vp),
+        ("gather_runs", _vp),
+        ("gather_order", _vp),
+        ("scatter_off", _vp),
+        ("scatter_runs", _vp),
+        ("scatter_order", _vp),
+        ("nruns", _i64),
+    ]
+
+
+class ShapeStruct(ctypes.Structure):
+    _fields_ = [
+        ("batch", _int),
+        ("num_heads", _int),
+        ("nlat_in", _int),
+        ("nlon_in", _int),
+        ("nlat_out", _int),
+        ("nlon_out", _int),
+        ("ck", _int),
+        ("cv", _int),
+        ("dtype", _int),
+    ]
+
+
+# every symbol include/s2attn.h declares: name -> (restype, argtypes)
+SYMBOLS = {
+    "s2attn_last_error": (ctypes.c_char_p, []),
+    "s2attn_abi_version": (_int, []),
+    "s2attn_plan_count": (_i64, [_vp, _vp, _i64, _int, _int, _int, _int]),
+    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_backward_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
+    "s2attn_backward": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_permute_to_nhwc": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "s2attn_permute_to_nchw": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+}
+
+_lib = None
+_lock = threading.Lock()
+
+
+def build(verbose: bool = False) -> str:
+    """Compile libs2attn.so for gfx950 with hipcc (always recompiles)."""
+    csrc = os.path.join(_HERE, "csrc")
+    subprocess.run(["make", "-C", csrc, "clean"], check=True, capture_output=not verbose)
+    proc = subprocess.run(["make", "-C", csrc], capture_output=True, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError(f"building libs2attn.so failed:\n{proc.stdout}\n{proc.stderr}")
+    if verbose:
+        print(proc.stdout)
+    return LIB_PATH
+
+
+def is_built() -> bool:
+    return os.path.exists(LIB_PATH)
+
+
+def load():
+    """Returns the loaded library with typed entry points; raises if it is not built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is not built. Run `make -C {os.path.join(_HERE, 'csrc')}` (needs hipcc); " "this package has no fallback implementation."
+            )
+        lib = ctypes.CDLL(LIB_PATH)
+        for name, (restype, argtypes) in SYMBOLS.items():
+            fn = getattr(lib, name)  # AttributeError if the export is missing
+            fn.restype = restype
+            fn.argtypes = argtypes
+        got = lib.s2attn_abi_version()
+        if got != ABI_VERSION:
+            raise RuntimeError(f"libs2attn.so has ABI version {got}, this package expects {ABI_VERSION}; rebuild it")
+        _lib = lib
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    """Turns a negative return code into a RuntimeError carrying the library's message."""
+    if rc < 0:
+        msg = load().s2attn_last_error()
+        raise RuntimeError(f"{what}: {msg.decode() if msg else f'error {rc}'}")

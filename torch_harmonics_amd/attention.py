@@ -1,0 +1,196 @@
+"""
+NeighborhoodAttentionS2: attention restricted to a geodesic disk around every output point of
+a spherical grid, weighted by the grid's quadrature.
+
+Constructor arguments, parameter names and shapes, buffers and forward semantics follow
+torch_harmonics/attention/attention.py:253-571 so that a state_dict moves between the two
+implementations unchanged.  The attention itself runs in the HIP kernels of libs2attn.so.
+"""
+
+import math
+from typing import Optional, Tuple, Union
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from ._attention_utils import _check_dtypes_match, _check_extent, _check_ndim
+from ._layout import to_nchw, to_nhwc
+from .neighborhood import precompute_neighborhood_s2
+from .ops import _neighborhood_s2_attention_optimized
+from .quadrature import precompute_latitudes
+
+__all__ = ["NeighborhoodAttentionS2"]
+
+
+def _xavier_uniform(c_out: int, c_in: int, bound: float) -> nn.Parameter:
+    return nn.Parameter(bound * (2 * torch.rand(c_out, c_in, 1, 1) - 1))
+
+
+class NeighborhoodAttentionS2(nn.Module):
+    r"""
+    Neighborhood attention on the 2-sphere.
+
+    Each output point :math:`x` attends to the input points inside the disk
+    :math:`\{x' : d(x, x') \le \theta_\mathrm{cutoff}\}` (great-circle distance); the softmax is
+    a quadrature of the continuous attention integral, i.e. every neighbor's weight is multiplied
+    by the quadrature weight of its latitude ring.
+
+    Parameters
+    ----------
+    in_channels : int
+        channels of the input signal
+    in_shape, out_shape : (nlat, nlon)
+        input (key/value) and output (query) grids; ``nlon_in`` must be a multiple of ``nlon_out``
+    grid_in, grid_out : str
+        ``"equiangular"``, ``"legendre-gauss"``, ``"lobatto"`` or ``"equiangular-trapezoidal"``
+    num_heads : int
+        attention heads; must divide ``k_channels`` and ``out_channels``
+    scale : float or Tensor, optional
+        multiplies the query; default ``1 / sqrt(k_channels // num_heads)``
+    use_qknorm : bool
+        per-head RMS normalisation of q and k with learnable gain ``1 + w``
+    bias : bool
+        bias on the four 1x1 projections
+    theta_cutoff : float, optional
+        disk radius in radians; default one latitude spacing of the output grid, ``pi / (nlat_out - 1)``
+    k_channels, out_channels : int, optional
+        width of the q/k projection and of the v/output projection; default ``in_channels``
+    optimized_kernel : bool
+        must stay True: the HIP kernels are the only implementation in this package
+    """
+
+    def __init__(
+        self,
+        in_channels: int,
+        in_shape: Tuple[int],
+        out_shape: Tuple[int],
+        grid_in: Optional[str] = "equiangular",
+        grid_out: Optional[str] = "equiangular",
+        num_heads: Optional[int] = 1,
+        scale: Optional[Union[torch.Tensor, float]] = None,
+        use_qknorm: Optional[bool] = False,
+        bias: Optional[bool] = True,
+        theta_cutoff: Optional[float] = None,
+        k_channels: Optional[int] = None,
+        out_channels: Optional[int] = None,
+        optimized_kernel: Optional[bool] = True,
+    ):
+        super().__init__()
+
+        self.nlat_in, self.nlon_in = in_shape
+        self.nlat_out, self.nlon_out = out_shape
+
+        self.upsample = (self.nlon_out % self.nlon_in == 0) and (self.nlon_in % self.nlon_out != 0)
+        if not (self.nlon_in % self.nlon_out == 0 or self.upsample):
+            raise ValueError(f"either nlon_in ({self.nlon_in}) must be an integer multiple of nlon_out ({self.nlon_out}), or vice versa, for the attention p-shift to be exact")
+        if self.upsample:
+            raise NotImplementedError("upsampling attention (nlon_out > nlon_in) is not implemented by the HIP kernels")
+        if not optimized_kernel:
+            raise NotImplementedError("optimized_kernel=False selects a pure-PyTorch loop in the reference; this package ships the HIP kernels only")
+        self.optimized_kernel = True
+
+        self.in_channels = in_channels
+        self.num_heads = num_heads
+        self.k_channels = in_channels if k_channels is None else k_channels
+        self.out_channels = in_channels if out_channels is None else out_channels
+
+        self.theta_cutoff = torch.pi / float(self.nlat_out - 1) if theta_cutoff is None else theta_cutoff
+        if self.theta_cutoff <= 0.0:
+            raise ValueError("Error, theta_cutoff has to be positive.")
+
+        if self.k_channels % self.num_heads != 0:
+            raise ValueError(f"Please make sure that number of heads {self.num_heads} divides k_channels {self.k_channels} evenly.")
+        if self.out_channels % self.num_heads != 0:
+            raise ValueError(f"Please make sure that number of heads {self.num_heads} divides out_channels {self.out_channels} evenly.")
+
+        # quadrature weight of every input latitude ring, normalised so that the rings sum to 4 pi
+        _, wgl = precompute_latitudes(self.nlat_in, grid=grid_in)
+        self.register_buffer("quad_weights", 2.0 * torch.pi * wgl.to(dtype=torch.float32) / self.nlon_in, persistent=False)
+
+        col_idx, row_off, row_idx = precompute_neighborhood_s2(in_shape, out_shape, grid_in=grid_in, grid_out=grid_out, theta_cutoff=self.theta_cutoff)
+        self.register_buffer("psi_row_idx", row_idx, persistent=False)
+        self.register_buffer("psi_col_idx", col_idx, persistent=False)
+        self.register_buffer("psi_roff_idx", row_off, persistent=False)
+
+        # projections are 1x1; stored in convolution shape, drawn in the order q, k, v, proj
+        bound_qk = math.sqrt(6.0 / (self.in_channels + self.k_channels))
+        bound_v = math.sqrt(6.0 / (self.in_channels + self.out_channels))
+        bound_proj = math.sqrt(3.0 / self.out_channels)
+        self.q_weights = _xavier_uniform(self.k_channels, self.in_channels, bound_qk)
+        self.k_weights = _xavier_uniform(self.k_channels, self.in_channels, bound_qk)
+        self.v_weights = _xavier_uniform(self.out_channels, self.in_channels, bound_v)
+        self.proj_weights = _xavier_uniform(self.out_channels, self.out_channels, bound_proj)
+
+        self.scale = scale if scale is not None else 1 / math.sqrt(self.k_channels // self.num_heads)
+
+        if bias:
+            self.q_bias = nn.Parameter(torch.zeros(self.k_channels))
+            self.k_bias = nn.Parameter(torch.zeros(self.k_channels))
+            self.v_bias = nn.Parameter(torch.zeros(self.out_channels))
+            self.proj_bias = nn.Parameter(torch.zeros(self.out_channels))
+        else:
+            self.q_bias = self.k_bias = self.v_bias = self.proj_bias = None
+
+        if use_qknorm:
+            self.q_norm_weights = nn.Parameter(torch.zeros(self.k_channels // self.num_heads))
+            self.k_norm_weights = nn.Parameter(torch.zeros(self.k_channels // self.num_heads))
+        else:
+            self.q_norm_weights = self.k_norm_weights = None
+
+        self.attention_handle = _neighborhood_s2_attention_optimized
+
+    def extra_repr(self):
+        return (
+            f"in_shape={(self.nlat_in, self.nlon_in)}, out_shape={(self.nlat_out, self.nlon_out)}, in_channels={self.in_channels}, "
+            f"out_channels={self.out_channels}, k_channels={self.k_channels}, theta_cutoff={self.theta_cutoff}"
+        )
+
+    def _head_rms_norm(self, x: torch.Tensor, gain: torch.Tensor) -> torch.Tensor:
+        B, H, W, C = x.shape
+        x = x.reshape(B, H, W, self.num_heads, -1)
+        x = F.rms_norm(x, normalized_shape=gain.shape, weight=1 + gain)
+        return x.reshape(B, H, W, C)
+
+    def forward(self, query: torch.Tensor, key: Optional[torch.Tensor] = None, value: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """
+        query : (B, in_channels, nlat_out, nlon_out); key, value : (B, in_channels, nlat_in, nlon_in), both
+        default to ``query`` (self-attention).  Returns (B, out_channels, nlat_out, nlon_out).
+        """
+        if key is None:
+            key = query
+        if value is None:
+            value = query
+
+        _check_ndim(query, 4, "query")
+        _check_ndim(key, 4, "key")
+        _check_ndim(value, 4, "value")
+        _check_dtypes_match((query, key, value))
+        _check_extent(query, -2, self.nlat_out, "query latitudes")
+        _check_extent(query, -1, self.nlon_out, "query longitudes")
+        _check_extent(key, -2, self.nlat_in, "key latitudes")
+        _check_extent(key, -1, self.nlon_in, "key longitudes")
+        _check_extent(value, -2, self.nlat_in, "value latitudes")
+        _check_extent(value, -1, self.nlon_in, "value longitudes")
+
+        # one channels-last conversion per distinct input tensor; everything after is NHWC
+        key_is_query, value_is_query, value_is_key = key is query, value is query, value is key
+        query = to_nhwc(query)
+        key = query if key_is_query else to_nhwc(key)
+        value = query if value_is_query else (key if value_is_key else to_nhwc(value))
+
+        query = F.linear(query, self.q_weights.view(self.q_weights.shape[0], -1), self.q_bias)
+        key = F.linear(key, self.k_weights.view(self.k_weights.shape[0], -1), self.k_bias)
+        value = F.linear(value, self.v_weights.view(self.v_weights.shape[0], -1), self.v_bias)
+
+        if self.q_norm_weights is not None:
+            query = self._head_rms_norm(query, self.q_norm_weights)
+        if self.k_norm_weights is not None:
+            key = self._head_rms_norm(key, self.k_norm_weights)
+
+        out = self.attention_handle(
+            key, value, query * self.scale, self.quad_weights, self.psi_col_idx, self.psi_roff_idx, self.num_heads, self.nlon_in, self.nlat_out, self.nlon_out
+        )
+
+        out = F.linear(out, self.proj_weights.view(self.proj_weights.shape[0], -1), self.proj_bias)
+        return to_nchw(out)

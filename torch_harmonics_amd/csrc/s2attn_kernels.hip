@@ -1,0 +1,776 @@
+// Spherical neighborhood attention on gfx950: forward, dq and dk/dv kernels, layout
+// permutes, and the C entry points declared in include/s2attn.h.
+//
+// Work decomposition (all three attention kernels)
+//   One wavefront (= one workgroup of 64 threads) owns 64 consecutive longitudes of
+//   one latitude for one (batch, head); lane i owns longitude w0 + i and keeps its
+//   per-point vectors (q and the y accumulator, or k, v and the dk, dv accumulators)
+//   in registers.  The neighborhood of a whole latitude is a short list of runs
+//   (lat, ws, len): for the 64 lanes together a run touches one contiguous, circular
+//   band of the other grid's longitudes, which the wavefront copies into LDS with
+//   coalesced loads and then slides over: lane i reads row pscale*i + t.  No
+//   cross-lane reduction and no atomics anywhere; dk/dv are produced by a transposed
+//   gather (runs regrouped by input latitude) instead of a scatter.
+//   Workgroups are issued longest latitude first; the linear block index has
+//   (batch, head) fastest so the 8 XCDs each see one head's band of K/V.
+//
+// Numerics: storage dtype in/out (fp32, bf16, fp16), everything else fp32.  Scores
+// are kept in the log2 domain (q is multiplied by log2(e) once) so the softmax uses
+// the hardware exp2.
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdio>
+
+#include "s2attn_internal.h"
+
+// ---------------------------------------------------------------------------------
+// error reporting
+// ---------------------------------------------------------------------------------
+static thread_local char g_err[512] = "";
+
+int s2attn_fail(int code, const char *fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+extern "C" const char *s2attn_last_error(void) { return g_err; }
+extern "C" int s2attn_abi_version(void) { return 1; }
+
+namespace s2 {
+
+constexpr int TQ = 64;          // grid points per wavefront tile (one per lane)
+constexpr int TL = 8;           // neighbors per lane between two LDS refills
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float NEG_BIG = -3.0e38f;
+
+struct Run {
+    int lat, ws, len, pad;
+};
+
+// ---- storage types -----------------------------------------------------------------
+struct bf16_t {
+    unsigned short bits;
+};
+struct f16_t {
+    _Float16 v;
+};
+
+__device__ inline float to_f32(float x) { return x; }
+__device__ inline float to_f32(bf16_t x) { return __uint_as_float(((unsigned)x.bits) << 16); }
+__device__ inline float to_f32(f16_t x) { return (float)x.v; }
+
+__device__ inline void from_f32(float &d, float x) { d = x; }
+__device__ inline void from_f32(bf16_t &d, float x)
+{
+    unsigned u = __float_as_uint(x);
+    if ((u & 0x7fffffffu) > 0x7f800000u) { // NaN
+        d.bits = (unsigned short)((u >> 16) | 0x0040u);
+    } else {
+        u += 0x7fffu + ((u >> 16) & 1u); // round to nearest even
+        d.bits = (unsigned short)(u >> 16);
+    }
+}
+__device__ inline void from_f32(f16_t &d, float x) { d.v = (_Float16)x; }
+
+template <typename T> struct Vec4;
+template <> struct Vec4<float> {
+    typedef float4 type;
+};
+template <> struct Vec4<bf16_t> {
+    typedef uint2 type;
+};
+template <> struct Vec4<f16_t> {
+    typedef uint2 type;
+};
+
+__device__ inline float4 load4(const float *p) { return *reinterpret_cast<const float4 *>(p); }
+__device__ inline float4 load4(const bf16_t *p)
+{
+    const uint2 r = *reinterpret_cast<const uint2 *>(p);
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16),
+                       __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ inline float4 load4(const f16_t *p)
+{
+    union {
+        uint2 u;
+        _Float16 h[4];
+    } r;
+    r.u = *reinterpret_cast<const uint2 *>(p);
+    return make_float4((float)r.h[0], (float)r.h[1], (float)r.h[2], (float)r.h[3]);
+}
+__device__ inline void store4(float *p, float4 v) { *reinterpret_cast<float4 *>(p) = v; }
+__device__ inline void store4(bf16_t *p, float4 v)
+{
+    bf16_t a, b, c, d;
+    from_f32(a, v.x);
+    from_f32(b, v.y);
+    from_f32(c, v.z);
+    from_f32(d, v.w);
+    uint2 r;
+    r.x = (unsigned)a.bits | ((unsigned)b.bits << 16);
+    r.y = (unsigned)c.bits | ((unsigned)d.bits << 16);
+    *reinterpret_cast<uint2 *>(p) = r;
+}
+__device__ inline void store4(f16_t *p, float4 v)
+{
+    union {
+        uint2 u;
+        _Float16 h[4];
+    } r;
+    r.h[0] = (_Float16)v.x;
+    r.h[1] = (_Float16)v.y;
+    r.h[2] = (_Float16)v.z;
+    r.h[3] = (_Float16)v.w;
+    *reinterpret_cast<uint2 *>(p) = r.u;
+}
+
+__device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+__device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
+
+// ---- LDS staging -------------------------------------------------------------------
+// Copies `nrows` grid points (longitudes c0, c0+1, ... wrapping at W) of one latitude and
+// one head into LDS as fp32 rows of P floats (zero padded past d), row stride P+4 floats so
+// that 128-bit reads by consecutive lanes fall in distinct banks.
+//   src : first element of (batch, latitude, longitude 0, head)
+//   ld  : elements between two longitudes (num_heads * d)
+template <typename T, int P, bool VEC>
+__device__ inline void stage_rows(float *dst, const T *src, long ld, int d, int c0, int W, int nrows, int lane)
+{
+    constexpr int LS = P + 4;
+    if (VEC) {
+        constexpr int V4 = P / 4;
+        for (int idx = lane; idx < nrows * V4; idx += TQ) {
+            const int r = idx / V4, c = 4 * (idx % V4);
+            int col = c0 + r;
+            while (col >= W) col -= W;
+            float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (c < d) val = load4(src + (long)col * ld + c);
+            *reinterpret_cast<float4 *>(dst + r * LS + c) = val;
+        }
+    } else {
+        for (int idx = lane; idx < nrows * P; idx += TQ) {
+            const int r = idx / P, c = idx % P;
+            int col = c0 + r;
+            while (col >= W) col -= W;
+            dst[r * LS + c] = (c < d) ? to_f32(src[(long)col * ld + c]) : 0.f;
+        }
+    }
+}
+
+// Writes `nrows` LDS rows back to consecutive longitudes c0.. (no wrap) of one latitude/head.
+template <typename T, int P, bool VEC>
+__device__ inline void unstage_rows(T *dst, const float *src, long ld, int d, int c0, int nrows, int lane)
+{
+    constexpr int LS = P + 4;
+    if (VEC) {
+        constexpr int V4 = P / 4;
+        for (int idx = lane; idx < nrows * V4; idx += TQ) {
+            const int r = idx / V4, c = 4 * (idx % V4);
+            if (c < d) store4(dst + (long)(c0 + r) * ld + c, *reinterpret_cast<const float4 *>(src + r * LS + c));
+        }
+    } else {
+        for (int idx = lane; idx < nrows * P; idx += TQ) {
+            const int r = idx / P, c = idx % P;
+            if (c < d) from_f32(dst[(long)(c0 + r) * ld + c], src[r * LS + c]);
+        }
+    }
+}
+
+template <int P> __device__ inline float dot_row(const float (&a)[P], const float *row)
+{
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
+#pragma unroll
+    for (int c = 0; c < P; c += 4) {
+        const float4 x = *reinterpret_cast<const float4 *>(row + c);
+        s0 = fmaf(a[c + 0], x.x, s0);
+        s1 = fmaf(a[c + 1], x.y, s1);
+        s2 = fmaf(a[c + 2], x.z, s2);
+        s3 = fmaf(a[c + 3], x.w, s3);
+    }
+    return (s0 + s1) + (s2 + s3);
+}
+
+struct Args {
+    const void *k, *v, *q, *dy;
+    void *y, *dk, *dv, *dq;
+    float2 *stats; // per (batch, head, ho, wo): (log2-sum-exp of the scaled scores, sum_j p_j <dy, v_j>)
+    const float *quad_w;
+    const int *goff, *gorder, *soff, *sorder;
+    const Run *gruns, *sruns;
+    int B, nh, Hi, Wi, Ho, Wo, dk_, dv_, pscale;
+    int tile_rows; // LDS rows per staged band
+};
+
+// ---------------------------------------------------------------------------------
+// forward:  y = sum_j a_j v_j / sum_j a_j
+// ---------------------------------------------------------------------------------
+template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd_kernel(const Args a)
+{
+    extern __shared__ float4 smem4[];
+    float *Ks = reinterpret_cast<float *>(smem4);
+    constexpr int LS = P + 4;
+    float *Vs = Ks + a.tile_rows * LS;
+
+    const int lane = threadIdx.x;
+    const int BH = a.B * a.nh;
+    const int ntile = (a.Wo + TQ - 1) / TQ;
+    int id = blockIdx.x;
+    const int bh = id % BH;
+    id /= BH;
+    const int wt = id % ntile;
+    const int ho = a.gorder[id / ntile];
+    const int b = bh / a.nh, h = bh % a.nh;
+    const int wo0 = wt * TQ;
+    const int nvalid = min(TQ, a.Wo - wo0);
+    const int ps = a.pscale;
+    const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
+
+    const T *kx = static_cast<const T *>(a.k);
+    const T *vx = static_cast<const T *>(a.v);
+    const T *qy = static_cast<const T *>(a.q);
+    T *y = static_cast<T *>(a.y);
+
+    // q for this lane, pre-multiplied by log2(e)
+    stage_rows<T, P, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, wo0, a.Wo, nvalid, lane);
+    __syncthreads();
+    float qr[P], acc[P];
+#pragma unroll
+    for (int c = 0; c < P; c++) {
+        qr[c] = Ks[lane * LS + c] * LOG2E;
+        acc[c] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f;
+
+    for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
+        const Run run = a.gruns[ri];
+        const float w = a.quad_w[run.lat];
+        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
+        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        for (int t0 = 0; t0 < run.len; t0 += TL) {
+            const int L = min(TL, run.len - t0);
+            const int c0 = (run.ws + t0 + ps * wo0) % a.Wi;
+            const int nrows = ps * (nvalid - 1) + L;
+            __syncthreads();
+            stage_rows<T, P, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, P, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            __syncthreads();
+
+            const float *krow = Ks + (ps * lane) * LS;
+            const float *vrow = Vs + (ps * lane) * LS;
+            float s[TL];
+            float cm = NEG_BIG;
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                s[t] = NEG_BIG;
+                if (t < L) {
+                    s[t] = dot_row<P>(qr, krow + t * LS);
+                    cm = fmaxf(cm, s[t]);
+                }
+            }
+            const float mn = fmaxf(m, cm);
+            const float corr = fast_exp2(m - mn);
+            m = mn;
+            S *= corr;
+#pragma unroll
+            for (int c = 0; c < P; c++) acc[c] *= corr;
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                if (t < L) {
+                    const float p = fast_exp2(s[t] - mn) * w;
+                    S += p;
+                    const float *vr = vrow + t * LS;
+#pragma unroll
+                    for (int c = 0; c < P; c += 4) {
+                        const float4 x = *reinterpret_cast<const float4 *>(vr + c);
+                        acc[c + 0] = fmaf(p, x.x, acc[c + 0]);
+                        acc[c + 1] = fmaf(p, x.y, acc[c + 1]);
+                        acc[c + 2] = fmaf(p, x.z, acc[c + 2]);
+                        acc[c + 3] = fmaf(p, x.w, acc[c + 3]);
+                    }
+                }
+            }
+        }
+    }
+
+    const float inv = 1.0f / S;
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < P; c += 4)
+        *reinterpret_cast<float4 *>(Ks + lane * LS + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
+    __syncthreads();
+    unstage_rows<T, P, VEC>(y + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, Ks, ldv, a.dv_, wo0, nvalid, lane);
+}
+
+// ---------------------------------------------------------------------------------
+// backward, query side:  dq = sum_j p_j (g_j - I) k_j   with g_j = <dy, v_j>, I = sum_j p_j g_j
+// accumulated online as (A_kg - I A_k) / S, A_k = sum a_j k_j, A_kg = sum a_j g_j k_j; also
+// emits (log2 sum a_j + max, I) per query for the dk/dv kernel.
+// ---------------------------------------------------------------------------------
+template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dq_kernel(const Args a)
+{
+    extern __shared__ float4 smem4[];
+    float *Ks = reinterpret_cast<float *>(smem4);
+    constexpr int LS = P + 4;
+    float *Vs = Ks + a.tile_rows * LS;
+
+    const int lane = threadIdx.x;
+    const int BH = a.B * a.nh;
+    const int ntile = (a.Wo + TQ - 1) / TQ;
+    int id = blockIdx.x;
+    const int bh = id % BH;
+    id /= BH;
+    const int wt = id % ntile;
+    const int ho = a.gorder[id / ntile];
+    const int b = bh / a.nh, h = bh % a.nh;
+    const int wo0 = wt * TQ;
+    const int nvalid = min(TQ, a.Wo - wo0);
+    const int ps = a.pscale;
+    const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
+
+    const T *kx = static_cast<const T *>(a.k);
+    const T *vx = static_cast<const T *>(a.v);
+    const T *qy = static_cast<const T *>(a.q);
+    const T *gy = static_cast<const T *>(a.dy);
+    T *dq = static_cast<T *>(a.dq);
+
+    stage_rows<T, P, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, wo0, a.Wo, nvalid, lane);
+    stage_rows<T, P, VEC>(Vs, gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, ldv, a.dv_, wo0, a.Wo, nvalid, lane);
+    __syncthreads();
+    float qr[P], gr[P], Ak[P], Akg[P];
+#pragma unroll
+    for (int c = 0; c < P; c++) {
+        qr[c] = Ks[lane * LS + c] * LOG2E;
+        gr[c] = Vs[lane * LS + c];
+        Ak[c] = 0.f;
+        Akg[c] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f, Ag = 0.f;
+
+    for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
+        const Run run = a.gruns[ri];
+        const float w = a.quad_w[run.lat];
+        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
+        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        for (int t0 = 0; t0 < run.len; t0 += TL) {
+            const int L = min(TL, run.len - t0);
+            const int c0 = (run.ws + t0 + ps * wo0) % a.Wi;
+            const int nrows = ps * (nvalid - 1) + L;
+            __syncthreads();
+            stage_rows<T, P, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, P, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            __syncthreads();
+
+            const float *krow = Ks + (ps * lane) * LS;
+            const float *vrow = Vs + (ps * lane) * LS;
+            float s[TL], g[TL];
+            float cm = NEG_BIG;
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                s[t] = NEG_BIG;
+                g[t] = 0.f;
+                if (t < L) {
+                    s[t] = dot_row<P>(qr, krow + t * LS);
+                    g[t] = dot_row<P>(gr, vrow + t * LS);
+                    cm = fmaxf(cm, s[t]);
+                }
+            }
+            const float mn = fmaxf(m, cm);
+            const float corr = fast_exp2(m - mn);
+            m = mn;
+            S *= corr;
+            Ag *= corr;
+#pragma unroll
+            for (int c = 0; c < P; c++) {
+                Ak[c] *= corr;
+                Akg[c] *= corr;
+            }
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                if (t < L) {
+                    const float p = fast_exp2(s[t] - mn) * w;
+                    const float pg = p * g[t];
+                    S += p;
+                    Ag += pg;
+                    const float *kr = krow + t * LS;
+#pragma unroll
+                    for (int c = 0; c < P; c += 4) {
+                        const float4 x = *reinterpret_cast<const float4 *>(kr + c);
+                        Ak[c + 0] = fmaf(p, x.x, Ak[c + 0]);
+                        Ak[c + 1] = fmaf(p, x.y, Ak[c + 1]);
+                        Ak[c + 2] = fmaf(p, x.z, Ak[c + 2]);
+                        Ak[c + 3] = fmaf(p, x.w, Ak[c + 3]);
+                        Akg[c + 0] = fmaf(pg, x.x, Akg[c + 0]);
+                        Akg[c + 1] = fmaf(pg, x.y, Akg[c + 1]);
+                        Akg[c + 2] = fmaf(pg, x.z, Akg[c + 2]);
+                        Akg[c + 3] = fmaf(pg, x.w, Akg[c + 3]);
+                    }
+                }
+            }
+        }
+    }
+
+    const float inv = 1.0f / S;
+    const float I = Ag * inv;
+    if (lane < nvalid) a.stats[((long)bh * a.Ho + ho) * a.Wo + wo0 + lane] = make_float2(m + fast_log2(S), I);
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < P; c += 4)
+        *reinterpret_cast<float4 *>(Ks + lane * LS + c)
+            = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
+                          (Akg[c + 3] - I * Ak[c + 3]) * inv);
+    __syncthreads();
+    unstage_rows<T, P, VEC>(dq + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, Ks, ldk, a.dk_, wo0, nvalid, lane);
+}
+
+// ---------------------------------------------------------------------------------
+// backward, key/value side (transposed gather).  Lane = input point (hi, wi).  For a run
+// (ho, ws, len) the queries that see this point are wo = (floor(delta/ps) - u) mod Wo with
+// delta = (wi - ws) mod Wi and neighbor index t = delta mod ps + ps*u < len:
+//   dv += p dy,  dk += p (g - I) q,   p = exp2(log2e q.k - lse2) * quad_w[hi]
+// ---------------------------------------------------------------------------------
+template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkdv_kernel(const Args a)
+{
+    extern __shared__ float4 smem4[];
+    float *Qs = reinterpret_cast<float *>(smem4);
+    constexpr int LS = P + 4;
+    float *Gs = Qs + a.tile_rows * LS;
+    float2 *Ss = reinterpret_cast<float2 *>(Gs + a.tile_rows * LS);
+
+    const int lane = threadIdx.x;
+    const int BH = a.B * a.nh;
+    const int ntile = (a.Wi + TQ - 1) / TQ;
+    int id = blockIdx.x;
+    const int bh = id % BH;
+    id /= BH;
+    const int ct = id % ntile;
+    const int hi = a.sorder[id / ntile];
+    const int b = bh / a.nh, h = bh % a.nh;
+    const int wi0 = ct * TQ;
+    const int nvalid = min(TQ, a.Wi - wi0);
+    const int ps = a.pscale;
+    const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
+
+    const T *kx = static_cast<const T *>(a.k);
+    const T *vx = static_cast<const T *>(a.v);
+    const T *qy = static_cast<const T *>(a.q);
+    const T *gy = static_cast<const T *>(a.dy);
+    T *dk = static_cast<T *>(a.dk);
+    T *dv = static_cast<T *>(a.dv);
+
+    stage_rows<T, P, VEC>(Qs, kx + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, ldk, a.dk_, wi0, a.Wi, nvalid, lane);
+    stage_rows<T, P, VEC>(Gs, vx + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, ldv, a.dv_, wi0, a.Wi, nvalid, lane);
+    __syncthreads();
+    float kr[P], vr[P], dkr[P], dvr[P];
+#pragma unroll
+    for (int c = 0; c < P; c++) {
+        kr[c] = Qs[lane * LS + c] * LOG2E;
+        vr[c] = Gs[lane * LS + c];
+        dkr[c] = 0.f;
+        dvr[c] = 0.f;
+    }
+    const float w = a.quad_w[hi];
+
+    for (int ri = a.soff[hi]; ri < a.soff[hi + 1]; ri++) {
+        const Run run = a.sruns[ri];
+        const int ho = run.lat;
+        int d0 = wi0 - run.ws;
+        if (d0 < 0) d0 += a.Wi;
+        // lane geometry relative to the first lane (no wrap: d0 + lane may exceed Wi)
+        int al, r0;
+        if (ps == 1) {
+            al = lane;
+            r0 = 0;
+        } else {
+            al = (d0 + lane) / ps - d0 / ps;
+            r0 = (d0 + lane) % ps;
+        }
+        const int a0 = d0 / ps;
+        const int span = (d0 + nvalid - 1) / ps - a0; // al of the last valid lane
+        const int U = (run.len + ps - 1) / ps;
+        const T *ql = qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_;
+        const T *gl = gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_;
+        const float2 *sl = a.stats + ((long)bh * a.Ho + ho) * a.Wo;
+
+        for (int u0 = 0; u0 < U; u0 += TL) {
+            const int UL = min(TL, U - u0);
+            int c0 = (a0 - u0 - UL + 1) % a.Wo;
+            if (c0 < 0) c0 += a.Wo;
+            const int nrows = span + UL;
+            __syncthreads();
+            stage_rows<T, P, VEC>(Qs, ql, ldk, a.dk_, c0, a.Wo, nrows, lane);
+            stage_rows<T, P, VEC>(Gs, gl, ldv, a.dv_, c0, a.Wo, nrows, lane);
+            for (int r = lane; r < nrows; r += TQ) {
+                int col = c0 + r;
+                while (col >= a.Wo) col -= a.Wo;
+                Ss[r] = sl[col];
+            }
+            __syncthreads();
+
+#pragma unroll
+            for (int j = 0; j < TL; j++) {
+                if (j < UL) {
+                    const int row = al + (UL - 1 - j);
+                    const int t = r0 + ps * (u0 + j);
+                    const float *qrow = Qs + row * LS;
+                    const float *grow = Gs + row * LS;
+                    float qq[P], gg[P];
+#pragma unroll
+                    for (int c = 0; c < P; c += 4) {
+                        const float4 x = *reinterpret_cast<const float4 *>(qrow + c);
+                        const float4 z = *reinterpret_cast<const float4 *>(grow + c);
+                        qq[c] = x.x, qq[c + 1] = x.y, qq[c + 2] = x.z, qq[c + 3] = x.w;
+                        gg[c] = z.x, gg[c + 1] = z.y, gg[c + 2] = z.z, gg[c + 3] = z.w;
+                    }
+                    float s0 = 0.f, s1 = 0.f, g0 = 0.f, g1 = 0.f;
+#pragma unroll
+                    for (int c = 0; c < P; c += 2) {
+                        s0 = fmaf(qq[c], kr[c], s0);
+                        s1 = fmaf(qq[c + 1], kr[c + 1], s1);
+                        g0 = fmaf(gg[c], vr[c], g0);
+                        g1 = fmaf(gg[c + 1], vr[c + 1], g1);
+                    }
+                    const float2 st = Ss[row];
+                    float p = fast_exp2((s0 + s1) - st.x) * w;
+                    if (t >= run.len) p = 0.f;
+                    const float coef = p * ((g0 + g1) - st.y);
+#pragma unroll
+                    for (int c = 0; c < P; c++) {
+                        dkr[c] = fmaf(coef, qq[c], dkr[c]);
+                        dvr[c] = fmaf(p, gg[c], dvr[c]);
+                    }
+                }
+            }
+        }
+    }
+
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < P; c += 4) {
+        *reinterpret_cast<float4 *>(Qs + lane * LS + c) = make_float4(dkr[c], dkr[c + 1], dkr[c + 2], dkr[c + 3]);
+        *reinterpret_cast<float4 *>(Gs + lane * LS + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
+    }
+    __syncthreads();
+    unstage_rows<T, P, VEC>(dk + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, Qs, ldk, a.dk_, wi0, nvalid, lane);
+    unstage_rows<T, P, VEC>(dv + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, Gs, ldv, a.dv_, wi0, nvalid, lane);
+}
+
+// ---------------------------------------------------------------------------------
+// layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
+// ---------------------------------------------------------------------------------
+template <typename E> __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ src, E *__restrict__ dst, long R, long S)
+{
+    __shared__ E tile[64][65];
+    const long bofs = (long)blockIdx.z * R * S;
+    const long s0 = (long)blockIdx.x * 64, r0 = (long)blockIdx.y * 64;
+    const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+    for (int i = ty; i < 64; i += 4) {
+        const long r = r0 + i, s = s0 + tx;
+        if (r < R && s < S) tile[i][tx] = src[bofs + r * S + s];
+    }
+    __syncthreads();
+    for (int i = ty; i < 64; i += 4) {
+        const long s = s0 + i, r = r0 + tx;
+        if (r < R && s < S) dst[bofs + s * R + r] = tile[tx][i];
+    }
+}
+
+} // namespace s2
+
+// ---------------------------------------------------------------------------------
+// host side
+// ---------------------------------------------------------------------------------
+namespace {
+
+using namespace s2;
+
+int check_shape(const s2attn_shape *sh)
+{
+    if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "shape is null");
+    if (sh->batch < 1 || sh->nlat_in < 1 || sh->nlon_in < 1 || sh->nlat_out < 1 || sh->nlon_out < 1)
+        return s2attn_fail(S2ATTN_E_INVALID, "batch and grid extents must be positive");
+    if (sh->num_heads < 1) return s2attn_fail(S2ATTN_E_INVALID, "num_heads must be positive, got %d", sh->num_heads);
+    if (sh->ck < 1 || sh->cv < 1) return s2attn_fail(S2ATTN_E_INVALID, "per-head channel counts must be positive");
+    if (sh->nlon_in % sh->nlon_out != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d)", sh->nlon_in, sh->nlon_out);
+    if (sh->dtype != S2ATTN_F32 && sh->dtype != S2ATTN_BF16 && sh->dtype != S2ATTN_F16)
+        return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
+    if (sh->ck > 32 || sh->cv > 32)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 32 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
+    return S2ATTN_OK;
+}
+
+int esize(int dtype) { return dtype == S2ATTN_F32 ? 4 : 2; }
+
+bool aligned(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
+
+enum Which { FWD, DQ, DKDV };
+
+template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a, hipStream_t stream)
+{
+    const int BH = a.B * a.nh;
+    constexpr int LS = P + 4;
+    void (*kern)(const Args) = nullptr;
+    long nblocks = 0;
+    size_t lds = 0;
+    if (which == FWD) {
+        kern = fwd_kernel<T, P, VEC>;
+        nblocks = (long)a.Ho * ((a.Wo + TQ - 1) / TQ) * BH;
+        lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
+    } else if (which == DQ) {
+        kern = dq_kernel<T, P, VEC>;
+        nblocks = (long)a.Ho * ((a.Wo + TQ - 1) / TQ) * BH;
+        lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
+    } else {
+        kern = dkdv_kernel<T, P, VEC>;
+        nblocks = (long)a.Hi * ((a.Wi + TQ - 1) / TQ) * BH;
+        lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
+    }
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "longitude ratio %d needs %zu bytes of LDS per workgroup", a.pscale, lds);
+    if (lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(TQ), lds, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+
+template <typename T, bool VEC> int launch_p(Which which, const Args &a, hipStream_t stream)
+{
+    const int d = a.dk_ > a.dv_ ? a.dk_ : a.dv_;
+    if (d <= 4) return launch_one<T, 4, VEC>(which, a, stream);
+    if (d <= 8) return launch_one<T, 8, VEC>(which, a, stream);
+    if (d <= 16) return launch_one<T, 16, VEC>(which, a, stream);
+    return launch_one<T, 32, VEC>(which, a, stream);
+}
+
+template <typename T> int launch_t(Which which, const Args &a, bool vec, hipStream_t stream)
+{
+    return vec ? launch_p<T, true>(which, a, stream) : launch_p<T, false>(which, a, stream);
+}
+
+int launch(Which which, const Args &a, int dtype, bool vec, hipStream_t stream)
+{
+    if (dtype == S2ATTN_F32) return launch_t<float>(which, a, vec, stream);
+    if (dtype == S2ATTN_BF16) return launch_t<bf16_t>(which, a, vec, stream);
+    return launch_t<f16_t>(which, a, vec, stream);
+}
+
+void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const float *quad_w)
+{
+    a.quad_w = quad_w;
+    a.goff = plan->gather_off;
+    a.gruns = reinterpret_cast<const Run *>(plan->gather_runs);
+    a.gorder = plan->gather_order;
+    a.soff = plan->scatter_off;
+    a.sruns = reinterpret_cast<const Run *>(plan->scatter_runs);
+    a.sorder = plan->scatter_order;
+    a.B = sh->batch;
+    a.nh = sh->num_heads;
+    a.Hi = sh->nlat_in;
+    a.Wi = sh->nlon_in;
+    a.Ho = sh->nlat_out;
+    a.Wo = sh->nlon_out;
+    a.dk_ = sh->ck;
+    a.dv_ = sh->cv;
+    a.pscale = sh->nlon_in / sh->nlon_out;
+}
+
+} // namespace
+
+extern "C" int s2attn_forward(const void *k, const void *v, const void *q, const float *quad_weights, void *y,
+                              const s2attn_plan *plan, const s2attn_shape *shape, void *stream)
+{
+    int rc = check_shape(shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!k || !v || !q || !y || !quad_weights) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!plan || !plan->gather_off || !plan->gather_order || (plan->nruns > 0 && !plan->gather_runs))
+        return s2attn_fail(S2ATTN_E_INVALID, "plan is missing its gather arrays");
+    Args a = {};
+    fill_args(a, plan, shape, quad_weights);
+    a.k = k, a.v = v, a.q = q, a.y = y;
+    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    const size_t al = 4 * (size_t)esize(shape->dtype);
+    const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(y, al);
+    return launch(FWD, a, shape->dtype, vec, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape)
+{
+    const int rc = check_shape(shape);
+    if (rc != S2ATTN_OK) return rc;
+    return (int64_t)shape->batch * shape->num_heads * shape->nlat_out * shape->nlon_out * (int64_t)sizeof(float2);
+}
+
+extern "C" int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
+                               void *dk, void *dv, void *dq, void *workspace, const s2attn_plan *plan,
+                               const s2attn_shape *shape, void *stream)
+{
+    int rc = check_shape(shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!k || !v || !q || !dy || !dk || !dv || !dq || !quad_weights || !workspace) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!plan || !plan->gather_off || !plan->gather_order || !plan->scatter_off || !plan->scatter_order
+        || (plan->nruns > 0 && (!plan->gather_runs || !plan->scatter_runs)))
+        return s2attn_fail(S2ATTN_E_INVALID, "plan is missing arrays");
+    if (!aligned(workspace, sizeof(float2))) return s2attn_fail(S2ATTN_E_INVALID, "workspace must be 8-byte aligned");
+    Args a = {};
+    fill_args(a, plan, shape, quad_weights);
+    a.k = k, a.v = v, a.q = q, a.dy = dy, a.dk = dk, a.dv = dv, a.dq = dq;
+    a.stats = static_cast<float2 *>(workspace);
+    const size_t al = 4 * (size_t)esize(shape->dtype);
+    const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(dy, al)
+                     && aligned(dk, al) && aligned(dv, al) && aligned(dq, al);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    rc = launch(DQ, a, shape->dtype, vec, st);
+    if (rc != S2ATTN_OK) return rc;
+    a.tile_rows = (TQ - 1) / a.pscale + 1 + TL;
+    if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile is also used to stage the lane-owned k/v and dk/dv rows
+    return launch(DKDV, a, shape->dtype, vec, st);
+}
+
+namespace {
+template <typename E> int launch_transpose(const void *src, void *dst, long nb, long R, long S, hipStream_t stream)
+{
+    if (nb == 0 || R == 0 || S == 0) return S2ATTN_OK;
+    const long gx = (S + 63) / 64, gy = (R + 63) / 64;
+    if (gx > 0x7fffffffL || gy > 65535 || nb > 65535) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "permute grid (%ld, %ld, %ld) exceeds launch limits", gx, gy, nb);
+    hipLaunchKernelGGL(s2::transpose_kernel<E>, dim3((unsigned)gx, (unsigned)gy, (unsigned)nb), dim3(256), 0, stream, static_cast<const E *>(src),
+                       static_cast<E *>(dst), R, S);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+
+int permute(const void *src, void *dst, long nb, long R, long S, int elem_size, void *stream)
+{
+    if (nb < 0 || R < 0 || S < 0) return s2attn_fail(S2ATTN_E_INVALID, "negative extent");
+    if ((!src || !dst) && nb * R * S > 0) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    switch (elem_size) {
+    case 2: return launch_transpose<unsigned short>(src, dst, nb, R, S, st);
+    case 4: return launch_transpose<unsigned int>(src, dst, nb, R, S, st);
+    case 8: return launch_transpose<unsigned long long>(src, dst, nb, R, S, st);
+    default: return s2attn_fail(S2ATTN_E_INVALID, "element size %d is not 2, 4 or 8 bytes", elem_size);
+    }
+}
+} // namespace
+
+extern "C" int s2attn_permute_to_nhwc(const void *src, void *dst, int64_t B, int64_t C, int64_t H, int64_t W, int elem_size, void *stream)
+{
+    return permute(src, dst, B, C, H * W, elem_size, stream); // [C, HW] -> [HW, C]
+}
+
+extern "C" int s2attn_permute_to_nchw(const void *src, void *dst, int64_t B, int64_t H, int64_t W, int64_t C, int elem_size, void *stream)
+{
+    return permute(src, dst, B, H * W, C, elem_size, stream); // [HW, C] -> [C, HW]
+}

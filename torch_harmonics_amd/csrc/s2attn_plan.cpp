@@ -1,0 +1,140 @@
+// Host-side conversion of the CSR neighborhood into longitude runs (see include/s2attn.h).
+//
+// The reference keeps the neighborhood as one int64 column index per neighbor and
+// only reorders rows by length (attention_cuda_utils.cu:74-113).  On the sphere
+// every row is a stack of longitude intervals, one per input latitude, so a row of
+// thousands of neighbors collapses to a handful of (lat, start, len) runs.  Runs
+// are what lets a wavefront stage one contiguous band of K/V per latitude in LDS
+// and slide all of its queries over it.
+
+#include "s2attn_internal.h"
+
+#include <algorithm>
+#include <cstdio>
+#include <numeric>
+#include <vector>
+
+namespace {
+
+struct HostRun {
+    int32_t ho, hi, ws, len;
+};
+
+// Splits the CSR into maximal runs of consecutive longitudes inside one input
+// latitude, then joins a run that ends at nlon_in-1 with a run of the same
+// latitude that starts at 0 into a single circular run.
+int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in, int nlat_out,
+              int nlon_out, std::vector<HostRun> *out, int64_t *count)
+{
+    if (!col_idx && nnz > 0) return s2attn_fail(S2ATTN_E_INVALID, "col_idx is null");
+    if (!row_off) return s2attn_fail(S2ATTN_E_INVALID, "row_off is null");
+    if (nlat_in < 1 || nlon_in < 1 || nlat_out < 1 || nlon_out < 1)
+        return s2attn_fail(S2ATTN_E_INVALID, "grid extents must be positive");
+    if (nlon_in % nlon_out != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d)", nlon_in, nlon_out);
+    if (row_off[0] != 0 || row_off[nlat_out] != nnz)
+        return s2attn_fail(S2ATTN_E_INVALID, "row_off must start at 0 and end at nnz (%lld), got %lld..%lld", (long long)nnz,
+                           (long long)row_off[0], (long long)row_off[nlat_out]);
+
+    const int64_t ncol = (int64_t)nlat_in * nlon_in;
+    int64_t total = 0;
+    std::vector<HostRun> row;
+    for (int ho = 0; ho < nlat_out; ho++) {
+        const int64_t z0 = row_off[ho], z1 = row_off[ho + 1];
+        if (z1 < z0) return s2attn_fail(S2ATTN_E_INVALID, "row_off decreases at row %d", ho);
+        row.clear();
+        for (int64_t z = z0; z < z1; z++) {
+            const int64_t col = col_idx[z];
+            if (col < 0 || col >= ncol)
+                return s2attn_fail(S2ATTN_E_INVALID, "col_idx[%lld] = %lld outside [0, %lld)", (long long)z, (long long)col,
+                                   (long long)ncol);
+            const int32_t hi = (int32_t)(col / nlon_in), wi = (int32_t)(col % nlon_in);
+            if (!row.empty() && row.back().hi == hi && row.back().ws + row.back().len == wi && row.back().len < nlon_in) {
+                row.back().len++;
+            } else {
+                row.push_back({ho, hi, wi, 1});
+            }
+        }
+        // circular join inside each group of runs that share a latitude
+        size_t i = 0;
+        while (i < row.size()) {
+            size_t j = i;
+            while (j + 1 < row.size() && row[j + 1].hi == row[i].hi) j++;
+            if (j > i && row[i].ws == 0 && row[j].ws + row[j].len == nlon_in && row[i].len + row[j].len <= nlon_in) {
+                row[j].len += row[i].len;
+                row[i].len = 0; // dropped
+            }
+            i = j + 1;
+        }
+        for (const HostRun &r : row) {
+            if (r.len == 0) continue;
+            total++;
+            if (out) out->push_back(r);
+        }
+    }
+    *count = total;
+    return S2ATTN_OK;
+}
+
+} // namespace
+
+extern "C" int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                                     int nlat_out, int nlon_out)
+{
+    int64_t n = 0;
+    const int rc = decompose(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, nullptr, &n);
+    return rc == S2ATTN_OK ? n : (int64_t)rc;
+}
+
+extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                                 int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
+                                 int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order)
+{
+    if (!gather_off || !gather_order || !scatter_off || !scatter_order || (nruns > 0 && (!gather_runs || !scatter_runs)))
+        return s2attn_fail(S2ATTN_E_INVALID, "plan output array is null");
+
+    std::vector<HostRun> runs;
+    int64_t n = 0;
+    const int rc = decompose(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, &runs, &n);
+    if (rc != S2ATTN_OK) return rc;
+    if (n != nruns) return s2attn_fail(S2ATTN_E_INVALID, "nruns = %lld does not match the CSR (%lld runs)", (long long)nruns, (long long)n);
+
+    const int pscale = nlon_in / nlon_out;
+
+    // gather side: runs are already grouped by ho, in CSR order
+    std::vector<int64_t> gwork(nlat_out, 0);
+    std::fill(gather_off, gather_off + nlat_out + 1, 0);
+    for (int64_t i = 0; i < n; i++) {
+        const HostRun &r = runs[i];
+        gather_runs[4 * i + 0] = r.hi;
+        gather_runs[4 * i + 1] = r.ws;
+        gather_runs[4 * i + 2] = r.len;
+        gather_runs[4 * i + 3] = 0;
+        gather_off[r.ho + 1]++;
+        gwork[r.ho] += r.len;
+    }
+    for (int ho = 0; ho < nlat_out; ho++) gather_off[ho + 1] += gather_off[ho];
+
+    // scatter side: stable counting sort by hi keeps ho ascending inside a group
+    std::vector<int64_t> swork(nlat_in, 0);
+    std::fill(scatter_off, scatter_off + nlat_in + 1, 0);
+    for (int64_t i = 0; i < n; i++) scatter_off[runs[i].hi + 1]++;
+    for (int hi = 0; hi < nlat_in; hi++) scatter_off[hi + 1] += scatter_off[hi];
+    std::vector<int32_t> cursor(scatter_off, scatter_off + nlat_in);
+    for (int64_t i = 0; i < n; i++) {
+        const HostRun &r = runs[i];
+        const int32_t s = cursor[r.hi]++;
+        scatter_runs[4 * s + 0] = r.ho;
+        scatter_runs[4 * s + 1] = r.ws;
+        scatter_runs[4 * s + 2] = r.len;
+        scatter_runs[4 * s + 3] = 0;
+        swork[r.hi] += (r.len + pscale - 1) / pscale;
+    }
+
+    // longest group first (stable, so equal groups keep latitude order)
+    std::iota(gather_order, gather_order + nlat_out, 0);
+    std::stable_sort(gather_order, gather_order + nlat_out, [&](int32_t a, int32_t b) { return gwork[a] > gwork[b]; });
+    std::iota(scatter_order, scatter_order + nlat_in, 0);
+    std::stable_sort(scatter_order, scatter_order + nlat_in, [&](int32_t a, int32_t b) { return swork[a] > swork[b]; });
+    return S2ATTN_OK;
+}

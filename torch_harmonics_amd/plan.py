@@ -1,0 +1,102 @@
+"""
+Neighborhood plans: the run-length form of psi that the kernels consume, built once per
+(col_idx, row_off) pair by the C++ builder in libs2attn.so and cached.
+
+The reference re-sorts the CSR rows by length on the device on every call
+(attention_cuda_utils.cu:74-113).  Here the conversion happens on the host the first time
+a psi is seen (one device-to-host copy of the two index tensors) and later calls reuse the
+device-resident plan.  A cache entry keeps its col_idx/row_off tensors alive, so their
+addresses cannot be recycled for a different psi while the entry exists, and an in-place
+edit of either tensor changes its version counter and misses the cache.
+"""
+
+import threading
+from collections import OrderedDict
+
+import torch
+
+from . import _lib
+
+_MAX_ENTRIES = 32
+_cache = OrderedDict()
+_lock = threading.Lock()
+
+
+class Plan:
+    """Six int32 arrays on one device plus the ctypes view the library takes."""
+
+    def __init__(self, arrays, nruns, keepalive):
+        self.gather_off, self.gather_runs, self.gather_order, self.scatter_off, self.scatter_runs, self.scatter_order = arrays
+        self.nruns = nruns
+        self._keepalive = keepalive
+        self.struct = _lib.PlanStruct(
+            self.gather_off.data_ptr(),
+            self.gather_runs.data_ptr(),
+            self.gather_order.data_ptr(),
+            self.scatter_off.data_ptr(),
+            self.scatter_runs.data_ptr(),
+            self.scatter_order.data_ptr(),
+            nruns,
+        )
+
+
+def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int):
+    """
+    Runs the library's host builder on CPU copies of the CSR.  Returns
+    ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns)
+    as CPU int32 tensors; gather_runs / scatter_runs have shape (nruns, 4) = (lat, ws, len, 0).
+    """
+    lib = _lib.load()
+    ci = col_idx.detach().to(device="cpu", dtype=torch.int64).contiguous()
+    ro = row_off.detach().to(device="cpu", dtype=torch.int64).contiguous()
+    if ro.numel() != nlat_out + 1:
+        raise RuntimeError(f"row_off must have nlat_out + 1 = {nlat_out + 1} entries, got {ro.numel()}")
+    nnz = ci.numel()
+    nruns = lib.s2attn_plan_count(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out)
+    _lib.check(nruns, "s2attn_plan_count")
+    arrays = [
+        torch.zeros(nlat_out + 1, dtype=torch.int32),
+        torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
+        torch.zeros(nlat_out, dtype=torch.int32),
+        torch.zeros(nlat_in + 1, dtype=torch.int32),
+        torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
+        torch.zeros(nlat_in, dtype=torch.int32),
+    ]
+    rc = lib.s2attn_plan_build(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays])
+    _lib.check(rc, "s2attn_plan_build")
+    return arrays, int(nruns)
+
+
+def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int) -> Plan:
+    """Device plan for this psi, from the cache when the same tensors were seen before."""
+    key = (
+        col_idx.data_ptr(),
+        row_off.data_ptr(),
+        col_idx.numel(),
+        row_off.numel(),
+        col_idx._version,
+        row_off._version,
+        str(col_idx.device),
+        nlat_in,
+        nlon_in,
+        nlat_out,
+        nlon_out,
+    )
+    with _lock:
+        plan = _cache.get(key)
+        if plan is not None:
+            _cache.move_to_end(key)
+            return plan
+    arrays, nruns = build_host_plan(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    dev = col_idx.device
+    plan = Plan([a.to(dev) for a in arrays], nruns, (col_idx, row_off))
+    with _lock:
+        _cache[key] = plan
+        while len(_cache) > _MAX_ENTRIES:
+            _cache.popitem(last=False)
+    return plan
+
+
+def clear_plan_cache() -> None:
+    with _lock:
+        _cache.clear()
