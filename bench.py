@@ -1,0 +1,288 @@
+#!/usr/bin/env python
+"""
+Benchmark of the spherical neighborhood-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--config cfg3] [--no-cpu-baseline]
+
+One step = one forward plus one backward of the attention op (the C ABI behind
+torch_harmonics_amd.ops) on the ERA5-shaped configuration: equiangular 721x1440 grid in and
+out, batch 1, 256 channels in 8 heads, fp32, theta_cutoff = 3 latitude spacings.  Inputs are
+synthetic (low-degree spherical-harmonic fields plus noise, projected by randomly initialised
+q/k/v weights) and resident in HBM before the timed region.  Prints ONE JSON line.
+
+Reported alongside the throughput:
+  roofline      the slowest kernel of the step, timed with events recorded on the launch stream
+                around every launch of it inside the timed region
+  cpu_baseline  the CPU port of the reference algorithm (oracle/, reference release flags, OpenMP)
+                on a bounded sample of the same workload, on this machine's host cores
+"""
+
+import argparse
+import ctypes
+import json
+import math
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+FP32_VALU_PEAK_TFLOPS = 78.6  # 157.3 TFLOP/s vector fp32 is quoted with packed FMA; these kernels are built without packed fp32
+
+CONFIGS = {
+    "cfg1": dict(in_shape=(32, 64), out_shape=(32, 64), grid_in="equiangular", grid_out="equiangular", B=1, C=16, nh=1, theta_cutoff=None),
+    "cfg2": dict(in_shape=(128, 256), out_shape=(128, 256), grid_in="equiangular", grid_out="equiangular", B=4, C=64, nh=4, theta_cutoff=4 * math.pi / 127),
+    "cfg3": dict(in_shape=(721, 1440), out_shape=(721, 1440), grid_in="equiangular", grid_out="equiangular", B=1, C=256, nh=8, theta_cutoff=3 * math.pi / 720),
+    "cfg4": dict(in_shape=(721, 1440), out_shape=(360, 720), grid_in="equiangular", grid_out="legendre-gauss", B=2, C=128, nh=4, theta_cutoff=2 * math.pi / 359),
+}
+
+
+def smooth_field(B, C, nlat, nlon, grid, gen, device, lmax=8, noise=0.25):
+    """(B, C, nlat, nlon) fp32: per channel a random combination of real spherical harmonics up to degree lmax
+    (coefficients N(0,1)/(l+1)) plus noise*N(0,1), standardised to unit variance per channel."""
+    from scipy.special import lpmv
+
+    from torch_harmonics_amd.quadrature import precompute_latitudes
+
+    theta, _ = precompute_latitudes(nlat, grid)
+    x = np.cos(theta.numpy())
+    lam = 2 * np.pi * np.arange(nlon) / nlon
+    basis, damp = [], []
+    for l in range(lmax + 1):
+        for m in range(l + 1):
+            norm = math.sqrt((2 * l + 1) / (4 * math.pi) * math.factorial(l - m) / math.factorial(l + m))
+            leg = norm * lpmv(m, l, x)
+            basis.append(np.outer(leg, np.cos(m * lam)))
+            damp.append(1.0 / (l + 1))
+            if m > 0:
+                basis.append(np.outer(leg, np.sin(m * lam)))
+                damp.append(1.0 / (l + 1))
+    basis = torch.tensor(np.stack(basis), dtype=torch.float32, device=device).reshape(len(damp), -1)
+    damp = torch.tensor(damp, dtype=torch.float32)
+    coef = (torch.randn(B * C, len(damp), generator=gen) * damp).to(device)
+    f = (coef @ basis).reshape(B, C, nlat, nlon)
+    f = f + noise * torch.randn(B, C, nlat, nlon, generator=gen).to(device)
+    f = (f - f.mean(dim=(2, 3), keepdim=True)) / f.std(dim=(2, 3), keepdim=True)
+    return f.contiguous()
+
+
+def make_workload(cfg, device, seed=333):
+    """Module with seeded random weights, its NCHW input, and the op-level tensors k, v, q (scaled), dy in NHWC."""
+    from torch_harmonics_amd import NeighborhoodAttentionS2, to_nhwc
+
+    torch.manual_seed(seed)
+    mod = NeighborhoodAttentionS2(
+        cfg["C"], cfg["in_shape"], cfg["out_shape"], grid_in=cfg["grid_in"], grid_out=cfg["grid_out"], num_heads=cfg["nh"], theta_cutoff=cfg["theta_cutoff"]
+    ).to(device)
+    gen = torch.Generator().manual_seed(seed)
+    x_in = smooth_field(cfg["B"], cfg["C"], *cfg["in_shape"], cfg["grid_in"], gen, device)
+    same = cfg["in_shape"] == cfg["out_shape"] and cfg["grid_in"] == cfg["grid_out"]
+    x_out = x_in if same else smooth_field(cfg["B"], cfg["C"], *cfg["out_shape"], cfg["grid_out"], gen, device)
+    with torch.no_grad():
+        xi, xo = to_nhwc(x_in), to_nhwc(x_out)
+        k = torch.nn.functional.linear(xi, mod.k_weights.view(mod.k_channels, -1), mod.k_bias).contiguous()
+        v = torch.nn.functional.linear(xi, mod.v_weights.view(mod.out_channels, -1), mod.v_bias).contiguous()
+        q = (torch.nn.functional.linear(xo, mod.q_weights.view(mod.k_channels, -1), mod.q_bias) * mod.scale).contiguous()
+        dy = torch.randn(q.shape[:3] + (v.shape[3],), generator=gen).to(device)
+    return mod, x_in, x_out, k, v, q, dy
+
+
+def cpu_baseline(cfg, mod, k, v, q, dy):
+    """
+    Times the fp32 CPU port of the reference algorithm (oracle/s2attn_oracle.c, built with the reference's
+    release flags) forward + backward on a sample of the workload: the first two heads and every 12th output
+    latitude (both pole rows included, so the reference backward's per-neighbor scratch is sized by the longest
+    row, as in the full problem).  Throughput is neighbor pairs of the sample per second.
+    """
+    from oracle import cpu_attention as oracle
+
+    nh_s = min(2, cfg["nh"])
+    ck, cv = mod.k_channels // cfg["nh"], mod.out_channels // cfg["nh"]
+    Ho, Wo = cfg["out_shape"]
+    stride = 12 if Ho >= 120 else 1
+    rows = torch.arange(0, Ho, stride)
+    if rows[-1] != Ho - 1:
+        rows = torch.cat([rows, torch.tensor([Ho - 1])])
+    col, ro = mod.psi_col_idx.cpu(), mod.psi_roff_idx.cpu()
+    lens = (ro[1:] - ro[:-1])[rows]
+    ro_s = torch.zeros(len(rows) + 1, dtype=torch.int64)
+    ro_s[1:] = torch.cumsum(lens, 0)
+    col_s = torch.cat([col[ro[r] : ro[r + 1]] for r in rows.tolist()])
+    ks = k[..., : nh_s * ck].cpu().contiguous()
+    vs = v[..., : nh_s * cv].cpu().contiguous()
+    qs = q[:, rows][..., : nh_s * ck].cpu().contiguous()
+    gs = dy[:, rows][..., : nh_s * cv].cpu().contiguous()
+    w = mod.quad_weights.cpu()
+    pairs = cfg["B"] * nh_s * Wo * int(lens.sum())
+    scratch_gb = 2 * cfg["B"] * nh_s * len(rows) * Wo * int(lens.max()) * 4 / 1e9
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    t0 = time.perf_counter()
+    oracle.forward_f32(ks, vs, qs, w, col_s, ro_s, nh_s, fast=True)
+    t1 = time.perf_counter()
+    oracle.backward_f32(ks, vs, qs, gs, w, col_s, ro_s, nh_s, fast=True)
+    t2 = time.perf_counter()
+    return {
+        "value": pairs / (t2 - t0),
+        "unit": "pairs/s",
+        "cores": cores,
+        "kind": "port",
+        "sample": f"{nh_s} of {cfg['nh']} heads x {len(rows)} of {Ho} output latitudes (every {stride}th, both poles) = {pairs} pairs; "
+        f"fwd {1e3 * (t1 - t0):.0f} ms + bwd {1e3 * (t2 - t1):.0f} ms; reference bwd scratch {scratch_gb:.1f} GB",
+        "fwd_ms": 1e3 * (t1 - t0),
+        "bwd_ms": 1e3 * (t2 - t1),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-module", action="store_true", help="skip the module-level (projections + permutes) timing")
+    args = ap.parse_args()
+
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs a ROCm GPU", file=sys.stderr)
+        sys.exit(2)
+
+    from torch_harmonics_amd import _lib, ops
+    from torch_harmonics_amd.plan import get_plan
+
+    lib = _lib.load()  # raises if libs2attn.so is missing: there is no fallback to time
+    cfg = CONFIGS[args.config]
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    mod, x_in, x_out, k, v, q, dy = make_workload(cfg, dev)
+    (Hi, Wi), (Ho, Wo) = cfg["in_shape"], cfg["out_shape"]
+    nh, B = cfg["nh"], cfg["B"]
+    nnz = mod.psi_col_idx.numel()
+    pairs = B * nh * Wo * nnz
+    wq, ci, ro = mod.quad_weights, mod.psi_col_idx, mod.psi_roff_idx
+    esz = 4
+
+    def step():
+        y = ops.forward(k, v, q, wq, ci, ro, nh, Wi, Ho, Wo)
+        return y, ops.backward(k, v, q, dy, wq, ci, ro, nh, Wi, Ho, Wo)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # ---- per-kernel durations: events on the launch stream around each launch, same K steps ----
+    plan = get_plan(ci, ro, Hi, Wi, Ho, Wo)
+    shape = _lib.ShapeStruct(B, nh, Hi, Wi, Ho, Wo, k.shape[3] // nh, v.shape[3] // nh, _lib.S2ATTN_F32)
+    y = torch.empty(q.shape[:3] + (v.shape[3],), device=dev)
+    dk, dv, dq = torch.empty_like(k), torch.empty_like(v), torch.empty_like(q)
+    ws = torch.empty(lib.s2attn_backward_workspace_bytes(ctypes.byref(shape)) // 4, device=dev)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    pl, sh = ctypes.byref(plan.struct), ctypes.byref(shape)
+    ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
+    for s in range(args.steps):
+        ev[s][0].record()
+        _lib.check(lib.s2attn_forward(k.data_ptr(), v.data_ptr(), q.data_ptr(), wq.data_ptr(), y.data_ptr(), pl, sh, stream), "fwd")
+        ev[s][1].record()
+        _lib.check(lib.s2attn_backward_dq(k.data_ptr(), v.data_ptr(), q.data_ptr(), dy.data_ptr(), wq.data_ptr(), dq.data_ptr(), ws.data_ptr(), pl, sh, stream), "dq")
+        ev[s][2].record()
+        _lib.check(
+            lib.s2attn_backward_dkdv(k.data_ptr(), v.data_ptr(), q.data_ptr(), dy.data_ptr(), wq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), pl, sh, stream), "dkdv"
+        )
+        ev[s][3].record()
+    torch.cuda.synchronize()
+    t_fwd = sum(e[0].elapsed_time(e[1]) for e in ev) / args.steps
+    t_dq = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
+    t_dkdv = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
+
+    nk, nv, nq, ny = k.numel(), v.numel(), q.numel(), y.numel()
+    alg = {  # compulsory traffic of each kernel: every tensor it must read or write, once
+        "s2attn fwd_kernel": (esz * (nq + nk + nv + ny), t_fwd),
+        "s2attn dq_kernel": (esz * (nq + nk + nv + ny + nq), t_dq),
+        "s2attn dkdv_kernel": (esz * (nq + nk + nv + ny + nk + nv), t_dkdv),
+    }
+    dom = max(alg, key=lambda n: alg[n][1])
+    dom_bytes, dom_ms = alg[dom]
+    achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
+    step_bytes = esz * ((nq + nk + nv + ny) + (nq + nk + nv + ny + nq + nk + nv))
+    d = k.shape[3] // nh
+    flops_alg = 14 * d * pairs
+
+    out = {
+        "metric": "NeighborhoodAttentionS2 fwd+bwd neighbor-pairs/s",
+        "value": pairs / (ms_step * 1e-3),
+        "unit": "pairs/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.config}: {cfg['grid_in']} {Hi}x{Wi} -> {cfg['grid_out']} {Ho}x{Wo}, B={B}, C={cfg['C']}, heads={nh}, fp32, theta_cutoff={cfg['theta_cutoff']}, nnz={nnz}, pairs={pairs}",
+            "level": "op (s2attn forward + backward through the C ABI); module-level time in module_ms_per_step",
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": dom,
+            "achieved": achieved,
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": achieved / HBM_PEAK_GBS,
+            "traffic": None,
+            "algorithmic_bytes": dom_bytes,
+            "kernel_ms": dom_ms,
+        },
+        "kernel_ms": {"fwd": t_fwd, "dq": t_dq, "dkdv": t_dkdv},
+        "step_hbm_frac": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "step_fp32_valu_frac": flops_alg / (ms_step * 1e-3) / 1e12 / FP32_VALU_PEAK_TFLOPS,
+    }
+
+    if not args.no_module:
+        xq = x_out.clone().requires_grad_(True)
+        same = x_in is x_out
+        xk = None if same else x_in.clone().requires_grad_(True)
+        gout = torch.randn(B, mod.out_channels, Ho, Wo, device=dev)
+
+        def mstep():
+            o = mod(xq) if same else mod(xq, xk, xk)
+            o.backward(gout)
+            mod.zero_grad(set_to_none=True)
+            xq.grad = None
+            if xk is not None:
+                xk.grad = None
+
+        for _ in range(2):
+            mstep()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        nm = max(3, args.steps // 2)
+        for _ in range(nm):
+            mstep()
+        torch.cuda.synchronize()
+        out["module_ms_per_step"] = 1e3 * (time.perf_counter() - t0) / nm
+
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy)
+
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -110,6 +110,20 @@ int s2attn_backward(const void *k, const void *v, const void *q, const void *dy,
                     void *stream);
 
 /*
+ * The two phases of s2attn_backward as separate launches (same arguments, same workspace), for callers that time
+ * them individually or need only one side.  Together they replace the same reference entry point as
+ * s2attn_backward (attention_cuda_bwd.cu:856-956).
+ *   s2attn_backward_dq    writes dq and fills the workspace with the per-query softmax statistics
+ *   s2attn_backward_dkdv  reads that workspace (so it must follow s2attn_backward_dq on the stream) and writes dk, dv
+ */
+int s2attn_backward_dq(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, void *dq,
+                       void *workspace, const s2attn_plan *plan, const s2attn_shape *shape, void *stream);
+
+int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
+                         void *dk, void *dv, const void *workspace, const s2attn_plan *plan, const s2attn_shape *shape,
+                         void *stream);
+
+/*
  * Layout conversion.  Replace attention_kernels::permute_to_nhwc / permute_to_nchw
  * (attention_interface.cpp:85-86; CUDA kernels attention_cuda_utils.cuh:417-576).
  * Pure element moves; elem_size is 2 or 4 bytes.  dst must not alias src.

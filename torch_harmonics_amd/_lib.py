@@ -57,6 +57,8 @@ SYMBOLS = {
     "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
     "s2attn_backward": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_backward_dq": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_backward_dkdv": (_int, [_vp] * 8 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_permute_to_nhwc": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "s2attn_permute_to_nchw": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
 }

@@ -711,31 +711,65 @@ extern "C" int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape)
     return (int64_t)shape->batch * shape->num_heads * shape->nlat_out * shape->nlon_out * (int64_t)sizeof(float2);
 }
 
-extern "C" int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
-                               void *dk, void *dv, void *dq, void *workspace, const s2attn_plan *plan,
-                               const s2attn_shape *shape, void *stream)
+namespace {
+int backward_args(Args &a, bool &vec, const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, const void *workspace,
+                  const s2attn_plan *plan, const s2attn_shape *shape)
 {
-    int rc = check_shape(shape);
+    const int rc = check_shape(shape);
     if (rc != S2ATTN_OK) return rc;
-    if (!k || !v || !q || !dy || !dk || !dv || !dq || !quad_weights || !workspace) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!k || !v || !q || !dy || !quad_weights || !workspace) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!plan || !plan->gather_off || !plan->gather_order || !plan->scatter_off || !plan->scatter_order
         || (plan->nruns > 0 && (!plan->gather_runs || !plan->scatter_runs)))
         return s2attn_fail(S2ATTN_E_INVALID, "plan is missing arrays");
     if (!aligned(workspace, sizeof(float2))) return s2attn_fail(S2ATTN_E_INVALID, "workspace must be 8-byte aligned");
-    Args a = {};
     fill_args(a, plan, shape, quad_weights);
-    a.k = k, a.v = v, a.q = q, a.dy = dy, a.dk = dk, a.dv = dv, a.dq = dq;
-    a.stats = static_cast<float2 *>(workspace);
+    a.k = k, a.v = v, a.q = q, a.dy = dy;
+    a.stats = static_cast<float2 *>(const_cast<void *>(workspace));
     const size_t al = 4 * (size_t)esize(shape->dtype);
-    const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(dy, al)
-                     && aligned(dk, al) && aligned(dv, al) && aligned(dq, al);
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    a.tile_rows = a.pscale * (TQ - 1) + TL;
-    rc = launch(DQ, a, shape->dtype, vec, st);
+    vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(dy, al);
+    return S2ATTN_OK;
+}
+} // namespace
+
+extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, void *dq,
+                                  void *workspace, const s2attn_plan *plan, const s2attn_shape *shape, void *stream)
+{
+    Args a = {};
+    bool vec = false;
+    const int rc = backward_args(a, vec, k, v, q, dy, quad_weights, workspace, plan, shape);
     if (rc != S2ATTN_OK) return rc;
+    if (!dq) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    a.dq = dq;
+    vec = vec && aligned(dq, 4 * (size_t)esize(shape->dtype));
+    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    return launch(DQ, a, shape->dtype, vec, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
+                                    void *dk, void *dv, const void *workspace, const s2attn_plan *plan,
+                                    const s2attn_shape *shape, void *stream)
+{
+    Args a = {};
+    bool vec = false;
+    const int rc = backward_args(a, vec, k, v, q, dy, quad_weights, workspace, plan, shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!dk || !dv) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    a.dk = dk, a.dv = dv;
+    const size_t al = 4 * (size_t)esize(shape->dtype);
+    vec = vec && aligned(dk, al) && aligned(dv, al);
     a.tile_rows = (TQ - 1) / a.pscale + 1 + TL;
-    if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile is also used to stage the lane-owned k/v and dk/dv rows
-    return launch(DKDV, a, shape->dtype, vec, st);
+    if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile also stages the lane-owned k/v and dk/dv rows
+    return launch(DKDV, a, shape->dtype, vec, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
+                               void *dk, void *dv, void *dq, void *workspace, const s2attn_plan *plan,
+                               const s2attn_shape *shape, void *stream)
+{
+    if (!dk || !dv || !dq) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    const int rc = s2attn_backward_dq(k, v, q, dy, quad_weights, dq, workspace, plan, shape, stream);
+    if (rc != S2ATTN_OK) return rc;
+    return s2attn_backward_dkdv(k, v, q, dy, quad_weights, dk, dv, workspace, plan, shape, stream);
 }
 
 namespace {
