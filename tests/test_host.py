@@ -1,0 +1,295 @@
+"""
+Host-side logic that runs without a GPU: the C ABI's exports and argument checks, the plan builder,
+the product geometry, the module's constructor/state and the operators' shape propagation and errors.
+"""
+
+import ctypes
+import math
+import os
+import re
+from collections import Counter
+
+import pytest
+import torch
+
+import torch_harmonics_amd as tha
+from oracle import geometry as ogeo
+from torch_harmonics_amd import _lib, ops
+from torch_harmonics_amd.neighborhood import precompute_neighborhood_s2
+from torch_harmonics_amd.plan import build_host_plan
+from torch_harmonics_amd.quadrature import precompute_latitudes, precompute_longitudes
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+# ---- C ABI -----------------------------------------------------------------------------------
+
+
+def test_library_loads_and_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "s2attn.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(s2attn_[a-z0-9_]+)\s*\(", header))
+    assert {"s2attn_forward", "s2attn_backward", "s2attn_plan_build", "s2attn_permute_to_nhwc"} <= declared
+    assert declared == set(_lib.SYMBOLS), "ctypes table and header disagree"
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for name in declared:
+        assert hasattr(lib, name), f"{name} is declared in include/s2attn.h but not exported"
+    assert _lib.load().s2attn_abi_version() == _lib.ABI_VERSION
+    assert tha.optimized_kernels_is_available()
+
+
+def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
+    lib = _lib.load()
+    shape = _lib.ShapeStruct(1, 2, 4, 8, 4, 8, 8, 8, _lib.S2ATTN_F32)
+    plan = _lib.PlanStruct(None, None, None, None, None, None, 0)
+    rc = lib.s2attn_forward(None, None, None, None, None, ctypes.byref(plan), ctypes.byref(shape), None)
+    assert rc == -1 and b"null" in lib.s2attn_last_error()
+    bad = _lib.ShapeStruct(1, 2, 4, 9, 4, 6, 8, 8, _lib.S2ATTN_F32)  # 9 % 6 != 0
+    assert lib.s2attn_backward_workspace_bytes(ctypes.byref(bad)) == -1
+    assert b"multiple" in lib.s2attn_last_error()
+    wide = _lib.ShapeStruct(1, 1, 4, 8, 4, 8, 48, 48, _lib.S2ATTN_F32)
+    assert lib.s2attn_backward_workspace_bytes(ctypes.byref(wide)) == -2  # unsupported head width
+    dt = _lib.ShapeStruct(1, 1, 4, 8, 4, 8, 8, 8, 7)
+    assert lib.s2attn_backward_workspace_bytes(ctypes.byref(dt)) == -1
+    assert lib.s2attn_backward_workspace_bytes(ctypes.byref(shape)) == 1 * 2 * 4 * 8 * 8
+    assert lib.s2attn_permute_to_nhwc(None, None, 1, 2, 3, 4, 3, None) == -1  # element size 3
+
+
+# ---- plan builder -------------------------------------------------------------------------------
+
+
+def _pairs_from_csr(col, roff, Wi, Wo):
+    ps = Wi // Wo
+    ref = Counter()
+    for ho in range(len(roff) - 1):
+        for z in range(int(roff[ho]), int(roff[ho + 1])):
+            hi, wi = divmod(int(col[z]), Wi)
+            for wo in range(Wo):
+                ref[(ho, wo, hi, (wi + ps * wo) % Wi)] += 1
+    return ref
+
+
+def _pairs_from_plan(arrays, Hi, Wi, Ho, Wo):
+    """Expands both run groupings back into (ho, wo, hi, wi) pairs the way the kernels index them."""
+    goff, gruns, gorder, soff, sruns, sorder = [a.numpy() for a in arrays]
+    ps = Wi // Wo
+    gather, scatter = Counter(), Counter()
+    for ho in range(Ho):
+        for ri in range(goff[ho], goff[ho + 1]):
+            hi, ws, ln, _ = (int(x) for x in gruns[ri])
+            for wo in range(Wo):
+                for t in range(ln):
+                    gather[(ho, wo, hi, (ws + t + ps * wo) % Wi)] += 1
+    for hi in range(Hi):
+        for ri in range(soff[hi], soff[hi + 1]):
+            ho, ws, ln, _ = (int(x) for x in sruns[ri])
+            for wi in range(Wi):
+                delta = (wi - ws) % Wi
+                t = delta % ps
+                u = 0
+                while t < ln:
+                    scatter[(ho, (delta // ps - u) % Wo, hi, wi)] += 1
+                    u += 1
+                    t += ps
+    return gather, scatter, gorder, sorder
+
+
+@pytest.mark.parametrize(
+    "ins,outs,gi,go,tc",
+    [
+        ((6, 12), (6, 12), "equiangular", "equiangular", None),
+        ((2, 4), (2, 4), "equiangular", "equiangular", None),
+        ((12, 24), (6, 8), "equiangular", "equiangular", None),
+        ((9, 12), (5, 4), "equiangular", "equiangular", None),
+        ((12, 24), (6, 12), "legendre-gauss", "legendre-gauss", 0.7),
+        ((6, 12), (6, 12), "equiangular", "equiangular", 7.0),
+    ],
+)
+def test_plan_covers_exactly_the_csr_pairs(ins, outs, gi, go, tc):
+    col, roff, _ = precompute_neighborhood_s2(ins, outs, gi, go, tc)
+    arrays, nruns = build_host_plan(col, roff, ins[0], ins[1], outs[0], outs[1])
+    ref = _pairs_from_csr(col, roff, ins[1], outs[1])
+    gather, scatter, gorder, sorder = _pairs_from_plan(arrays, ins[0], ins[1], outs[0], outs[1])
+    assert gather == ref and scatter == ref
+    assert sorted(gorder.tolist()) == list(range(outs[0])) and sorted(sorder.tolist()) == list(range(ins[0]))
+    lens = (roff[1:] - roff[:-1]).tolist()
+    assert all(lens[gorder[i]] >= lens[gorder[i + 1]] for i in range(outs[0] - 1)), "rows must be ordered longest first"
+    assert nruns <= col.numel()
+
+
+def test_plan_handles_arbitrary_unsorted_csr_with_duplicates():
+    gen = torch.Generator().manual_seed(5)
+    Hi, Wi, Ho, Wo = 5, 12, 4, 6
+    rows = [torch.randint(0, Hi * Wi, (n,), generator=gen) for n in (7, 0, 19, 3)]
+    col = torch.cat(rows)
+    roff = torch.tensor([0, 7, 7, 26, 29])
+    arrays, nruns = build_host_plan(col, roff, Hi, Wi, Ho, Wo)
+    gather, scatter, _, _ = _pairs_from_plan(arrays, Hi, Wi, Ho, Wo)
+    ref = _pairs_from_csr(col, roff, Wi, Wo)
+    assert gather == ref and scatter == ref
+
+
+def test_plan_merges_wrapping_intervals_into_one_circular_run():
+    Wi = 16
+    col = torch.tensor([0, 1, 2, 14, 15, 16 + 5, 16 + 6])  # lat 0: {14,15,0,1,2}; lat 1: {5,6}
+    roff = torch.tensor([0, 7])
+    arrays, nruns = build_host_plan(col, roff, 2, Wi, 1, Wi)
+    assert nruns == 2
+    assert arrays[1][:2].tolist() == [[0, 14, 5, 0], [1, 5, 2, 0]]
+
+
+def test_plan_builder_rejects_malformed_csr():
+    good_col = torch.tensor([0, 1, 2])
+    with pytest.raises(RuntimeError, match="outside"):
+        build_host_plan(torch.tensor([0, 1, 99]), torch.tensor([0, 3]), 2, 4, 1, 4)
+    with pytest.raises(RuntimeError, match="row_off"):
+        build_host_plan(good_col, torch.tensor([0, 2]), 2, 4, 1, 4)
+    with pytest.raises(RuntimeError, match="multiple"):
+        build_host_plan(good_col, torch.tensor([0, 3]), 2, 4, 1, 3)
+    with pytest.raises(RuntimeError, match="nlat_out"):
+        build_host_plan(good_col, torch.tensor([0, 1, 3]), 2, 4, 1, 4)
+
+
+# ---- geometry -------------------------------------------------------------------------------------
+
+
+@pytest.mark.parametrize("grid", ["equiangular", "legendre-gauss", "lobatto", "equiangular-trapezoidal"])
+@pytest.mark.parametrize("nlat", [2, 5, 32, 33])
+def test_product_quadrature_equals_oracle(grid, nlat):
+    th, w = precompute_latitudes(nlat, grid)
+    tho, wo = ogeo.colatitudes_and_weights(nlat, grid)
+    assert torch.equal(th, tho) and torch.equal(w, wo)
+    assert torch.equal(precompute_longitudes(24), ogeo.longitudes(24))
+    with pytest.raises(ValueError):
+        precompute_latitudes(8, "healpix")
+
+
+@pytest.mark.parametrize(
+    "ins,outs,gi,go,tc",
+    [
+        ((32, 64), (32, 64), "equiangular", "equiangular", None),
+        ((12, 24), (3, 6), "equiangular", "equiangular", None),
+        ((11, 24), (7, 12), "equiangular", "equiangular", None),
+        ((24, 48), (12, 24), "equiangular", "legendre-gauss", 0.3),
+        ((16, 32), (16, 32), "lobatto", "lobatto", 0.25),
+        ((128, 256), (128, 256), "equiangular", "equiangular", 4 * math.pi / 127),
+        ((6, 12), (6, 12), "equiangular", "equiangular", 2 * math.pi),
+    ],
+)
+def test_product_neighborhood_equals_oracle(ins, outs, gi, go, tc):
+    col, roff, row = precompute_neighborhood_s2(ins, outs, gi, go, tc)
+    col_o, roff_o = ogeo.neighborhood_csr(ins, outs, gi, go, tc)
+    assert torch.equal(col, col_o) and torch.equal(roff, roff_o)
+    assert col.dtype == torch.int64 and roff.dtype == torch.int64
+    assert torch.equal(row, torch.repeat_interleave(torch.arange(outs[0]), roff[1:] - roff[:-1]))
+
+
+def test_product_neighborhood_at_benchmark_resolution():
+    col, roff, _ = precompute_neighborhood_s2((721, 1440), (721, 1440), theta_cutoff=3 * math.pi / 720)
+    lens = roff[1:] - roff[:-1]
+    assert col.numel() == 99625 and int(lens.min()) == 29 and int(lens.max()) == 5760 and int(lens.median()) == 41
+
+
+# ---- module ---------------------------------------------------------------------------------------
+
+
+def test_module_state_and_defaults():
+    m = tha.NeighborhoodAttentionS2(8, (12, 24), (6, 12), num_heads=2, k_channels=4, out_channels=6, use_qknorm=True)
+    sd = m.state_dict()
+    assert {k: tuple(v.shape) for k, v in sd.items()} == {
+        "q_weights": (4, 8, 1, 1),
+        "k_weights": (4, 8, 1, 1),
+        "v_weights": (6, 8, 1, 1),
+        "proj_weights": (6, 6, 1, 1),
+        "q_bias": (4,),
+        "k_bias": (4,),
+        "v_bias": (6,),
+        "proj_bias": (6,),
+        "q_norm_weights": (2,),
+        "k_norm_weights": (2,),
+    }
+    assert {n for n, _ in m.named_buffers()} == {"quad_weights", "psi_row_idx", "psi_col_idx", "psi_roff_idx"}
+    assert m.theta_cutoff == pytest.approx(math.pi / 5) and m.scale == pytest.approx(1 / math.sqrt(2))
+    assert m.quad_weights.dtype == torch.float32 and m.quad_weights.shape == (12,)
+    assert m.psi_roff_idx.shape == (7,) and not m.upsample
+    bound = math.sqrt(6.0 / (8 + 4))
+    assert float(m.q_weights.abs().max()) <= bound and float(m.proj_bias.abs().max()) == 0
+    m2 = tha.NeighborhoodAttentionS2(8, (12, 24), (6, 12), num_heads=2, k_channels=4, out_channels=6, use_qknorm=True)
+    m2.load_state_dict(sd)
+    nb = tha.NeighborhoodAttentionS2(4, (6, 12), (6, 12), bias=False)
+    assert nb.q_bias is None and "q_bias" not in nb.state_dict()
+
+
+def test_module_constructor_errors():
+    with pytest.raises(ValueError, match="integer multiple"):
+        tha.NeighborhoodAttentionS2(4, (6, 10), (6, 4))
+    with pytest.raises(ValueError, match="divides k_channels"):
+        tha.NeighborhoodAttentionS2(6, (6, 12), (6, 12), num_heads=4)
+    with pytest.raises(ValueError, match="divides out_channels"):
+        tha.NeighborhoodAttentionS2(4, (6, 12), (6, 12), num_heads=4, out_channels=6)
+    with pytest.raises(ValueError, match="positive"):
+        tha.NeighborhoodAttentionS2(4, (6, 12), (6, 12), theta_cutoff=0.0)
+    with pytest.raises(NotImplementedError):
+        tha.NeighborhoodAttentionS2(4, (6, 12), (12, 24))  # upsampling
+    with pytest.raises(NotImplementedError):
+        tha.NeighborhoodAttentionS2(4, (6, 12), (6, 12), optimized_kernel=False)
+
+
+def test_module_forward_checks_shapes_and_has_no_cpu_path():
+    m = tha.NeighborhoodAttentionS2(4, (12, 24), (6, 12))
+    with pytest.raises(RuntimeError, match="4-dimensional"):
+        m(torch.randn(4, 6, 12))
+    with pytest.raises(RuntimeError, match="query latitudes"):
+        m(torch.randn(1, 4, 7, 12), torch.randn(1, 4, 12, 24), torch.randn(1, 4, 12, 24))
+    with pytest.raises(RuntimeError, match="key longitudes"):
+        m(torch.randn(1, 4, 6, 12), torch.randn(1, 4, 12, 23), torch.randn(1, 4, 12, 24))
+    with pytest.raises(RuntimeError, match="single dtype"):
+        m(torch.randn(1, 4, 6, 12), torch.randn(1, 4, 12, 24).double(), torch.randn(1, 4, 12, 24))
+    with pytest.raises(RuntimeError, match="only run on a ROCm GPU"):
+        m(torch.randn(1, 4, 6, 12), torch.randn(1, 4, 12, 24), torch.randn(1, 4, 12, 24))
+
+
+# ---- operators ------------------------------------------------------------------------------------
+
+
+def _op_args(device="cpu", dtype=torch.float32, nh=2):
+    m = tha.NeighborhoodAttentionS2(8, (12, 24), (6, 12), num_heads=nh)
+    k = torch.randn(2, 12, 24, 8, device=device, dtype=dtype)
+    v = torch.randn(2, 12, 24, 4, device=device, dtype=dtype)
+    q = torch.randn(2, 6, 12, 8, device=device, dtype=dtype)
+    psi = [t.to(device) for t in (m.quad_weights, m.psi_col_idx, m.psi_roff_idx)]
+    return k, v, q, psi
+
+
+def test_operator_shape_propagation_on_meta_tensors():
+    k, v, q, psi = _op_args("meta", torch.bfloat16)
+    y = ops._neighborhood_s2_attention_optimized(k, v, q, *psi, 2, 24, 6, 12)
+    assert y.shape == (2, 6, 12, 4) and y.dtype == torch.bfloat16 and y.device.type == "meta"
+    y = ops.forward(k, v, q, *psi, 2, 24, 6, 12)
+    assert y.shape == (2, 6, 12, 4)
+    dk, dv, dq = ops.backward(k, v, q, y, *psi, 2, 24, 6, 12)
+    assert dk.shape == k.shape and dv.shape == v.shape and dq.shape == q.shape
+    x = torch.empty(2, 3, 4, 5, device="meta")
+    assert ops.permute_to_nhwc(x).shape == (2, 4, 5, 3) and ops.permute_to_nchw(x).shape == (2, 5, 3, 4)
+
+
+def test_operator_argument_errors():
+    k, v, q, psi = _op_args()
+    with pytest.raises(RuntimeError, match="divisible by num_heads"):
+        ops.forward(k, v, q, *psi, 3, 24, 6, 12)
+    with pytest.raises(RuntimeError, match="must match q dtype"):
+        ops.forward(k.double(), v, q, *psi, 2, 24, 6, 12)
+    with pytest.raises(RuntimeError, match="vice versa"):
+        ops.forward(k, v, q, *psi, 2, 24, 6, 9)
+    with pytest.raises(RuntimeError, match="num_heads must be positive"):
+        ops.forward(k, v, q, *psi, 0, 24, 6, 12)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.forward(k.transpose(1, 2), v, q, *psi, 2, 24, 6, 12)
+    with pytest.raises(RuntimeError, match="dy dtype"):
+        ops.backward(k, v, q, torch.randn(2, 6, 12, 4).half(), *psi, 2, 24, 6, 12)
+    with pytest.raises(RuntimeError, match="only run on a ROCm GPU"):
+        ops.forward(k, v, q, *psi, 2, 24, 6, 12)
+    with pytest.raises(RuntimeError, match="only run on a ROCm GPU"):
+        ops.permute_to_nhwc(torch.randn(1, 2, 3, 4))
+    with pytest.raises(NotImplementedError):
+        ops.forward(q, q[..., :4].contiguous(), k, *psi, 2, 12, 12, 24)  # upsampling direction

@@ -15,11 +15,15 @@ def _check_extent(tensor: torch.Tensor, dim: int, expected: int, name: str) -> N
     torch._check(tensor.shape[dim] == expected, lambda: f"Expected {name} shape[{dim}] == {expected}")
 
 
+def _dtype_mismatch_message() -> str:
+    return "all attention inputs must share a single dtype"
+
+
 def _check_dtypes_match(tensors) -> None:
     """RuntimeError unless all tensors share one dtype: the kernels read every activation as q's element type."""
     first = tensors[0].dtype
     for t in tensors[1:]:
-        torch._check(t.dtype == first, "all attention inputs must share a single dtype")
+        torch._check(t.dtype == first, _dtype_mismatch_message)
 
 
 def _setup_context_attention_backward(ctx, inputs, output):
