@@ -131,6 +131,23 @@ __device__ inline void store4(f16_t *p, float4 v)
     *reinterpret_cast<uint2 *>(p) = r.u;
 }
 
+
+// raw 4-channel fetch (kept in registers while a band is in flight) and its widening to fp32
+__device__ inline float4 widen4(float4 r, const float *) { return r; }
+__device__ inline float4 widen4(uint2 r, const bf16_t *)
+{
+    return make_float4(__uint_as_float(r.x << 16), __uint_as_float(r.x & 0xffff0000u), __uint_as_float(r.y << 16), __uint_as_float(r.y & 0xffff0000u));
+}
+__device__ inline float4 widen4(uint2 r, const f16_t *)
+{
+    union {
+        uint2 u;
+        _Float16 h[4];
+    } c;
+    c.u = r;
+    return make_float4((float)c.h[0], (float)c.h[1], (float)c.h[2], (float)c.h[3]);
+}
+
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
@@ -562,6 +579,448 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
 }
 
 // ---------------------------------------------------------------------------------
+// Software-pipelined band staging (fast path: vector loads, pscale == 1, nlon >= tile rows).
+// A band of up to TQ-1+TL grid points is fetched into registers with one 16-byte (8-byte for
+// 16-bit storage) load per lane and iteration, NIT iterations, while the previous band is being
+// consumed from LDS; it is written to LDS afterwards.  Lane constants: row r0 = lane / (P/4) of
+// each group of RPI rows, channel offset cb = 4 * (lane % (P/4)).
+// ---------------------------------------------------------------------------------
+template <typename T, int P> struct Band {
+    static constexpr int V4 = P / 4;
+    static constexpr int RPI = TQ / V4;                       // rows fetched per iteration
+    static constexpr int NIT = (TQ - 1 + TL + RPI - 1) / RPI; // iterations for the largest band
+    static constexpr int LS = P + 4;
+    typedef typename Vec4<T>::type raw_t;
+    raw_t raw[NIT];
+
+    // src: (batch, latitude, longitude 0, head); ld: elements between longitudes.  All NIT * RPI rows are fetched
+    // (rows past the band wrap to valid longitudes and are never read back), so there is no predication; the
+    // fast path requires the head dim to equal P, so every lane's channel offset is valid.
+    __device__ inline void fetch(const T *src, unsigned ld, int c0, int W, int r0, int cb)
+    {
+        const int colA = c0 + r0;
+#pragma unroll
+        for (int it = 0; it < NIT; it++) {
+            int col = colA + it * RPI;
+            col -= (col >= W) ? W : 0;
+            raw[it] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
+        }
+    }
+    __device__ inline void commit(float *dst, int r0, int cb) const
+    {
+#pragma unroll
+        for (int it = 0; it < NIT; it++) *reinterpret_cast<float4 *>(dst + (r0 + it * RPI) * LS + cb) = widen4(raw[it], (const T *)nullptr);
+    }
+};
+
+#define S2_TILE_IDS(W_TILED)                                                   \
+    const int lane = threadIdx.x;                                             \
+    const int BH = a.B * a.nh;                                                \
+    const int ntile = ((W_TILED) + TQ - 1) / TQ;                              \
+    int id_ = blockIdx.x;                                                     \
+    const int bh = id_ % BH;                                                  \
+    id_ /= BH;                                                                \
+    const int wt = id_ % ntile;                                               \
+    const int rowsel = id_ / ntile;                                           \
+    const int b = bh / a.nh, h = bh % a.nh;                                   \
+    const int w0 = wt * TQ;                                                   \
+    const int nvalid = min(TQ, (W_TILED)-w0);
+
+// forward, fast path
+template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kernel(const Args a)
+{
+    typedef Band<T, P> BandT;
+    constexpr int LS = P + 4;
+    constexpr int ROWS = BandT::NIT * BandT::RPI;
+    extern __shared__ float4 smem4[];
+    float *Ks = reinterpret_cast<float *>(smem4);
+    float *Vs = Ks + ROWS * LS;
+
+    S2_TILE_IDS(a.Wo)
+    const int ho = a.gorder[rowsel];
+    const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
+    const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
+
+    const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * a.dk_;
+    const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * a.dv_;
+    const T *qy = static_cast<const T *>(a.q) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldk + (size_t)h * a.dk_;
+    T *y = static_cast<T *>(a.y) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldv + (size_t)h * a.dv_;
+
+    stage_rows<T, P, true>(Ks, qy, ldk, a.dk_, w0, a.Wo, nvalid, lane);
+    __syncthreads();
+    float qr[P], acc[P];
+#pragma unroll
+    for (int c = 0; c < P; c++) {
+        qr[c] = Ks[lane * LS + c] * LOG2E;
+        acc[c] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f;
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int t0 = 0;
+    Run run = {0, 0, 0, 0};
+    BandT kb, vb;
+    auto fetch = [&](const Run &rn, int t) {
+        int c0 = rn.ws + t + w0;
+        c0 -= (c0 >= a.Wi) ? a.Wi : 0;
+        c0 -= (c0 >= a.Wi) ? a.Wi : 0;
+        kb.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, r0, cb);
+        vb.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, r0, cb);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+    }
+    __syncthreads();
+    if (ri < rend) {
+        kb.commit(Ks, r0, cb);
+        vb.commit(Vs, r0, cb);
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const int L = min(TL, run.len - t0);
+        const float w = a.quad_w[run.lat];
+        int nri = ri, nt0 = t0 + TL;
+        Run nrun = run;
+        if (nt0 >= run.len) {
+            nri++;
+            nt0 = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, nt0);
+
+        const float *krow = Ks + lane * LS;
+        const float *vrow = Vs + lane * LS;
+        float s[TL];
+        float cm = NEG_BIG;
+#pragma unroll
+        for (int t = 0; t < TL; t++) {
+            s[t] = NEG_BIG;
+            if (t < L) {
+                s[t] = dot_row<P>(qr, krow + t * LS);
+                cm = fmaxf(cm, s[t]);
+            }
+        }
+        const float mn = fmaxf(m, cm);
+        if (__any(mn > m)) {
+            const float corr = fast_exp2(m - mn);
+            S *= corr;
+#pragma unroll
+            for (int c = 0; c < P; c++) acc[c] *= corr;
+        }
+        m = mn;
+#pragma unroll
+        for (int t = 0; t < TL; t++) {
+            if (t < L) {
+                const float p = fast_exp2(s[t] - mn) * w;
+                S += p;
+                const float *vr = vrow + t * LS;
+#pragma unroll
+                for (int c = 0; c < P; c += 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(vr + c);
+                    acc[c + 0] = fmaf(p, x.x, acc[c + 0]);
+                    acc[c + 1] = fmaf(p, x.y, acc[c + 1]);
+                    acc[c + 2] = fmaf(p, x.z, acc[c + 2]);
+                    acc[c + 3] = fmaf(p, x.w, acc[c + 3]);
+                }
+            }
+        }
+        __syncthreads();
+        if (more) {
+            kb.commit(Ks, r0, cb);
+            vb.commit(Vs, r0, cb);
+        }
+        __syncthreads();
+        ri = nri;
+        t0 = nt0;
+        run = nrun;
+    }
+
+    const float inv = 1.0f / S;
+#pragma unroll
+    for (int c = 0; c < P; c += 4)
+        *reinterpret_cast<float4 *>(Ks + lane * LS + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
+    __syncthreads();
+    unstage_rows<T, P, true>(y, Ks, ldv, a.dv_, w0, nvalid, lane);
+}
+
+// backward dq + statistics, fast path
+template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kernel(const Args a)
+{
+    typedef Band<T, P> BandT;
+    constexpr int LS = P + 4;
+    constexpr int ROWS = BandT::NIT * BandT::RPI;
+    extern __shared__ float4 smem4[];
+    float *Ks = reinterpret_cast<float *>(smem4);
+    float *Vs = Ks + ROWS * LS;
+
+    S2_TILE_IDS(a.Wo)
+    const int ho = a.gorder[rowsel];
+    const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
+    const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
+
+    const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * a.dk_;
+    const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * a.dv_;
+    const T *qy = static_cast<const T *>(a.q) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldk + (size_t)h * a.dk_;
+    const T *gy = static_cast<const T *>(a.dy) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldv + (size_t)h * a.dv_;
+    T *dq = static_cast<T *>(a.dq) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldk + (size_t)h * a.dk_;
+
+    stage_rows<T, P, true>(Ks, qy, ldk, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, P, true>(Vs, gy, ldv, a.dv_, w0, a.Wo, nvalid, lane);
+    __syncthreads();
+    float qr[P], gr[P], Ak[P], Akg[P];
+#pragma unroll
+    for (int c = 0; c < P; c++) {
+        qr[c] = Ks[lane * LS + c] * LOG2E;
+        gr[c] = Vs[lane * LS + c];
+        Ak[c] = 0.f;
+        Akg[c] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f, Ag = 0.f;
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int t0 = 0;
+    Run run = {0, 0, 0, 0};
+    BandT kb, vb;
+    auto fetch = [&](const Run &rn, int t) {
+        int c0 = rn.ws + t + w0;
+        c0 -= (c0 >= a.Wi) ? a.Wi : 0;
+        c0 -= (c0 >= a.Wi) ? a.Wi : 0;
+        kb.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, r0, cb);
+        vb.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, r0, cb);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+    }
+    __syncthreads();
+    if (ri < rend) {
+        kb.commit(Ks, r0, cb);
+        vb.commit(Vs, r0, cb);
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const int L = min(TL, run.len - t0);
+        const float w = a.quad_w[run.lat];
+        int nri = ri, nt0 = t0 + TL;
+        Run nrun = run;
+        if (nt0 >= run.len) {
+            nri++;
+            nt0 = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, nt0);
+
+        const float *krow = Ks + lane * LS;
+        const float *vrow = Vs + lane * LS;
+        float s[TL], g[TL];
+        float cm = NEG_BIG;
+#pragma unroll
+        for (int t = 0; t < TL; t++) {
+            s[t] = NEG_BIG;
+            g[t] = 0.f;
+            if (t < L) {
+                s[t] = dot_row<P>(qr, krow + t * LS);
+                g[t] = dot_row<P>(gr, vrow + t * LS);
+                cm = fmaxf(cm, s[t]);
+            }
+        }
+        const float mn = fmaxf(m, cm);
+        if (__any(mn > m)) {
+            const float corr = fast_exp2(m - mn);
+            S *= corr;
+            Ag *= corr;
+#pragma unroll
+            for (int c = 0; c < P; c++) {
+                Ak[c] *= corr;
+                Akg[c] *= corr;
+            }
+        }
+        m = mn;
+#pragma unroll
+        for (int t = 0; t < TL; t++) {
+            if (t < L) {
+                const float p = fast_exp2(s[t] - mn) * w;
+                const float pg = p * g[t];
+                S += p;
+                Ag += pg;
+                const float *kr = krow + t * LS;
+#pragma unroll
+                for (int c = 0; c < P; c += 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(kr + c);
+                    Ak[c + 0] = fmaf(p, x.x, Ak[c + 0]);
+                    Ak[c + 1] = fmaf(p, x.y, Ak[c + 1]);
+                    Ak[c + 2] = fmaf(p, x.z, Ak[c + 2]);
+                    Ak[c + 3] = fmaf(p, x.w, Ak[c + 3]);
+                    Akg[c + 0] = fmaf(pg, x.x, Akg[c + 0]);
+                    Akg[c + 1] = fmaf(pg, x.y, Akg[c + 1]);
+                    Akg[c + 2] = fmaf(pg, x.z, Akg[c + 2]);
+                    Akg[c + 3] = fmaf(pg, x.w, Akg[c + 3]);
+                }
+            }
+        }
+        __syncthreads();
+        if (more) {
+            kb.commit(Ks, r0, cb);
+            vb.commit(Vs, r0, cb);
+        }
+        __syncthreads();
+        ri = nri;
+        t0 = nt0;
+        run = nrun;
+    }
+
+    const float inv = 1.0f / S;
+    const float I = Ag * inv;
+    if (lane < nvalid) a.stats[((size_t)bh * a.Ho + ho) * a.Wo + w0 + lane] = make_float2(m + fast_log2(S), I);
+#pragma unroll
+    for (int c = 0; c < P; c += 4)
+        *reinterpret_cast<float4 *>(Ks + lane * LS + c)
+            = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
+                          (Akg[c + 3] - I * Ak[c + 3]) * inv);
+    __syncthreads();
+    unstage_rows<T, P, true>(dq, Ks, ldk, a.dk_, w0, nvalid, lane);
+}
+
+// backward dk/dv, fast path (pscale == 1: the queries that see input longitude wi through run (ho, ws, len)
+// are wo = wi - ws - t, t in [0, len))
+template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_kernel(const Args a)
+{
+    typedef Band<T, P> BandT;
+    constexpr int LS = P + 4;
+    constexpr int ROWS = BandT::NIT * BandT::RPI;
+    extern __shared__ float4 smem4[];
+    float *Qs = reinterpret_cast<float *>(smem4);
+    float *Gs = Qs + ROWS * LS;
+    float2 *Ss = reinterpret_cast<float2 *>(Gs + ROWS * LS);
+
+    S2_TILE_IDS(a.Wi)
+    const int hi = a.sorder[rowsel];
+    const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
+    const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
+
+    const T *kx = static_cast<const T *>(a.k) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldk + (size_t)h * a.dk_;
+    const T *vx = static_cast<const T *>(a.v) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldv + (size_t)h * a.dv_;
+    const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldk + (size_t)h * a.dk_;
+    const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * a.dv_;
+    const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
+    T *dk = static_cast<T *>(a.dk) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldk + (size_t)h * a.dk_;
+    T *dv = static_cast<T *>(a.dv) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldv + (size_t)h * a.dv_;
+
+    stage_rows<T, P, true>(Qs, kx, ldk, a.dk_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, P, true>(Gs, vx, ldv, a.dv_, w0, a.Wi, nvalid, lane);
+    __syncthreads();
+    float kr[P], vr[P], dkr[P], dvr[P];
+#pragma unroll
+    for (int c = 0; c < P; c++) {
+        kr[c] = Qs[lane * LS + c] * LOG2E;
+        vr[c] = Gs[lane * LS + c];
+        dkr[c] = 0.f;
+        dvr[c] = 0.f;
+    }
+    const float w = a.quad_w[hi];
+
+    int ri = a.soff[hi];
+    const int rend = a.soff[hi + 1];
+    int u0 = 0;
+    Run run = {0, 0, 0, 0};
+    BandT qb, gb;
+    float2 sraw[2];
+    auto fetch = [&](const Run &rn, int u) {
+        const int UL = min(TL, rn.len - u);
+        int c0 = w0 - rn.ws - u - UL + 1; // first query longitude of the band, in (-2 Wo, Wo)
+        c0 += (c0 < 0) ? a.Wo : 0;
+        c0 += (c0 < 0) ? a.Wo : 0;
+        const int nrows = nvalid - 1 + UL;
+        qb.fetch(qy + (size_t)rn.lat * a.Wo * ldk, ldk, c0, a.Wo, r0, cb);
+        gb.fetch(gy + (size_t)rn.lat * a.Wo * ldv, ldv, c0, a.Wo, r0, cb);
+        const float2 *sl = stats + (size_t)rn.lat * a.Wo;
+#pragma unroll
+        for (int it = 0; it < 2; it++) {
+            const int r = lane + it * TQ;
+            int col = c0 + r;
+            col -= (col >= a.Wo) ? a.Wo : 0;
+            sraw[it] = make_float2(0.f, 0.f);
+            if (r < nrows) sraw[it] = sl[col];
+        }
+    };
+    auto commit = [&]() {
+        qb.commit(Qs, r0, cb);
+        gb.commit(Gs, r0, cb);
+        Ss[lane] = sraw[0];
+        if (lane + TQ < ROWS) Ss[lane + TQ] = sraw[1];
+    };
+    if (ri < rend) {
+        run = a.sruns[ri];
+        fetch(run, 0);
+    }
+    __syncthreads();
+    if (ri < rend) commit();
+    __syncthreads();
+
+    while (ri < rend) {
+        const int UL = min(TL, run.len - u0);
+        int nri = ri, nu0 = u0 + TL;
+        Run nrun = run;
+        if (nu0 >= run.len) {
+            nri++;
+            nu0 = 0;
+            if (nri < rend) nrun = a.sruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, nu0);
+
+#pragma unroll
+        for (int j = 0; j < TL; j++) {
+            if (j < UL) {
+                const int row = lane + (UL - 1 - j);
+                const float *qrow = Qs + row * LS;
+                const float *grow = Gs + row * LS;
+                const float s = dot_row<P>(kr, qrow);
+                const float g = dot_row<P>(vr, grow);
+                const float2 st = Ss[row];
+                const float p = fast_exp2(s - st.x) * w;
+                const float coef = p * (g - st.y);
+#pragma unroll
+                for (int c = 0; c < P; c += 4) {
+                    const float4 x = *reinterpret_cast<const float4 *>(qrow + c);
+                    const float4 z = *reinterpret_cast<const float4 *>(grow + c);
+                    dkr[c + 0] = fmaf(coef, x.x, dkr[c + 0]);
+                    dkr[c + 1] = fmaf(coef, x.y, dkr[c + 1]);
+                    dkr[c + 2] = fmaf(coef, x.z, dkr[c + 2]);
+                    dkr[c + 3] = fmaf(coef, x.w, dkr[c + 3]);
+                    dvr[c + 0] = fmaf(p, z.x, dvr[c + 0]);
+                    dvr[c + 1] = fmaf(p, z.y, dvr[c + 1]);
+                    dvr[c + 2] = fmaf(p, z.z, dvr[c + 2]);
+                    dvr[c + 3] = fmaf(p, z.w, dvr[c + 3]);
+                }
+            }
+        }
+        __syncthreads();
+        if (more) commit();
+        __syncthreads();
+        ri = nri;
+        u0 = nu0;
+        run = nrun;
+    }
+
+#pragma unroll
+    for (int c = 0; c < P; c += 4) {
+        *reinterpret_cast<float4 *>(Qs + lane * LS + c) = make_float4(dkr[c], dkr[c + 1], dkr[c + 2], dkr[c + 3]);
+        *reinterpret_cast<float4 *>(Gs + lane * LS + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
+    }
+    __syncthreads();
+    unstage_rows<T, P, true>(dk, Qs, ldk, a.dk_, w0, nvalid, lane);
+    unstage_rows<T, P, true>(dv, Gs, ldv, a.dv_, w0, nvalid, lane);
+}
+
+// ---------------------------------------------------------------------------------
 // layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
 // ---------------------------------------------------------------------------------
 template <typename E> __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ src, E *__restrict__ dst, long R, long S)
@@ -612,23 +1071,28 @@ bool aligned(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) %
 
 enum Which { FWD, DQ, DKDV };
 
-template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a, hipStream_t stream)
+template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a0, hipStream_t stream)
 {
+    Args a = a0;
     const int BH = a.B * a.nh;
     constexpr int LS = P + 4;
     void (*kern)(const Args) = nullptr;
     long nblocks = 0;
     size_t lds = 0;
+    // fast path: 16-byte loads, equal longitude counts, and a grid at least as wide as one staged band
+    constexpr int FAST_ROWS = Band<T, P>::NIT * Band<T, P>::RPI;
+    const bool fast = VEC && a.pscale == 1 && a.Wi >= FAST_ROWS && a.dk_ == P && a.dv_ == P;
+    if (fast) a.tile_rows = FAST_ROWS;
     if (which == FWD) {
-        kern = fwd_kernel<T, P, VEC>;
+        kern = fast ? fwd_fast_kernel<T, P> : fwd_kernel<T, P, VEC>;
         nblocks = (long)a.Ho * ((a.Wo + TQ - 1) / TQ) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
     } else if (which == DQ) {
-        kern = dq_kernel<T, P, VEC>;
+        kern = fast ? dq_fast_kernel<T, P> : dq_kernel<T, P, VEC>;
         nblocks = (long)a.Ho * ((a.Wo + TQ - 1) / TQ) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
     } else {
-        kern = dkdv_kernel<T, P, VEC>;
+        kern = fast ? dkdv_fast_kernel<T, P> : dkdv_kernel<T, P, VEC>;
         nblocks = (long)a.Hi * ((a.Wi + TQ - 1) / TQ) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
     }
