@@ -52,22 +52,26 @@ int s2attn_abi_version(void);
  * gather runs   grouped by output latitude ho:  lat = hi, neighbors (hi, (ws + t + pscale*wo) mod nlon_in), t in [0, len)
  * scatter runs  the same runs grouped by input latitude hi: lat = ho
  *
- * plus, for each grouping, the group offsets and the groups ordered by
- * decreasing work (longest first), which is the launch order of the kernels.
+ * plus, for each grouping, the group offsets and a launch order of the groups.  The order lists first the
+ * latitudes whose runs are long enough for the dense matrix-core kernels (ndense of them, most work first) and
+ * then the others for the vector kernels (most work first); starting the longest latitudes first is the load
+ * balancing for the ~200:1 spread of row lengths between the poles and the equator.
  * Any CSR is representable (worst case every entry is its own run).
  *
  * s2attn_plan_count   number of runs the CSR decomposes into, or a negative error.
  * s2attn_plan_build   fills caller-allocated host arrays:
  *     gather_off  [nlat_out+1]   gather_runs  [4*nruns]   gather_order  [nlat_out]
  *     scatter_off [nlat_in+1]    scatter_runs [4*nruns]   scatter_order [nlat_in]
- * The caller copies the six arrays to the device and passes them in s2attn_plan.
+ *     ndense [2]  number of dense latitudes at the front of gather_order and of scatter_order
+ * The caller copies the six arrays to the device and passes them, with the two counts, in s2attn_plan.
  */
 int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
                           int nlat_out, int nlon_out);
 
 int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
                       int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
-                      int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order);
+                      int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order,
+                      int32_t *ndense);
 
 typedef struct s2attn_plan {
     const int32_t *gather_off;    /* device, [nlat_out+1] */
@@ -77,6 +81,8 @@ typedef struct s2attn_plan {
     const int32_t *scatter_runs;  /* device, [4*nruns]    (backward only) */
     const int32_t *scatter_order; /* device, [nlat_in]    (backward only) */
     int64_t nruns;
+    int32_t gather_ndense;  /* leading entries of gather_order that go to the dense kernels  */
+    int32_t scatter_ndense; /* leading entries of scatter_order that go to the dense kernels */
 } s2attn_plan;
 
 typedef struct s2attn_shape {

@@ -107,7 +107,7 @@ def _pairs_from_plan(arrays, Hi, Wi, Ho, Wo):
 )
 def test_plan_covers_exactly_the_csr_pairs(ins, outs, gi, go, tc):
     col, roff, _ = precompute_neighborhood_s2(ins, outs, gi, go, tc)
-    arrays, nruns = build_host_plan(col, roff, ins[0], ins[1], outs[0], outs[1])
+    arrays, nruns, ndense = build_host_plan(col, roff, ins[0], ins[1], outs[0], outs[1])
     ref = _pairs_from_csr(col, roff, ins[1], outs[1])
     gather, scatter, gorder, sorder = _pairs_from_plan(arrays, ins[0], ins[1], outs[0], outs[1])
     assert gather == ref and scatter == ref
@@ -123,7 +123,7 @@ def test_plan_handles_arbitrary_unsorted_csr_with_duplicates():
     rows = [torch.randint(0, Hi * Wi, (n,), generator=gen) for n in (7, 0, 19, 3)]
     col = torch.cat(rows)
     roff = torch.tensor([0, 7, 7, 26, 29])
-    arrays, nruns = build_host_plan(col, roff, Hi, Wi, Ho, Wo)
+    arrays, nruns, ndense = build_host_plan(col, roff, Hi, Wi, Ho, Wo)
     gather, scatter, _, _ = _pairs_from_plan(arrays, Hi, Wi, Ho, Wo)
     ref = _pairs_from_csr(col, roff, Wi, Wo)
     assert gather == ref and scatter == ref
@@ -133,7 +133,7 @@ def test_plan_merges_wrapping_intervals_into_one_circular_run():
     Wi = 16
     col = torch.tensor([0, 1, 2, 14, 15, 16 + 5, 16 + 6])  # lat 0: {14,15,0,1,2}; lat 1: {5,6}
     roff = torch.tensor([0, 7])
-    arrays, nruns = build_host_plan(col, roff, 2, Wi, 1, Wi)
+    arrays, nruns, ndense = build_host_plan(col, roff, 2, Wi, 1, Wi)
     assert nruns == 2
     assert arrays[1][:2].tolist() == [[0, 14, 5, 0], [1, 5, 2, 0]]
 

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -31,6 +31,8 @@ class PlanStruct(ctypes.Structure):
         ("scatter_runs", _vp),
         ("scatter_order", _vp),
         ("nruns", _i64),
+        ("gather_ndense", ctypes.c_int32),
+        ("scatter_ndense", ctypes.c_int32),
     ]
 
 
@@ -53,7 +55,7 @@ SYMBOLS = {
     "s2attn_last_error": (ctypes.c_char_p, []),
     "s2attn_abi_version": (_int, []),
     "s2attn_plan_count": (_i64, [_vp, _vp, _i64, _int, _int, _int, _int]),
-    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
     "s2attn_backward": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),

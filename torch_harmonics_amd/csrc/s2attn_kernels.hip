@@ -40,7 +40,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 1; }
+extern "C" int s2attn_abi_version(void) { return 2; }
 
 namespace s2 {
 
@@ -223,6 +223,7 @@ struct Args {
     const Run *gruns, *sruns;
     int B, nh, Hi, Wi, Ho, Wo, dk_, dv_, pscale;
     int tile_rows; // LDS rows per staged band
+    int row_first; // first entry of gorder / sorder this launch covers (dense rows come first, see s2attn_plan_split)
 };
 
 // ---------------------------------------------------------------------------------
@@ -242,7 +243,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd
     const int bh = id % BH;
     id /= BH;
     const int wt = id % ntile;
-    const int ho = a.gorder[id / ntile];
+    const int ho = a.gorder[a.row_first + id / ntile];
     const int b = bh / a.nh, h = bh % a.nh;
     const int wo0 = wt * TQ;
     const int nvalid = min(TQ, a.Wo - wo0);
@@ -344,7 +345,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dq_
     const int bh = id % BH;
     id /= BH;
     const int wt = id % ntile;
-    const int ho = a.gorder[id / ntile];
+    const int ho = a.gorder[a.row_first + id / ntile];
     const int b = bh / a.nh, h = bh % a.nh;
     const int wo0 = wt * TQ;
     const int nvalid = min(TQ, a.Wo - wo0);
@@ -467,7 +468,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
     const int bh = id % BH;
     id /= BH;
     const int ct = id % ntile;
-    const int hi = a.sorder[id / ntile];
+    const int hi = a.sorder[a.row_first + id / ntile];
     const int b = bh / a.nh, h = bh % a.nh;
     const int wi0 = ct * TQ;
     const int nvalid = min(TQ, a.Wi - wi0);
@@ -637,7 +638,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kern
     float *Vs = Ks + ROWS * LS;
 
     S2_TILE_IDS(a.Wo)
-    const int ho = a.gorder[rowsel];
+    const int ho = a.gorder[a.row_first + rowsel];
     const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
     const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
 
@@ -758,7 +759,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kerne
     float *Vs = Ks + ROWS * LS;
 
     S2_TILE_IDS(a.Wo)
-    const int ho = a.gorder[rowsel];
+    const int ho = a.gorder[a.row_first + rowsel];
     const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
     const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
 
@@ -901,7 +902,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
     float2 *Ss = reinterpret_cast<float2 *>(Gs + ROWS * LS);
 
     S2_TILE_IDS(a.Wi)
-    const int hi = a.sorder[rowsel];
+    const int hi = a.sorder[a.row_first + rowsel];
     const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
     const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
 
@@ -1020,6 +1021,194 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
     unstage_rows<T, P, true>(dv, Gs, ldv, a.dv_, w0, nvalid, lane);
 }
 
+
+// ---------------------------------------------------------------------------------
+// Dense (matrix-core) kernels for latitudes whose runs are long: near the poles a query sees hundreds to thousands
+// of consecutive longitudes per latitude, which is a dense 32 x 32 block problem.  fp32 MFMA (v_mfma_f32_32x32x2_f32)
+// runs at twice the non-packed vector rate and keeps fp32 products and accumulation.
+//
+// One wavefront owns 32 consecutive longitudes (lane l: column j = l % 32, half = l / 32) and walks each run in
+// tiles of 32 band positions u (query j sees u - j in [0, len)).  Register layout facts used throughout:
+//   A operand: lane l supplies A[i = l % 32][k = l / 32];  B operand: lane l supplies B[k = l / 32][j = l % 32];
+//   D: register v of lane l holds D[i = 8 (v / 4) + 4 (l / 32) + v % 4][j = l % 32].
+// Scores are produced transposed, S^T[key][query] = K Q^T, so that a lane holds 16 keys of ITS query column: the
+// softmax row statistics need one cross-half exchange, and the 16 probability registers are, unchanged, the B
+// operand of the second product Y^T[channel][query] += V^T[channel][key] P^T[key][query] when MFMA step v uses the
+// keys kappa(v, half) = 8 (v / 4) + 4 half + v % 4.
+// ---------------------------------------------------------------------------------
+typedef float f16v __attribute__((ext_vector_type(16)));
+constexpr int MT = 32;        // queries and keys per tile
+constexpr int MLK = 36;       // LDS row stride of the K-side tile (128-bit reads, rows 16 B-group skewed)
+constexpr int MLV = 40;       // LDS row stride of the V-side tile (32-bit reads by channel; the two halves read rows 4 apart)
+
+__device__ inline int kappa(int v, int half) { return 8 * (v / 4) + 4 * half + (v % 4); }
+
+// fetch one 32-row tile (rows c0.., wrapping once at W) of a latitude/head into registers: 4 loads of 16 B per lane
+template <typename T> struct Tile32 {
+    typedef typename Vec4<T>::type raw_t;
+    raw_t raw[4];
+    __device__ inline void fetch(const T *src, unsigned ld, int c0, int W, int lane)
+    {
+        const int colA = c0 + (lane >> 3), cb = 4 * (lane & 7);
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            int col = colA + it * 8;
+            col -= (col >= W) ? W : 0;
+            raw[it] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
+        }
+    }
+    template <int LS> __device__ inline void commit(float *dst, int lane) const
+    {
+        const int r0 = lane >> 3, cb = 4 * (lane & 7);
+#pragma unroll
+        for (int it = 0; it < 4; it++) *reinterpret_cast<float4 *>(dst + (r0 + it * 8) * LS + cb) = widen4(raw[it], (const T *)nullptr);
+    }
+};
+
+#define S2_MFMA_IDS(W_TILED)                                                  \
+    const int lane = threadIdx.x;                                             \
+    const int j = lane & 31, half = lane >> 5;                                \
+    const int BH = a.B * a.nh;                                                \
+    const int ntile = ((W_TILED) + MT - 1) / MT;                              \
+    int id_ = blockIdx.x;                                                     \
+    const int bh = id_ % BH;                                                  \
+    id_ /= BH;                                                                \
+    const int wt = id_ % ntile;                                               \
+    const int rowsel = id_ / ntile;                                           \
+    const int b = bh / a.nh, h = bh % a.nh;                                   \
+    const int w0 = wt * MT;                                                   \
+    const int nvalid = min(MT, (W_TILED)-w0);
+
+// forward, head dim 32, pscale 1
+template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(const Args a)
+{
+    __shared__ float Ks[MT * MLK];
+    __shared__ float Vs[MT * MLV];
+
+    S2_MFMA_IDS(a.Wo)
+    const int ho = a.gorder[a.row_first + rowsel];
+    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
+    const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
+    const bool mine = j < nvalid;
+    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+
+    // B operand of the score product: Q[query j][channels 16 half .. 16 half + 15], in the log2 domain
+    float qb[16];
+    {
+        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 16 * half;
+#pragma unroll
+        for (int c = 0; c < 16; c += 4) {
+            const float4 x = load4(qrow + c);
+            qb[c] = x.x * LOG2E, qb[c + 1] = x.y * LOG2E, qb[c + 2] = x.z * LOG2E, qb[c + 3] = x.w * LOG2E;
+        }
+    }
+    f16v acc;
+#pragma unroll
+    for (int v = 0; v < 16; v++) acc[v] = 0.f;
+    float m = NEG_BIG, S = 0.f;
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int u0 = 0;
+    Run run = {0, 0, 0, 0};
+    Tile32<T> kt, vt;
+    auto fetch = [&](const Run &rn, int u) {
+        const int c0 = (rn.ws + w0 + u) % a.Wi;
+        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane);
+        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+        kt.template commit<MLK>(Ks, lane);
+        vt.template commit<MLV>(Vs, lane);
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const float w = a.quad_w[run.lat];
+        const int len = run.len;
+        int nri = ri, nu0 = u0 + MT;
+        Run nrun = run;
+        if (nu0 >= len + MT - 1) {
+            nri++;
+            nu0 = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, nu0);
+
+        // S^T = K Q^T
+        f16v sc;
+#pragma unroll
+        for (int v = 0; v < 16; v++) sc[v] = 0.f;
+        {
+            const float *kr = Ks + j * MLK + 16 * half;
+#pragma unroll
+            for (int c = 0; c < 16; c += 4) {
+                const float4 x = *reinterpret_cast<const float4 *>(kr + c);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[c + 0], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[c + 1], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[c + 2], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[c + 3], sc, 0, 0, 0);
+            }
+        }
+        // band mask on the first and last tiles of a run: key position u = u0 + kappa is a neighbor of query j iff 0 <= u - j < len
+        const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
+        if (edge) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int t = u0 + kappa(v, half) - j;
+                sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
+            }
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mn = fmaxf(m, mx);
+        const float corr = fast_exp2(m - mn);
+        m = mn;
+        float rs = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            float p = fast_exp2(sc[v] - mn) * w;
+            if (edge) p = (sc[v] == NEG_BIG) ? 0.f : p;
+            sc[v] = p;
+            rs += p;
+        }
+        rs += __shfl_xor(rs, 32);
+        S = S * corr + rs;
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc[v] *= corr;
+
+        // Y^T += V^T P^T
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float x = Vs[kappa(v, half) * MLV + j];
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], acc, 0, 0, 0);
+        }
+
+        __syncthreads();
+        if (more) {
+            kt.template commit<MLK>(Ks, lane);
+            vt.template commit<MLV>(Vs, lane);
+        }
+        __syncthreads();
+        ri = nri;
+        u0 = nu0;
+        run = nrun;
+    }
+
+    if (mine) {
+        const float inv = 1.0f / S;
+        T *y = static_cast<T *>(a.y) + pt * ldv + (size_t)h * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; g++) store4(y + 8 * g, make_float4(acc[4 * g] * inv, acc[4 * g + 1] * inv, acc[4 * g + 2] * inv, acc[4 * g + 3] * inv));
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
 // ---------------------------------------------------------------------------------
@@ -1071,9 +1260,11 @@ bool aligned(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) %
 
 enum Which { FWD, DQ, DKDV };
 
-template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a0, hipStream_t stream)
+template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a0, int row_first, int row_count, hipStream_t stream)
 {
     Args a = a0;
+    a.row_first = row_first;
+    if (row_count <= 0) return S2ATTN_OK;
     const int BH = a.B * a.nh;
     constexpr int LS = P + 4;
     void (*kern)(const Args) = nullptr;
@@ -1085,15 +1276,15 @@ template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a
     if (fast) a.tile_rows = FAST_ROWS;
     if (which == FWD) {
         kern = fast ? fwd_fast_kernel<T, P> : fwd_kernel<T, P, VEC>;
-        nblocks = (long)a.Ho * ((a.Wo + TQ - 1) / TQ) * BH;
+        nblocks = (long)row_count * ((a.Wo + TQ - 1) / TQ) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
     } else if (which == DQ) {
         kern = fast ? dq_fast_kernel<T, P> : dq_kernel<T, P, VEC>;
-        nblocks = (long)a.Ho * ((a.Wo + TQ - 1) / TQ) * BH;
+        nblocks = (long)row_count * ((a.Wo + TQ - 1) / TQ) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
     } else {
         kern = fast ? dkdv_fast_kernel<T, P> : dkdv_kernel<T, P, VEC>;
-        nblocks = (long)a.Hi * ((a.Wi + TQ - 1) / TQ) * BH;
+        nblocks = (long)row_count * ((a.Wi + TQ - 1) / TQ) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
     }
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
@@ -1108,25 +1299,58 @@ template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a
     return S2ATTN_OK;
 }
 
-template <typename T, bool VEC> int launch_p(Which which, const Args &a, hipStream_t stream)
+template <typename T, bool VEC> int launch_p(Which which, const Args &a, int row_first, int row_count, hipStream_t stream)
 {
     const int d = a.dk_ > a.dv_ ? a.dk_ : a.dv_;
-    if (d <= 4) return launch_one<T, 4, VEC>(which, a, stream);
-    if (d <= 8) return launch_one<T, 8, VEC>(which, a, stream);
-    if (d <= 16) return launch_one<T, 16, VEC>(which, a, stream);
-    return launch_one<T, 32, VEC>(which, a, stream);
+    if (d <= 4) return launch_one<T, 4, VEC>(which, a, row_first, row_count, stream);
+    if (d <= 8) return launch_one<T, 8, VEC>(which, a, row_first, row_count, stream);
+    if (d <= 16) return launch_one<T, 16, VEC>(which, a, row_first, row_count, stream);
+    return launch_one<T, 32, VEC>(which, a, row_first, row_count, stream);
 }
 
-template <typename T> int launch_t(Which which, const Args &a, bool vec, hipStream_t stream)
+// dense kernels: head dims 32, pscale 1, vector-aligned rows, nlon >= 32
+template <typename T> int launch_dense(Which which, const Args &a0, int row_count, hipStream_t stream)
 {
-    return vec ? launch_p<T, true>(which, a, stream) : launch_p<T, false>(which, a, stream);
+    if (row_count <= 0) return S2ATTN_OK;
+    Args a = a0;
+    a.row_first = 0;
+    void (*kern)(const Args) = nullptr;
+    long nblocks = 0;
+    if (which == FWD) {
+        kern = fwd_mfma_kernel<T>;
+        nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
+    } else {
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "no dense kernel for this pass");
+    }
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
 }
 
-int launch(Which which, const Args &a, int dtype, bool vec, hipStream_t stream)
+bool dense_ok(Which which, const Args &a, bool vec)
 {
-    if (dtype == S2ATTN_F32) return launch_t<float>(which, a, vec, stream);
-    if (dtype == S2ATTN_BF16) return launch_t<bf16_t>(which, a, vec, stream);
-    return launch_t<f16_t>(which, a, vec, stream);
+    return which == FWD && vec && a.pscale == 1 && a.dk_ == 32 && a.dv_ == 32 && a.Wi >= 64;
+}
+
+template <typename T> int launch_t(Which which, const Args &a, bool vec, int ndense, hipStream_t stream)
+{
+    const int nrows = which == DKDV ? a.Hi : a.Ho;
+    int first = 0;
+    if (ndense > 0 && dense_ok(which, a, vec)) {
+        const int rc = launch_dense<T>(which, a, ndense, stream);
+        if (rc != S2ATTN_OK) return rc;
+        first = ndense;
+    }
+    return vec ? launch_p<T, true>(which, a, first, nrows - first, stream) : launch_p<T, false>(which, a, first, nrows - first, stream);
+}
+
+int launch(Which which, const Args &a, int dtype, bool vec, int ndense, hipStream_t stream)
+{
+    if (dtype == S2ATTN_F32) return launch_t<float>(which, a, vec, ndense, stream);
+    if (dtype == S2ATTN_BF16) return launch_t<bf16_t>(which, a, vec, ndense, stream);
+    return launch_t<f16_t>(which, a, vec, ndense, stream);
 }
 
 void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const float *quad_w)
@@ -1165,7 +1389,7 @@ extern "C" int s2attn_forward(const void *k, const void *v, const void *q, const
     a.tile_rows = a.pscale * (TQ - 1) + TL;
     const size_t al = 4 * (size_t)esize(shape->dtype);
     const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(y, al);
-    return launch(FWD, a, shape->dtype, vec, static_cast<hipStream_t>(stream));
+    return launch(FWD, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape)
@@ -1206,7 +1430,7 @@ extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, c
     a.dq = dq;
     vec = vec && aligned(dq, 4 * (size_t)esize(shape->dtype));
     a.tile_rows = a.pscale * (TQ - 1) + TL;
-    return launch(DQ, a, shape->dtype, vec, static_cast<hipStream_t>(stream));
+    return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
@@ -1223,7 +1447,7 @@ extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q,
     vec = vec && aligned(dk, al) && aligned(dv, al);
     a.tile_rows = (TQ - 1) / a.pscale + 1 + TL;
     if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile also stages the lane-owned k/v and dk/dv rows
-    return launch(DKDV, a, shape->dtype, vec, static_cast<hipStream_t>(stream));
+    return launch(DKDV, a, shape->dtype, vec, plan->scatter_ndense, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,

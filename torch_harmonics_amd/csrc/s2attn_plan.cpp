@@ -86,11 +86,41 @@ extern "C" int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_
     return rc == S2ATTN_OK ? n : (int64_t)rc;
 }
 
+namespace {
+
+// Cost model (SIMD cycles per 32 grid points) deciding which kernel family a latitude goes to.  The matrix-core
+// kernels pay per 32 x 32 tile whether or not the band fills it; the vector kernels pay per neighbor plus a fixed
+// amount per chunk of 8.  Constants fitted to measured kernel times on MI355X.
+struct RowCost {
+    int64_t dense = 0, vector = 0;
+    void add(int len)
+    {
+        dense += (int64_t)((len + 31 + 31) / 32) * 2750;
+        vector += (int64_t)len * 170 + (int64_t)((len + 7) / 8) * 300;
+    }
+};
+
+// order: dense latitudes first (most work first), then the others (most work first); returns the dense count
+int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order)
+{
+    const int n = (int)cost.size();
+    std::vector<int32_t> dense, vec;
+    for (int i = 0; i < n; i++) (cost[i].dense < cost[i].vector ? dense : vec).push_back(i);
+    std::stable_sort(dense.begin(), dense.end(), [&](int32_t a, int32_t b) { return cost[a].dense > cost[b].dense; });
+    std::stable_sort(vec.begin(), vec.end(), [&](int32_t a, int32_t b) { return cost[a].vector > cost[b].vector; });
+    std::copy(dense.begin(), dense.end(), order);
+    std::copy(vec.begin(), vec.end(), order + dense.size());
+    return (int32_t)dense.size();
+}
+
+} // namespace
+
 extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
                                  int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
-                                 int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order)
+                                 int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order,
+                                 int32_t *ndense)
 {
-    if (!gather_off || !gather_order || !scatter_off || !scatter_order || (nruns > 0 && (!gather_runs || !scatter_runs)))
+    if (!gather_off || !gather_order || !scatter_off || !scatter_order || !ndense || (nruns > 0 && (!gather_runs || !scatter_runs)))
         return s2attn_fail(S2ATTN_E_INVALID, "plan output array is null");
 
     std::vector<HostRun> runs;
@@ -102,7 +132,7 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
     const int pscale = nlon_in / nlon_out;
 
     // gather side: runs are already grouped by ho, in CSR order
-    std::vector<int64_t> gwork(nlat_out, 0);
+    std::vector<RowCost> gcost(nlat_out), scost(nlat_in);
     std::fill(gather_off, gather_off + nlat_out + 1, 0);
     for (int64_t i = 0; i < n; i++) {
         const HostRun &r = runs[i];
@@ -111,12 +141,11 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
         gather_runs[4 * i + 2] = r.len;
         gather_runs[4 * i + 3] = 0;
         gather_off[r.ho + 1]++;
-        gwork[r.ho] += r.len;
+        gcost[r.ho].add(r.len);
     }
     for (int ho = 0; ho < nlat_out; ho++) gather_off[ho + 1] += gather_off[ho];
 
     // scatter side: stable counting sort by hi keeps ho ascending inside a group
-    std::vector<int64_t> swork(nlat_in, 0);
     std::fill(scatter_off, scatter_off + nlat_in + 1, 0);
     for (int64_t i = 0; i < n; i++) scatter_off[runs[i].hi + 1]++;
     for (int hi = 0; hi < nlat_in; hi++) scatter_off[hi + 1] += scatter_off[hi];
@@ -128,13 +157,10 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
         scatter_runs[4 * s + 1] = r.ws;
         scatter_runs[4 * s + 2] = r.len;
         scatter_runs[4 * s + 3] = 0;
-        swork[r.hi] += (r.len + pscale - 1) / pscale;
+        scost[r.hi].add((r.len + pscale - 1) / pscale);
     }
 
-    // longest group first (stable, so equal groups keep latitude order)
-    std::iota(gather_order, gather_order + nlat_out, 0);
-    std::stable_sort(gather_order, gather_order + nlat_out, [&](int32_t a, int32_t b) { return gwork[a] > gwork[b]; });
-    std::iota(scatter_order, scatter_order + nlat_in, 0);
-    std::stable_sort(scatter_order, scatter_order + nlat_in, [&](int32_t a, int32_t b) { return swork[a] > swork[b]; });
+    ndense[0] = order_rows(gcost, gather_order);
+    ndense[1] = order_rows(scost, scatter_order);
     return S2ATTN_OK;
 }

@@ -25,9 +25,10 @@ _lock = threading.Lock()
 class Plan:
     """Six int32 arrays on one device plus the ctypes view the library takes."""
 
-    def __init__(self, arrays, nruns, keepalive):
+    def __init__(self, arrays, nruns, ndense, keepalive):
         self.gather_off, self.gather_runs, self.gather_order, self.scatter_off, self.scatter_runs, self.scatter_order = arrays
         self.nruns = nruns
+        self.gather_ndense, self.scatter_ndense = ndense
         self._keepalive = keepalive
         self.struct = _lib.PlanStruct(
             self.gather_off.data_ptr(),
@@ -37,14 +38,17 @@ class Plan:
             self.scatter_runs.data_ptr(),
             self.scatter_order.data_ptr(),
             nruns,
+            self.gather_ndense,
+            self.scatter_ndense,
         )
 
 
 def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int):
     """
     Runs the library's host builder on CPU copies of the CSR.  Returns
-    ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns)
-    as CPU int32 tensors; gather_runs / scatter_runs have shape (nruns, 4) = (lat, ws, len, 0).
+    ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns, (gather_ndense, scatter_ndense))
+    as CPU int32 tensors; gather_runs / scatter_runs have shape (nruns, 4) = (lat, ws, len, 0); the first *_ndense entries
+    of each order are the latitudes the dense matrix-core kernels take.
     """
     lib = _lib.load()
     ci = col_idx.detach().to(device="cpu", dtype=torch.int64).contiguous()
@@ -62,9 +66,10 @@ def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, 
         torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
         torch.zeros(nlat_in, dtype=torch.int32),
     ]
-    rc = lib.s2attn_plan_build(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays])
+    ndense = torch.zeros(2, dtype=torch.int32)
+    rc = lib.s2attn_plan_build(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays], ndense.data_ptr())
     _lib.check(rc, "s2attn_plan_build")
-    return arrays, int(nruns)
+    return arrays, int(nruns), (int(ndense[0]), int(ndense[1]))
 
 
 def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int) -> Plan:
@@ -87,9 +92,9 @@ def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in
         if plan is not None:
             _cache.move_to_end(key)
             return plan
-    arrays, nruns = build_host_plan(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    arrays, nruns, ndense = build_host_plan(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
     dev = col_idx.device
-    plan = Plan([a.to(dev) for a in arrays], nruns, (col_idx, row_off))
+    plan = Plan([a.to(dev) for a in arrays], nruns, ndense, (col_idx, row_off))
     with _lock:
         _cache[key] = plan
         while len(_cache) > _MAX_ENTRIES:
