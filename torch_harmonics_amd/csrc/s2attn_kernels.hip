@@ -1209,6 +1209,313 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     }
 }
 
+
+// backward dq + statistics, dense: same column ownership as the forward.  Per tile four matrix products:
+//   S^T = K Q^T,  G^T = V dY^T,  A_k^T += K^T P^T,  A_kg^T += K^T (P o G)^T   (A operands of the last two are
+//   column reads of the K tile, B operands the probability registers), online softmax across tiles.
+template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const Args a)
+{
+    __shared__ float Ks[MT * MLK];
+    __shared__ float Vs[MT * MLK];
+
+    S2_MFMA_IDS(a.Wo)
+    const int ho = a.gorder[a.row_first + rowsel];
+    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
+    const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
+    const bool mine = j < nvalid;
+    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+
+    float qb[16], gb[16];
+    {
+        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 16 * half;
+        const T *grow = static_cast<const T *>(a.dy) + pt * ldv + (size_t)h * 32 + 16 * half;
+#pragma unroll
+        for (int c = 0; c < 16; c += 4) {
+            const float4 x = load4(qrow + c);
+            const float4 z = load4(grow + c);
+            qb[c] = x.x * LOG2E, qb[c + 1] = x.y * LOG2E, qb[c + 2] = x.z * LOG2E, qb[c + 3] = x.w * LOG2E;
+            gb[c] = z.x, gb[c + 1] = z.y, gb[c + 2] = z.z, gb[c + 3] = z.w;
+        }
+    }
+    f16v Ak, Akg;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        Ak[v] = 0.f;
+        Akg[v] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f, Ag = 0.f;
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int u0 = 0;
+    Run run = {0, 0, 0, 0};
+    Tile32<T> kt, vt;
+    auto fetch = [&](const Run &rn, int u) {
+        const int c0 = (rn.ws + w0 + u) % a.Wi;
+        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane);
+        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+        kt.template commit<MLK>(Ks, lane);
+        vt.template commit<MLK>(Vs, lane);
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const float w = a.quad_w[run.lat];
+        const int len = run.len;
+        int nri = ri, nu0 = u0 + MT;
+        Run nrun = run;
+        if (nu0 >= len + MT - 1) {
+            nri++;
+            nu0 = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, nu0);
+
+        f16v sc, gc;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            sc[v] = 0.f;
+            gc[v] = 0.f;
+        }
+        {
+            const float *kr = Ks + j * MLK + 16 * half;
+            const float *vr = Vs + j * MLK + 16 * half;
+#pragma unroll
+            for (int c = 0; c < 16; c += 4) {
+                const float4 x = *reinterpret_cast<const float4 *>(kr + c);
+                const float4 z = *reinterpret_cast<const float4 *>(vr + c);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[c + 0], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, gb[c + 0], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[c + 1], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, gb[c + 1], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[c + 2], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, gb[c + 2], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[c + 3], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, gb[c + 3], gc, 0, 0, 0);
+            }
+        }
+        const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
+        if (edge) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const int t = u0 + kappa(v, half) - j;
+                sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
+            }
+        }
+        float mx = sc[0];
+#pragma unroll
+        for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const float mn = fmaxf(m, mx);
+        const float corr = fast_exp2(m - mn);
+        m = mn;
+        float rs = 0.f, rg = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            float p = fast_exp2(sc[v] - mn) * w;
+            if (edge) p = (sc[v] == NEG_BIG) ? 0.f : p;
+            const float pg = p * gc[v];
+            sc[v] = p;
+            gc[v] = pg;
+            rs += p;
+            rg += pg;
+        }
+        rs += __shfl_xor(rs, 32);
+        rg += __shfl_xor(rg, 32);
+        S = S * corr + rs;
+        Ag = Ag * corr + rg;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            Ak[v] *= corr;
+            Akg[v] *= corr;
+        }
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float x = Ks[kappa(v, half) * MLK + j];
+            Ak = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], Ak, 0, 0, 0);
+            Akg = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], Akg, 0, 0, 0);
+        }
+
+        __syncthreads();
+        if (more) {
+            kt.template commit<MLK>(Ks, lane);
+            vt.template commit<MLK>(Vs, lane);
+        }
+        __syncthreads();
+        ri = nri;
+        u0 = nu0;
+        run = nrun;
+    }
+
+    if (mine) {
+        const float inv = 1.0f / S;
+        const float I = Ag * inv;
+        if (half == 0) a.stats[((size_t)bh * a.Ho + ho) * a.Wo + w0 + j] = make_float2(m + fast_log2(S), I);
+        T *dq = static_cast<T *>(a.dq) + pt * ldk + (size_t)h * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; g++)
+            store4(dq + 8 * g, make_float4((Akg[4 * g] - I * Ak[4 * g]) * inv, (Akg[4 * g + 1] - I * Ak[4 * g + 1]) * inv,
+                                           (Akg[4 * g + 2] - I * Ak[4 * g + 2]) * inv, (Akg[4 * g + 3] - I * Ak[4 * g + 3]) * inv));
+    }
+}
+
+// backward dk/dv, dense: lane owns INPUT longitude j of the tile.  For a run (ho, ws, len) the queries that see the
+// tile's keys are the len + 31 longitudes starting at w0 - ws - len + 1; query row r sees key j iff 0 <= r - j < len.
+// Per tile of 32 query rows:  S = Q K^T and G = dY V^T come out as [query][key] (a lane holds 16 queries of ITS key
+// column), P = exp2(S - lse_query) w, C = P (G - I_query), then dK^T += Q^T C and dV^T += dY^T P.
+template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(const Args a)
+{
+    __shared__ float Qs[MT * MLK];
+    __shared__ float Gs[MT * MLK];
+    __shared__ float Ls[MT];
+    __shared__ float Is[MT];
+
+    S2_MFMA_IDS(a.Wi)
+    const int hi = a.sorder[a.row_first + rowsel];
+    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldk + (size_t)h * 32;
+    const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * 32;
+    const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
+    const bool mine = j < nvalid;
+    const size_t pt = (size_t)(b * a.Hi + hi) * a.Wi + w0 + (mine ? j : 0);
+
+    float kb[16], vb[16];
+    {
+        const T *krow = static_cast<const T *>(a.k) + pt * ldk + (size_t)h * 32 + 16 * half;
+        const T *vrow = static_cast<const T *>(a.v) + pt * ldv + (size_t)h * 32 + 16 * half;
+#pragma unroll
+        for (int c = 0; c < 16; c += 4) {
+            const float4 x = load4(krow + c);
+            const float4 z = load4(vrow + c);
+            kb[c] = x.x * LOG2E, kb[c + 1] = x.y * LOG2E, kb[c + 2] = x.z * LOG2E, kb[c + 3] = x.w * LOG2E;
+            vb[c] = z.x, vb[c + 1] = z.y, vb[c + 2] = z.z, vb[c + 3] = z.w;
+        }
+    }
+    f16v dkt, dvt;
+#pragma unroll
+    for (int v = 0; v < 16; v++) {
+        dkt[v] = 0.f;
+        dvt[v] = 0.f;
+    }
+    const float w = a.quad_w[hi];
+
+    int ri = a.soff[hi];
+    const int rend = a.soff[hi + 1];
+    int r0 = 0;
+    Run run = {0, 0, 0, 0};
+    Tile32<T> qt, gt;
+    float2 st = make_float2(0.f, 0.f);
+    auto fetch = [&](const Run &rn, int r) {
+        int c0 = (w0 - rn.ws - rn.len + 1 + r) % a.Wo;
+        c0 += (c0 < 0) ? a.Wo : 0;
+        qt.fetch(qy + (size_t)rn.lat * a.Wo * ldk, ldk, c0, a.Wo, lane);
+        gt.fetch(gy + (size_t)rn.lat * a.Wo * ldv, ldv, c0, a.Wo, lane);
+        int col = c0 + j;
+        col -= (col >= a.Wo) ? a.Wo : 0;
+        st = stats[(size_t)rn.lat * a.Wo + col];
+    };
+    auto commit = [&]() {
+        qt.template commit<MLK>(Qs, lane);
+        gt.template commit<MLK>(Gs, lane);
+        if (half == 0) {
+            Ls[j] = st.x;
+            Is[j] = st.y;
+        }
+    };
+    if (ri < rend) {
+        run = a.sruns[ri];
+        fetch(run, 0);
+        commit();
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const int len = run.len;
+        int nri = ri, nr0 = r0 + MT;
+        Run nrun = run;
+        if (nr0 >= len + MT - 1) {
+            nri++;
+            nr0 = 0;
+            if (nri < rend) nrun = a.sruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, nr0);
+
+        f16v sc, gc;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            sc[v] = 0.f;
+            gc[v] = 0.f;
+        }
+        {
+            const float *qr = Qs + j * MLK + 16 * half;
+            const float *gr = Gs + j * MLK + 16 * half;
+#pragma unroll
+            for (int c = 0; c < 16; c += 4) {
+                const float4 x = *reinterpret_cast<const float4 *>(qr + c);
+                const float4 z = *reinterpret_cast<const float4 *>(gr + c);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, kb[c + 0], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, vb[c + 0], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, kb[c + 1], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, vb[c + 1], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, kb[c + 2], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, vb[c + 2], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, kb[c + 3], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, vb[c + 3], gc, 0, 0, 0);
+            }
+        }
+        const bool edge = (r0 < MT - 1) || (r0 + MT - 1 >= len);
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 8 * g + 4 * half);
+            const float4 i4 = *reinterpret_cast<const float4 *>(Is + 8 * g + 4 * half);
+            const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+            const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const int v = 4 * g + e;
+                float p = fast_exp2(sc[v] - lv[e]) * w;
+                if (edge) {
+                    const int t = r0 + kappa(v, half) - j;
+                    p = (t >= 0 && t < len) ? p : 0.f;
+                }
+                sc[v] = p;
+                gc[v] = p * (gc[v] - iv[e]);
+            }
+        }
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float x = Qs[kappa(v, half) * MLK + j];
+            const float z = Gs[kappa(v, half) * MLK + j];
+            dkt = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], dkt, 0, 0, 0);
+            dvt = __builtin_amdgcn_mfma_f32_32x32x2f32(z, sc[v], dvt, 0, 0, 0);
+        }
+
+        __syncthreads();
+        if (more) commit();
+        __syncthreads();
+        ri = nri;
+        r0 = nr0;
+        run = nrun;
+    }
+
+    if (mine) {
+        T *dk = static_cast<T *>(a.dk) + pt * ldk + (size_t)h * 32 + 4 * half;
+        T *dv = static_cast<T *>(a.dv) + pt * ldv + (size_t)h * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            store4(dk + 8 * g, make_float4(dkt[4 * g], dkt[4 * g + 1], dkt[4 * g + 2], dkt[4 * g + 3]));
+            store4(dv + 8 * g, make_float4(dvt[4 * g], dvt[4 * g + 1], dvt[4 * g + 2], dvt[4 * g + 3]));
+        }
+    }
+}
+
 // ---------------------------------------------------------------------------------
 // layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
 // ---------------------------------------------------------------------------------
@@ -1319,8 +1626,12 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
     if (which == FWD) {
         kern = fwd_mfma_kernel<T>;
         nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
+    } else if (which == DQ) {
+        kern = dq_mfma_kernel<T>;
+        nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
     } else {
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "no dense kernel for this pass");
+        kern = dkdv_mfma_kernel<T>;
+        nblocks = (long)row_count * ((a.Wi + MT - 1) / MT) * a.B * a.nh;
     }
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
@@ -1331,7 +1642,8 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
 
 bool dense_ok(Which which, const Args &a, bool vec)
 {
-    return which == FWD && vec && a.pscale == 1 && a.dk_ == 32 && a.dv_ == 32 && a.Wi >= 64;
+    (void)which;
+    return vec && a.pscale == 1 && a.dk_ == 32 && a.dv_ == 32 && a.Wi >= 64;
 }
 
 template <typename T> int launch_t(Which which, const Args &a, bool vec, int ndense, hipStream_t stream)
