@@ -1039,11 +1039,43 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
 typedef float f16v __attribute__((ext_vector_type(16)));
 constexpr int MT = 32;        // queries and keys per tile
 constexpr int MLK = 36;       // LDS row stride of the K-side tile (128-bit reads, rows 16 B-group skewed)
-constexpr int MLV = 40;       // LDS row stride of the V-side tile (32-bit reads by channel; the two halves read rows 4 apart)
 
 __device__ inline int kappa(int v, int half) { return 8 * (v / 4) + 4 * half + (v % 4); }
 
-// fetch one 32-row tile (rows c0.., wrapping once at W) of a latitude/head into registers: 4 loads of 16 B per lane
+// Staging unit of the dense kernels: up to 40 consecutive longitudes (rows c0.., wrapping once at W) of one
+// latitude/head, fetched into registers with one 16-byte load per lane per 8 rows.  Matrix-core tiles use the first
+// 32 rows; the vector path for short runs uses all 40 (32 columns + up to 9 neighbors - 1).
+constexpr int MR = 40;  // rows of the LDS tile
+constexpr int VC = 9;   // neighbors per vector-path chunk (MT - 1 + VC <= MR)
+constexpr int LMIN = 20; // runs at least this long go through the matrix cores
+
+template <typename T> struct Tile40 {
+    typedef typename Vec4<T>::type raw_t;
+    raw_t raw[5];
+    __device__ inline void fetch(const T *src, unsigned ld, int c0, int W, int lane, bool fifth)
+    {
+        const int colA = c0 + (lane >> 3), cb = 4 * (lane & 7);
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            int col = colA + it * 8;
+            col -= (col >= W) ? W : 0;
+            raw[it] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
+        }
+        if (fifth) {
+            int col = colA + 32;
+            col -= (col >= W) ? W : 0;
+            raw[4] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
+        }
+    }
+    __device__ inline void commit(float *dst, int lane, bool fifth) const
+    {
+        const int r0 = lane >> 3, cb = 4 * (lane & 7);
+#pragma unroll
+        for (int it = 0; it < 4; it++) *reinterpret_cast<float4 *>(dst + (r0 + it * 8) * MLK + cb) = widen4(raw[it], (const T *)nullptr);
+        if (fifth) *reinterpret_cast<float4 *>(dst + (r0 + 32) * MLK + cb) = widen4(raw[4], (const T *)nullptr);
+    }
+};
+
 template <typename T> struct Tile32 {
     typedef typename Vec4<T>::type raw_t;
     raw_t raw[4];
@@ -1065,6 +1097,12 @@ template <typename T> struct Tile32 {
     }
 };
 
+// A run is walked either in matrix-core tiles of 32 band positions (pos = first position, len + 31 positions in all)
+// or, when short, in vector chunks of VC neighbors (pos = first neighbor index).
+__device__ inline bool run_is_dense(int len) { return len >= LMIN; }
+__device__ inline bool run_done(int len, int next_pos) { return run_is_dense(len) ? next_pos >= len + MT - 1 : next_pos >= len; }
+__device__ inline int run_stride(int len) { return run_is_dense(len) ? MT : VC; }
+
 #define S2_MFMA_IDS(W_TILED)                                                  \
     const int lane = threadIdx.x;                                             \
     const int j = lane & 31, half = lane >> 5;                                \
@@ -1079,11 +1117,13 @@ template <typename T> struct Tile32 {
     const int w0 = wt * MT;                                                   \
     const int nvalid = min(MT, (W_TILED)-w0);
 
-// forward, head dim 32, pscale 1
+// forward, head dim 32, pscale 1.  Lane (j, half) keeps channels 8g + 4 half + e (g, e < 4) of query j: that is the
+// accumulator layout of the matrix-core product, and the vector path for short runs uses the same one (each half
+// computes half of a dot product, one cross-half exchange completes it).
 template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(const Args a)
 {
-    __shared__ float Ks[MT * MLK];
-    __shared__ float Vs[MT * MLV];
+    __shared__ float Ks[MR * MLK];
+    __shared__ float Vs[MR * MLK];
 
     S2_MFMA_IDS(a.Wo)
     const int ho = a.gorder[a.row_first + rowsel];
@@ -1093,14 +1133,13 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     const bool mine = j < nvalid;
     const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
 
-    // B operand of the score product: Q[query j][channels 16 half .. 16 half + 15], in the log2 domain
     float qb[16];
     {
-        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 16 * half;
+        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 4 * half;
 #pragma unroll
-        for (int c = 0; c < 16; c += 4) {
-            const float4 x = load4(qrow + c);
-            qb[c] = x.x * LOG2E, qb[c + 1] = x.y * LOG2E, qb[c + 2] = x.z * LOG2E, qb[c + 3] = x.w * LOG2E;
+        for (int g = 0; g < 4; g++) {
+            const float4 x = load4(qrow + 8 * g);
+            qb[4 * g] = x.x * LOG2E, qb[4 * g + 1] = x.y * LOG2E, qb[4 * g + 2] = x.z * LOG2E, qb[4 * g + 3] = x.w * LOG2E;
         }
     }
     f16v acc;
@@ -1110,94 +1149,152 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
 
     int ri = a.goff[ho];
     const int rend = a.goff[ho + 1];
-    int u0 = 0;
+    int pos = 0;
     Run run = {0, 0, 0, 0};
-    Tile32<T> kt, vt;
-    auto fetch = [&](const Run &rn, int u) {
-        const int c0 = (rn.ws + w0 + u) % a.Wi;
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane);
+    Tile40<T> kt, vt;
+    auto fetch = [&](const Run &rn, int p) {
+        const int c0 = (rn.ws + w0 + p) % a.Wi;
+        const bool fifth = !run_is_dense(rn.len);
+        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane, fifth);
+        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane, fifth);
     };
     if (ri < rend) {
         run = a.gruns[ri];
         fetch(run, 0);
-        kt.template commit<MLK>(Ks, lane);
-        vt.template commit<MLV>(Vs, lane);
+        kt.commit(Ks, lane, !run_is_dense(run.len));
+        vt.commit(Vs, lane, !run_is_dense(run.len));
     }
     __syncthreads();
 
     while (ri < rend) {
         const float w = a.quad_w[run.lat];
         const int len = run.len;
-        int nri = ri, nu0 = u0 + MT;
+        int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
-        if (nu0 >= len + MT - 1) {
+        if (run_done(len, npos)) {
             nri++;
-            nu0 = 0;
+            npos = 0;
             if (nri < rend) nrun = a.gruns[nri];
         }
         const bool more = nri < rend;
-        if (more) fetch(nrun, nu0);
+        if (more) fetch(nrun, npos);
 
-        // S^T = K Q^T
-        f16v sc;
+        const float *kq = Ks + j * MLK + 4 * half; // row j, this half's channel groups at +8g
+        const float *vq = Vs + j * MLK + 4 * half;
+        if (run_is_dense(len)) {
+            // ---- matrix-core tile: S^T = K Q^T ----
+            const int u0 = pos;
+            f16v sc;
 #pragma unroll
-        for (int v = 0; v < 16; v++) sc[v] = 0.f;
-        {
-            const float *kr = Ks + j * MLK + 16 * half;
+            for (int v = 0; v < 16; v++) sc[v] = 0.f;
 #pragma unroll
-            for (int c = 0; c < 16; c += 4) {
-                const float4 x = *reinterpret_cast<const float4 *>(kr + c);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[c + 0], sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[c + 1], sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[c + 2], sc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[c + 3], sc, 0, 0, 0);
+            for (int g = 0; g < 4; g++) {
+                const float4 x = *reinterpret_cast<const float4 *>(kq + 8 * g);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[4 * g + 0], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[4 * g + 1], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[4 * g + 2], sc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[4 * g + 3], sc, 0, 0, 0);
             }
-        }
-        // band mask on the first and last tiles of a run: key position u = u0 + kappa is a neighbor of query j iff 0 <= u - j < len
-        const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
-        if (edge) {
+            // band mask on the first and last tiles: key position u = u0 + kappa is a neighbor of query j iff 0 <= u - j < len
+            const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
+            if (edge) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int t = u0 + kappa(v, half) - j;
+                    sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
+                }
+            }
+            float mx = sc[0];
+#pragma unroll
+            for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float mn = fmaxf(m, mx);
+            if (__any(mn > m)) {
+                const float corr = fast_exp2(m - mn);
+                S *= corr;
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[v] *= corr;
+            }
+            m = mn;
+            float rs = 0.f;
+            if (edge) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float p = (sc[v] == NEG_BIG) ? 0.f : fast_exp2(sc[v] - mn) * w;
+                    sc[v] = p;
+                    rs += p;
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const float p = fast_exp2(sc[v] - mn) * w;
+                    sc[v] = p;
+                    rs += p;
+                }
+            }
+            rs += __shfl_xor(rs, 32);
+            S += rs;
+            // Y^T += V^T P^T
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int t = u0 + kappa(v, half) - j;
-                sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
+                const float x = Vs[kappa(v, half) * MLK + j];
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], acc, 0, 0, 0);
             }
-        }
-        float mx = sc[0];
+        } else {
+            // ---- vector chunk: neighbors pos .. pos + L - 1, query j reads staged rows j + t ----
+            const int L = min(VC, len - pos);
+            float s[VC];
+            float cm = NEG_BIG;
 #pragma unroll
-        for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float mn = fmaxf(m, mx);
-        const float corr = fast_exp2(m - mn);
-        m = mn;
-        float rs = 0.f;
+            for (int t = 0; t < VC; t++) {
+                s[t] = NEG_BIG;
+                if (t < L) {
+                    float part = 0.f;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            float p = fast_exp2(sc[v] - mn) * w;
-            if (edge) p = (sc[v] == NEG_BIG) ? 0.f : p;
-            sc[v] = p;
-            rs += p;
-        }
-        rs += __shfl_xor(rs, 32);
-        S = S * corr + rs;
+                    for (int g = 0; g < 4; g++) {
+                        const float4 x = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
+                        part = fmaf(qb[4 * g], x.x, part);
+                        part = fmaf(qb[4 * g + 1], x.y, part);
+                        part = fmaf(qb[4 * g + 2], x.z, part);
+                        part = fmaf(qb[4 * g + 3], x.w, part);
+                    }
+                    s[t] = part + __shfl_xor(part, 32);
+                    cm = fmaxf(cm, s[t]);
+                }
+            }
+            const float mn = fmaxf(m, cm);
+            if (__any(mn > m)) {
+                const float corr = fast_exp2(m - mn);
+                S *= corr;
 #pragma unroll
-        for (int v = 0; v < 16; v++) acc[v] *= corr;
-
-        // Y^T += V^T P^T
+                for (int v = 0; v < 16; v++) acc[v] *= corr;
+            }
+            m = mn;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float x = Vs[kappa(v, half) * MLV + j];
-            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], acc, 0, 0, 0);
+            for (int t = 0; t < VC; t++) {
+                if (t < L) {
+                    const float p = fast_exp2(s[t] - mn) * w;
+                    S += p;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float4 x = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
+                        acc[4 * g] = fmaf(p, x.x, acc[4 * g]);
+                        acc[4 * g + 1] = fmaf(p, x.y, acc[4 * g + 1]);
+                        acc[4 * g + 2] = fmaf(p, x.z, acc[4 * g + 2]);
+                        acc[4 * g + 3] = fmaf(p, x.w, acc[4 * g + 3]);
+                    }
+                }
+            }
         }
 
         __syncthreads();
         if (more) {
-            kt.template commit<MLK>(Ks, lane);
-            vt.template commit<MLV>(Vs, lane);
+            kt.commit(Ks, lane, !run_is_dense(nrun.len));
+            vt.commit(Vs, lane, !run_is_dense(nrun.len));
         }
         __syncthreads();
         ri = nri;
-        u0 = nu0;
+        pos = npos;
         run = nrun;
     }
 
@@ -1208,7 +1305,6 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
         for (int g = 0; g < 4; g++) store4(y + 8 * g, make_float4(acc[4 * g] * inv, acc[4 * g + 1] * inv, acc[4 * g + 2] * inv, acc[4 * g + 3] * inv));
     }
 }
-
 
 // backward dq + statistics, dense: same column ownership as the forward.  Per tile four matrix products:
 //   S^T = K Q^T,  G^T = V dY^T,  A_k^T += K^T P^T,  A_kg^T += K^T (P o G)^T   (A operands of the last two are
@@ -1650,10 +1746,12 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
 {
     const int nrows = which == DKDV ? a.Hi : a.Ho;
     int first = 0;
-    if (ndense > 0 && dense_ok(which, a, vec)) {
-        const int rc = launch_dense<T>(which, a, ndense, stream);
+    if (dense_ok(which, a, vec)) {
+        // the forward kernel handles short runs itself (vector path inside), so it takes every latitude
+        const int take = which == FWD ? nrows : ndense;
+        const int rc = launch_dense<T>(which, a, take, stream);
         if (rc != S2ATTN_OK) return rc;
-        first = ndense;
+        first = take;
     }
     return vec ? launch_p<T, true>(which, a, first, nrows - first, stream) : launch_p<T, false>(which, a, first, nrows - first, stream);
 }

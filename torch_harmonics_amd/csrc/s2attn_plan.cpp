@@ -95,8 +95,8 @@ struct RowCost {
     int64_t dense = 0, vector = 0;
     void add(int len)
     {
-        dense += (int64_t)((len + 31 + 31) / 32) * 3850;
-        vector += (int64_t)len * 450 + (int64_t)((len + 7) / 8) * 150;
+        dense += (int64_t)((len + 31 + 31) / 32) * 5200;
+        vector += (int64_t)len * 770;
     }
 };
 
