@@ -69,6 +69,16 @@ SMALL_CASES = [
     (1, 1, 16, 16, (12, 160), (12, 160), "equiangular", "equiangular", 0.3),
     (1, 1, 8, 8, (10, 200), (10, 100), "equiangular", "equiangular", 0.35),
     (2, 1, 4, 4, (6, 12), (6, 12), "equiangular", "equiangular", 7.0),
+    # wide heads: 2 or 4 lanes per grid point
+    (1, 2, 64, 64, (16, 32), (16, 32), "legendre-gauss", "legendre-gauss", 0.4),
+    (1, 1, 48, 40, (12, 24), (6, 12), "equiangular", "equiangular", 0.6),
+    (1, 1, 128, 128, (10, 20), (10, 20), "equiangular", "equiangular", 0.7),
+    (1, 2, 96, 72, (12, 48), (12, 16), "equiangular", "equiangular", 0.5),
+    (1, 1, 33, 65, (8, 16), (8, 16), "equiangular", "equiangular", 0.8),
+    # head dim 32 on grids wide enough for the matrix-core kernels (nlon >= 64), incl. full-circle rows and long runs
+    (1, 2, 32, 32, (24, 96), (24, 96), "equiangular", "equiangular", 0.5),
+    (2, 1, 32, 32, (16, 128), (16, 128), "legendre-gauss", "legendre-gauss", 0.9),
+    (1, 1, 32, 32, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
 ]
 
 
@@ -111,6 +121,21 @@ def test_cfg2_reduced_batch():
     dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, quad, col_idx, row_off, 4)
     for name, got, want in (("dk", dk, dk64), ("dv", dv, dv64), ("dq", dq, dq64)):
         assert_close(name, got, want, **F32_TOL)
+
+
+def test_cfg5_shape_reduced_grid_bf16():
+    """The bf16 configuration's shape at a reduced grid: Legendre-Gauss 46x90 in and out, 2 heads of 64 channels, bf16
+    storage, cutoff 8 latitude spacings (every query sees a few hundred neighbors), inputs N(0,1) scaled 0.5."""
+    ins = outs = (46, 90)
+    col_idx, row_off, quad = _psi(ins, outs, "legendre-gauss", "legendre-gauss", 8 * math.pi / 45)
+    k, v, q, dy = randn_inputs(2, 46, 90, 46, 90, 2, 64, 64, scale=0.5)
+    k, v, q, dy = [t.to(torch.bfloat16).float() for t in (k, v, q, dy)]
+    y, dk, dv, dq = _run_hip(k, v, q, dy, quad, col_idx, row_off, 2, dtype=torch.bfloat16)
+    y64 = oracle.forward_f64(k, v, q, quad, col_idx, row_off, 2)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, quad, col_idx, row_off, 2)
+    for name, got, want in (("y", y, y64), ("dk", dk, dk64), ("dv", dv, dv64), ("dq", dq, dq64)):
+        rms = want.pow(2).mean().sqrt().item()
+        assert_close(name, got, want, rtol=2e-2, atol=2e-2 * rms)
 
 
 @pytest.mark.parametrize("dtype,tol", [(torch.bfloat16, 2e-2), (torch.float16, 2e-2)], ids=["bf16", "fp16"])

@@ -579,6 +579,315 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
     unstage_rows<T, P, VEC>(dv + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, Gs, ldv, a.dv_, wi0, nvalid, lane);
 }
 
+
+// ---------------------------------------------------------------------------------
+// Wide heads (32 < head dim <= 128): same single-wavefront tiling as the generic kernels, but LPQ = 2 or 4
+// adjacent lanes share one grid point and each keeps a 32-channel slice of its vectors, so the register
+// footprint stays that of a 32-channel head; a dot product is completed by LPQ-lane butterfly adds.
+// A wavefront therefore covers 64 / LPQ longitudes.
+// ---------------------------------------------------------------------------------
+template <int LPQ> __device__ inline float slice_sum(float x)
+{
+#pragma unroll
+    for (int o = 1; o < LPQ; o <<= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+#define S2_WIDE_IDS(W_TILED)                                                  \
+    constexpr int TQW = TQ / LPQ;                                             \
+    constexpr int PT = 32 * LPQ;                                              \
+    constexpr int LS = PT + 4;                                                \
+    const int lane = threadIdx.x;                                             \
+    const int qi = lane / LPQ, sl = lane % LPQ;                               \
+    const int BH = a.B * a.nh;                                                \
+    const int ntile = ((W_TILED) + TQW - 1) / TQW;                            \
+    int id_ = blockIdx.x;                                                     \
+    const int bh = id_ % BH;                                                  \
+    id_ /= BH;                                                                \
+    const int wt = id_ % ntile;                                               \
+    const int rowsel = id_ / ntile;                                           \
+    const int b = bh / a.nh, h = bh % a.nh;                                   \
+    const int w0 = wt * TQW;                                                  \
+    const int nvalid = min(TQW, (W_TILED)-w0);                                \
+    const int ps = a.pscale;                                                  \
+    const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
+
+template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void fwd_wide_kernel(const Args a)
+{
+    extern __shared__ float4 smem4[];
+    float *Ks = reinterpret_cast<float *>(smem4);
+    S2_WIDE_IDS(a.Wo)
+    float *Vs = Ks + a.tile_rows * LS;
+    const int ho = a.gorder[a.row_first + rowsel];
+    const T *kx = static_cast<const T *>(a.k);
+    const T *vx = static_cast<const T *>(a.v);
+    const T *qy = static_cast<const T *>(a.q);
+    T *y = static_cast<T *>(a.y);
+
+    stage_rows<T, PT, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, w0, a.Wo, nvalid, lane);
+    __syncthreads();
+    float qr[32], acc[32];
+#pragma unroll
+    for (int c = 0; c < 32; c++) {
+        qr[c] = Ks[qi * LS + sl * 32 + c] * LOG2E;
+        acc[c] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f;
+
+    for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
+        const Run run = a.gruns[ri];
+        const float w = a.quad_w[run.lat];
+        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
+        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        for (int t0 = 0; t0 < run.len; t0 += TL) {
+            const int L = min(TL, run.len - t0);
+            const int c0 = (run.ws + t0 + ps * w0) % a.Wi;
+            const int nrows = ps * (nvalid - 1) + L;
+            __syncthreads();
+            stage_rows<T, PT, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            __syncthreads();
+            const float *krow = Ks + (ps * qi) * LS + sl * 32;
+            const float *vrow = Vs + (ps * qi) * LS + sl * 32;
+            float s[TL];
+            float cm = NEG_BIG;
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                s[t] = NEG_BIG;
+                if (t < L) {
+                    s[t] = slice_sum<LPQ>(dot_row<32>(qr, krow + t * LS));
+                    cm = fmaxf(cm, s[t]);
+                }
+            }
+            const float mn = fmaxf(m, cm);
+            const float corr = fast_exp2(m - mn);
+            m = mn;
+            S *= corr;
+#pragma unroll
+            for (int c = 0; c < 32; c++) acc[c] *= corr;
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                if (t < L) {
+                    const float p = fast_exp2(s[t] - mn) * w;
+                    S += p;
+                    const float *vr = vrow + t * LS;
+#pragma unroll
+                    for (int c = 0; c < 32; c += 4) {
+                        const float4 x = *reinterpret_cast<const float4 *>(vr + c);
+                        acc[c + 0] = fmaf(p, x.x, acc[c + 0]);
+                        acc[c + 1] = fmaf(p, x.y, acc[c + 1]);
+                        acc[c + 2] = fmaf(p, x.z, acc[c + 2]);
+                        acc[c + 3] = fmaf(p, x.w, acc[c + 3]);
+                    }
+                }
+            }
+        }
+    }
+    const float inv = 1.0f / S;
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 32; c += 4)
+        *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
+    __syncthreads();
+    unstage_rows<T, PT, VEC>(y + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, Ks, ldv, a.dv_, w0, nvalid, lane);
+}
+
+template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void dq_wide_kernel(const Args a)
+{
+    extern __shared__ float4 smem4[];
+    float *Ks = reinterpret_cast<float *>(smem4);
+    S2_WIDE_IDS(a.Wo)
+    float *Vs = Ks + a.tile_rows * LS;
+    const int ho = a.gorder[a.row_first + rowsel];
+    const T *kx = static_cast<const T *>(a.k);
+    const T *vx = static_cast<const T *>(a.v);
+    const T *qy = static_cast<const T *>(a.q);
+    const T *gy = static_cast<const T *>(a.dy);
+    T *dq = static_cast<T *>(a.dq);
+
+    stage_rows<T, PT, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, PT, VEC>(Vs, gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, ldv, a.dv_, w0, a.Wo, nvalid, lane);
+    __syncthreads();
+    float qr[32], gr[32], Ak[32], Akg[32];
+#pragma unroll
+    for (int c = 0; c < 32; c++) {
+        qr[c] = Ks[qi * LS + sl * 32 + c] * LOG2E;
+        gr[c] = Vs[qi * LS + sl * 32 + c];
+        Ak[c] = 0.f;
+        Akg[c] = 0.f;
+    }
+    float m = NEG_BIG, S = 0.f, Ag = 0.f;
+
+    for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
+        const Run run = a.gruns[ri];
+        const float w = a.quad_w[run.lat];
+        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
+        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        for (int t0 = 0; t0 < run.len; t0 += TL) {
+            const int L = min(TL, run.len - t0);
+            const int c0 = (run.ws + t0 + ps * w0) % a.Wi;
+            const int nrows = ps * (nvalid - 1) + L;
+            __syncthreads();
+            stage_rows<T, PT, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            __syncthreads();
+            const float *krow = Ks + (ps * qi) * LS + sl * 32;
+            const float *vrow = Vs + (ps * qi) * LS + sl * 32;
+            float s[TL], g[TL];
+            float cm = NEG_BIG;
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                s[t] = NEG_BIG;
+                g[t] = 0.f;
+                if (t < L) {
+                    s[t] = slice_sum<LPQ>(dot_row<32>(qr, krow + t * LS));
+                    g[t] = slice_sum<LPQ>(dot_row<32>(gr, vrow + t * LS));
+                    cm = fmaxf(cm, s[t]);
+                }
+            }
+            const float mn = fmaxf(m, cm);
+            const float corr = fast_exp2(m - mn);
+            m = mn;
+            S *= corr;
+            Ag *= corr;
+#pragma unroll
+            for (int c = 0; c < 32; c++) {
+                Ak[c] *= corr;
+                Akg[c] *= corr;
+            }
+#pragma unroll
+            for (int t = 0; t < TL; t++) {
+                if (t < L) {
+                    const float p = fast_exp2(s[t] - mn) * w;
+                    const float pg = p * g[t];
+                    S += p;
+                    Ag += pg;
+                    const float *kr = krow + t * LS;
+#pragma unroll
+                    for (int c = 0; c < 32; c += 4) {
+                        const float4 x = *reinterpret_cast<const float4 *>(kr + c);
+                        Ak[c + 0] = fmaf(p, x.x, Ak[c + 0]);
+                        Ak[c + 1] = fmaf(p, x.y, Ak[c + 1]);
+                        Ak[c + 2] = fmaf(p, x.z, Ak[c + 2]);
+                        Ak[c + 3] = fmaf(p, x.w, Ak[c + 3]);
+                        Akg[c + 0] = fmaf(pg, x.x, Akg[c + 0]);
+                        Akg[c + 1] = fmaf(pg, x.y, Akg[c + 1]);
+                        Akg[c + 2] = fmaf(pg, x.z, Akg[c + 2]);
+                        Akg[c + 3] = fmaf(pg, x.w, Akg[c + 3]);
+                    }
+                }
+            }
+        }
+    }
+    const float inv = 1.0f / S;
+    const float I = Ag * inv;
+    if (qi < nvalid && sl == 0) a.stats[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = make_float2(m + fast_log2(S), I);
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 32; c += 4)
+        *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c)
+            = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
+                          (Akg[c + 3] - I * Ak[c + 3]) * inv);
+    __syncthreads();
+    unstage_rows<T, PT, VEC>(dq + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, Ks, ldk, a.dk_, w0, nvalid, lane);
+}
+
+template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void dkdv_wide_kernel(const Args a)
+{
+    extern __shared__ float4 smem4[];
+    float *Qs = reinterpret_cast<float *>(smem4);
+    S2_WIDE_IDS(a.Wi)
+    float *Gs = Qs + a.tile_rows * LS;
+    float2 *Ss = reinterpret_cast<float2 *>(Gs + a.tile_rows * LS);
+    const int hi = a.sorder[a.row_first + rowsel];
+    const T *kx = static_cast<const T *>(a.k);
+    const T *vx = static_cast<const T *>(a.v);
+    const T *qy = static_cast<const T *>(a.q);
+    const T *gy = static_cast<const T *>(a.dy);
+    T *dk = static_cast<T *>(a.dk);
+    T *dv = static_cast<T *>(a.dv);
+
+    stage_rows<T, PT, VEC>(Qs, kx + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, ldk, a.dk_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, PT, VEC>(Gs, vx + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, ldv, a.dv_, w0, a.Wi, nvalid, lane);
+    __syncthreads();
+    float kr[32], vr[32], dkr[32], dvr[32];
+#pragma unroll
+    for (int c = 0; c < 32; c++) {
+        kr[c] = Qs[qi * LS + sl * 32 + c] * LOG2E;
+        vr[c] = Gs[qi * LS + sl * 32 + c];
+        dkr[c] = 0.f;
+        dvr[c] = 0.f;
+    }
+    const float w = a.quad_w[hi];
+
+    for (int ri = a.soff[hi]; ri < a.soff[hi + 1]; ri++) {
+        const Run run = a.sruns[ri];
+        const int ho = run.lat;
+        int d0 = w0 - run.ws;
+        if (d0 < 0) d0 += a.Wi;
+        const int al = (d0 + qi) / ps - d0 / ps;
+        const int r0 = (d0 + qi) % ps;
+        const int a0 = d0 / ps;
+        const int span = (d0 + nvalid - 1) / ps - a0;
+        const int U = (run.len + ps - 1) / ps;
+        const T *ql = qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_;
+        const T *gl = gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_;
+        const float2 *sl2 = a.stats + ((long)bh * a.Ho + ho) * a.Wo;
+        for (int u0 = 0; u0 < U; u0 += TL) {
+            const int UL = min(TL, U - u0);
+            int c0 = (a0 - u0 - UL + 1) % a.Wo;
+            if (c0 < 0) c0 += a.Wo;
+            const int nrows = span + UL;
+            __syncthreads();
+            stage_rows<T, PT, VEC>(Qs, ql, ldk, a.dk_, c0, a.Wo, nrows, lane);
+            stage_rows<T, PT, VEC>(Gs, gl, ldv, a.dv_, c0, a.Wo, nrows, lane);
+            for (int r = lane; r < nrows; r += TQ) {
+                int col = c0 + r;
+                while (col >= a.Wo) col -= a.Wo;
+                Ss[r] = sl2[col];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int jj = 0; jj < TL; jj++) {
+                if (jj < UL) {
+                    const int row = al + (UL - 1 - jj);
+                    const int t = r0 + ps * (u0 + jj);
+                    const float *qrow = Qs + row * LS + sl * 32;
+                    const float *grow = Gs + row * LS + sl * 32;
+                    const float s = slice_sum<LPQ>(dot_row<32>(kr, qrow));
+                    const float g = slice_sum<LPQ>(dot_row<32>(vr, grow));
+                    const float2 st = Ss[row];
+                    float p = fast_exp2(s - st.x) * w;
+                    if (t >= run.len) p = 0.f;
+                    const float coef = p * (g - st.y);
+#pragma unroll
+                    for (int c = 0; c < 32; c += 4) {
+                        const float4 x = *reinterpret_cast<const float4 *>(qrow + c);
+                        const float4 z = *reinterpret_cast<const float4 *>(grow + c);
+                        dkr[c + 0] = fmaf(coef, x.x, dkr[c + 0]);
+                        dkr[c + 1] = fmaf(coef, x.y, dkr[c + 1]);
+                        dkr[c + 2] = fmaf(coef, x.z, dkr[c + 2]);
+                        dkr[c + 3] = fmaf(coef, x.w, dkr[c + 3]);
+                        dvr[c + 0] = fmaf(p, z.x, dvr[c + 0]);
+                        dvr[c + 1] = fmaf(p, z.y, dvr[c + 1]);
+                        dvr[c + 2] = fmaf(p, z.z, dvr[c + 2]);
+                        dvr[c + 3] = fmaf(p, z.w, dvr[c + 3]);
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int c = 0; c < 32; c += 4) {
+        *reinterpret_cast<float4 *>(Qs + qi * LS + sl * 32 + c) = make_float4(dkr[c], dkr[c + 1], dkr[c + 2], dkr[c + 3]);
+        *reinterpret_cast<float4 *>(Gs + qi * LS + sl * 32 + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
+    }
+    __syncthreads();
+    unstage_rows<T, PT, VEC>(dk + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, Qs, ldk, a.dk_, w0, nvalid, lane);
+    unstage_rows<T, PT, VEC>(dv + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, Gs, ldv, a.dv_, w0, nvalid, lane);
+}
+
 // ---------------------------------------------------------------------------------
 // Software-pipelined band staging (fast path: vector loads, pscale == 1, nlon >= tile rows).
 // A band of up to TQ-1+TL grid points is fetched into registers with one 16-byte (8-byte for
@@ -1652,8 +1961,8 @@ int check_shape(const s2attn_shape *sh)
         return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d)", sh->nlon_in, sh->nlon_out);
     if (sh->dtype != S2ATTN_F32 && sh->dtype != S2ATTN_BF16 && sh->dtype != S2ATTN_F16)
         return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
-    if (sh->ck > 32 || sh->cv > 32)
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 32 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
+    if (sh->ck > 128 || sh->cv > 128)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 128 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
     return S2ATTN_OK;
 }
 
@@ -1702,9 +2011,46 @@ template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a
     return S2ATTN_OK;
 }
 
+template <typename T, int LPQ, bool VEC> int launch_wide(Which which, const Args &a0, int row_first, int row_count, hipStream_t stream)
+{
+    if (row_count <= 0) return S2ATTN_OK;
+    Args a = a0;
+    a.row_first = row_first;
+    constexpr int TQW = TQ / LPQ, LS = 32 * LPQ + 4;
+    const int BH = a.B * a.nh;
+    void (*kern)(const Args) = nullptr;
+    long nblocks = 0;
+    size_t lds = 0;
+    if (which == DKDV) {
+        kern = dkdv_wide_kernel<T, LPQ, VEC>;
+        a.tile_rows = (TQW - 1) / a.pscale + 1 + TL;
+        if (a.tile_rows < TQW) a.tile_rows = TQW;
+        nblocks = (long)row_count * ((a.Wi + TQW - 1) / TQW) * BH;
+        lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
+    } else {
+        kern = which == FWD ? fwd_wide_kernel<T, LPQ, VEC> : dq_wide_kernel<T, LPQ, VEC>;
+        a.tile_rows = a.pscale * (TQW - 1) + TL;
+        if (a.tile_rows < TQW) a.tile_rows = TQW;
+        nblocks = (long)row_count * ((a.Wo + TQW - 1) / TQW) * BH;
+        lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
+    }
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "longitude ratio %d needs %zu bytes of LDS per workgroup", a.pscale, lds);
+    if (lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(TQ), lds, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+
 template <typename T, bool VEC> int launch_p(Which which, const Args &a, int row_first, int row_count, hipStream_t stream)
 {
     const int d = a.dk_ > a.dv_ ? a.dk_ : a.dv_;
+    if (d > 64) return launch_wide<T, 4, VEC>(which, a, row_first, row_count, stream);
+    if (d > 32) return launch_wide<T, 2, VEC>(which, a, row_first, row_count, stream);
     if (d <= 4) return launch_one<T, 4, VEC>(which, a, row_first, row_count, stream);
     if (d <= 8) return launch_one<T, 8, VEC>(which, a, row_first, row_count, stream);
     if (d <= 16) return launch_one<T, 16, VEC>(which, a, row_first, row_count, stream);
