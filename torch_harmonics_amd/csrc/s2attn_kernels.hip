@@ -1385,27 +1385,6 @@ template <typename T> struct Tile40 {
     }
 };
 
-template <typename T> struct Tile32 {
-    typedef typename Vec4<T>::type raw_t;
-    raw_t raw[4];
-    __device__ inline void fetch(const T *src, unsigned ld, int c0, int W, int lane)
-    {
-        const int colA = c0 + (lane >> 3), cb = 4 * (lane & 7);
-#pragma unroll
-        for (int it = 0; it < 4; it++) {
-            int col = colA + it * 8;
-            col -= (col >= W) ? W : 0;
-            raw[it] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
-        }
-    }
-    template <int LS> __device__ inline void commit(float *dst, int lane) const
-    {
-        const int r0 = lane >> 3, cb = 4 * (lane & 7);
-#pragma unroll
-        for (int it = 0; it < 4; it++) *reinterpret_cast<float4 *>(dst + (r0 + it * 8) * LS + cb) = widen4(raw[it], (const T *)nullptr);
-    }
-};
-
 // A run is walked either in matrix-core tiles of 32 band positions (pos = first position, len + 31 positions in all)
 // or, when short, in vector chunks of VC neighbors (pos = first neighbor index).
 __device__ inline bool run_is_dense(int len) { return len >= LMIN; }
@@ -1431,8 +1410,8 @@ __device__ inline int run_stride(int len) { return run_is_dense(len) ? MT : VC; 
 // computes half of a dot product, one cross-half exchange completes it).
 template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(const Args a)
 {
-    __shared__ float Ks[MR * MLK];
-    __shared__ float Vs[MR * MLK];
+    __shared__ __attribute__((aligned(16))) float Ks[MR * MLK];
+    __shared__ __attribute__((aligned(16))) float Vs[MR * MLK];
 
     S2_MFMA_IDS(a.Wo)
     const int ho = a.gorder[a.row_first + rowsel];
@@ -1615,13 +1594,14 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     }
 }
 
-// backward dq + statistics, dense: same column ownership as the forward.  Per tile four matrix products:
-//   S^T = K Q^T,  G^T = V dY^T,  A_k^T += K^T P^T,  A_kg^T += K^T (P o G)^T   (A operands of the last two are
-//   column reads of the K tile, B operands the probability registers), online softmax across tiles.
+// backward dq + statistics: same ownership as the forward (lane (j, half): query j, channels 8g + 4 half + e).
+// Matrix-core tile, four products:  S^T = K Q^T,  G^T = V dY^T,  A_k^T += K^T P^T,  A_kg^T += K^T (P o G)^T  (the A
+// operands of the last two are column reads of the K tile, the B operands the probability registers); short runs take
+// the vector path on the same accumulators.  Online softmax across tiles and chunks.
 template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const Args a)
 {
-    __shared__ float Ks[MT * MLK];
-    __shared__ float Vs[MT * MLK];
+    __shared__ __attribute__((aligned(16))) float Ks[MR * MLK];
+    __shared__ __attribute__((aligned(16))) float Vs[MR * MLK];
 
     S2_MFMA_IDS(a.Wo)
     const int ho = a.gorder[a.row_first + rowsel];
@@ -1633,14 +1613,14 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
 
     float qb[16], gb[16];
     {
-        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 16 * half;
-        const T *grow = static_cast<const T *>(a.dy) + pt * ldv + (size_t)h * 32 + 16 * half;
+        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 4 * half;
+        const T *grow = static_cast<const T *>(a.dy) + pt * ldv + (size_t)h * 32 + 4 * half;
 #pragma unroll
-        for (int c = 0; c < 16; c += 4) {
-            const float4 x = load4(qrow + c);
-            const float4 z = load4(grow + c);
-            qb[c] = x.x * LOG2E, qb[c + 1] = x.y * LOG2E, qb[c + 2] = x.z * LOG2E, qb[c + 3] = x.w * LOG2E;
-            gb[c] = z.x, gb[c + 1] = z.y, gb[c + 2] = z.z, gb[c + 3] = z.w;
+        for (int g = 0; g < 4; g++) {
+            const float4 x = load4(qrow + 8 * g);
+            const float4 z = load4(grow + 8 * g);
+            qb[4 * g] = x.x * LOG2E, qb[4 * g + 1] = x.y * LOG2E, qb[4 * g + 2] = x.z * LOG2E, qb[4 * g + 3] = x.w * LOG2E;
+            gb[4 * g] = z.x, gb[4 * g + 1] = z.y, gb[4 * g + 2] = z.z, gb[4 * g + 3] = z.w;
         }
     }
     f16v Ak, Akg;
@@ -1653,108 +1633,175 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
 
     int ri = a.goff[ho];
     const int rend = a.goff[ho + 1];
-    int u0 = 0;
+    int pos = 0;
     Run run = {0, 0, 0, 0};
-    Tile32<T> kt, vt;
-    auto fetch = [&](const Run &rn, int u) {
-        const int c0 = (rn.ws + w0 + u) % a.Wi;
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane);
+    Tile40<T> kt, vt;
+    auto fetch = [&](const Run &rn, int p) {
+        const int c0 = (rn.ws + w0 + p) % a.Wi;
+        const bool fifth = !run_is_dense(rn.len);
+        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane, fifth);
+        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane, fifth);
     };
     if (ri < rend) {
         run = a.gruns[ri];
         fetch(run, 0);
-        kt.template commit<MLK>(Ks, lane);
-        vt.template commit<MLK>(Vs, lane);
+        kt.commit(Ks, lane, !run_is_dense(run.len));
+        vt.commit(Vs, lane, !run_is_dense(run.len));
     }
     __syncthreads();
 
     while (ri < rend) {
         const float w = a.quad_w[run.lat];
         const int len = run.len;
-        int nri = ri, nu0 = u0 + MT;
+        int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
-        if (nu0 >= len + MT - 1) {
+        if (run_done(len, npos)) {
             nri++;
-            nu0 = 0;
+            npos = 0;
             if (nri < rend) nrun = a.gruns[nri];
         }
         const bool more = nri < rend;
-        if (more) fetch(nrun, nu0);
+        if (more) fetch(nrun, npos);
 
-        f16v sc, gc;
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            sc[v] = 0.f;
-            gc[v] = 0.f;
-        }
-        {
-            const float *kr = Ks + j * MLK + 16 * half;
-            const float *vr = Vs + j * MLK + 16 * half;
-#pragma unroll
-            for (int c = 0; c < 16; c += 4) {
-                const float4 x = *reinterpret_cast<const float4 *>(kr + c);
-                const float4 z = *reinterpret_cast<const float4 *>(vr + c);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[c + 0], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, gb[c + 0], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[c + 1], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, gb[c + 1], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[c + 2], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, gb[c + 2], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[c + 3], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, gb[c + 3], gc, 0, 0, 0);
-            }
-        }
-        const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
-        if (edge) {
+        const float *kq = Ks + j * MLK + 4 * half;
+        const float *vq = Vs + j * MLK + 4 * half;
+        if (run_is_dense(len)) {
+            const int u0 = pos;
+            f16v sc, gc;
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const int t = u0 + kappa(v, half) - j;
-                sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
+                sc[v] = 0.f;
+                gc[v] = 0.f;
             }
-        }
-        float mx = sc[0];
 #pragma unroll
-        for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
-        mx = fmaxf(mx, __shfl_xor(mx, 32));
-        const float mn = fmaxf(m, mx);
-        const float corr = fast_exp2(m - mn);
-        m = mn;
-        float rs = 0.f, rg = 0.f;
+            for (int g = 0; g < 4; g++) {
+                const float4 x = *reinterpret_cast<const float4 *>(kq + 8 * g);
+                const float4 z = *reinterpret_cast<const float4 *>(vq + 8 * g);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[4 * g + 0], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, gb[4 * g + 0], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[4 * g + 1], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, gb[4 * g + 1], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[4 * g + 2], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, gb[4 * g + 2], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[4 * g + 3], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, gb[4 * g + 3], gc, 0, 0, 0);
+            }
+            const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
+            if (edge) {
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            float p = fast_exp2(sc[v] - mn) * w;
-            if (edge) p = (sc[v] == NEG_BIG) ? 0.f : p;
-            const float pg = p * gc[v];
-            sc[v] = p;
-            gc[v] = pg;
-            rs += p;
-            rg += pg;
-        }
-        rs += __shfl_xor(rs, 32);
-        rg += __shfl_xor(rg, 32);
-        S = S * corr + rs;
-        Ag = Ag * corr + rg;
+                for (int v = 0; v < 16; v++) {
+                    const int t = u0 + kappa(v, half) - j;
+                    sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
+                }
+            }
+            float mx = sc[0];
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            Ak[v] *= corr;
-            Akg[v] *= corr;
-        }
+            for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
+            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            const float mn = fmaxf(m, mx);
+            if (__any(mn > m)) {
+                const float corr = fast_exp2(m - mn);
+                S *= corr;
+                Ag *= corr;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float x = Ks[kappa(v, half) * MLK + j];
-            Ak = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], Ak, 0, 0, 0);
-            Akg = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], Akg, 0, 0, 0);
+                for (int v = 0; v < 16; v++) {
+                    Ak[v] *= corr;
+                    Akg[v] *= corr;
+                }
+            }
+            m = mn;
+            float rs = 0.f, rg = 0.f;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                float p = fast_exp2(sc[v] - mn) * w;
+                if (edge) p = (sc[v] == NEG_BIG) ? 0.f : p;
+                const float pg = p * gc[v];
+                sc[v] = p;
+                gc[v] = pg;
+                rs += p;
+                rg += pg;
+            }
+            rs += __shfl_xor(rs, 32);
+            rg += __shfl_xor(rg, 32);
+            S += rs;
+            Ag += rg;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float x = Ks[kappa(v, half) * MLK + j];
+                Ak = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], Ak, 0, 0, 0);
+                Akg = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], Akg, 0, 0, 0);
+            }
+        } else {
+            const int L = min(VC, len - pos);
+            float s[VC], gd[VC];
+            float cm = NEG_BIG;
+#pragma unroll
+            for (int t = 0; t < VC; t++) {
+                s[t] = NEG_BIG;
+                gd[t] = 0.f;
+                if (t < L) {
+                    float ps_ = 0.f, pg_ = 0.f;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float4 x = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
+                        const float4 z = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
+                        ps_ = fmaf(qb[4 * g], x.x, ps_);
+                        ps_ = fmaf(qb[4 * g + 1], x.y, ps_);
+                        ps_ = fmaf(qb[4 * g + 2], x.z, ps_);
+                        ps_ = fmaf(qb[4 * g + 3], x.w, ps_);
+                        pg_ = fmaf(gb[4 * g], z.x, pg_);
+                        pg_ = fmaf(gb[4 * g + 1], z.y, pg_);
+                        pg_ = fmaf(gb[4 * g + 2], z.z, pg_);
+                        pg_ = fmaf(gb[4 * g + 3], z.w, pg_);
+                    }
+                    s[t] = ps_ + __shfl_xor(ps_, 32);
+                    gd[t] = pg_ + __shfl_xor(pg_, 32);
+                    cm = fmaxf(cm, s[t]);
+                }
+            }
+            const float mn = fmaxf(m, cm);
+            if (__any(mn > m)) {
+                const float corr = fast_exp2(m - mn);
+                S *= corr;
+                Ag *= corr;
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    Ak[v] *= corr;
+                    Akg[v] *= corr;
+                }
+            }
+            m = mn;
+#pragma unroll
+            for (int t = 0; t < VC; t++) {
+                if (t < L) {
+                    const float p = fast_exp2(s[t] - mn) * w;
+                    const float pg = p * gd[t];
+                    S += p;
+                    Ag += pg;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        const float4 x = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
+                        Ak[4 * g] = fmaf(p, x.x, Ak[4 * g]);
+                        Ak[4 * g + 1] = fmaf(p, x.y, Ak[4 * g + 1]);
+                        Ak[4 * g + 2] = fmaf(p, x.z, Ak[4 * g + 2]);
+                        Ak[4 * g + 3] = fmaf(p, x.w, Ak[4 * g + 3]);
+                        Akg[4 * g] = fmaf(pg, x.x, Akg[4 * g]);
+                        Akg[4 * g + 1] = fmaf(pg, x.y, Akg[4 * g + 1]);
+                        Akg[4 * g + 2] = fmaf(pg, x.z, Akg[4 * g + 2]);
+                        Akg[4 * g + 3] = fmaf(pg, x.w, Akg[4 * g + 3]);
+                    }
+                }
+            }
         }
 
         __syncthreads();
         if (more) {
-            kt.template commit<MLK>(Ks, lane);
-            vt.template commit<MLK>(Vs, lane);
+            kt.commit(Ks, lane, !run_is_dense(nrun.len));
+            vt.commit(Vs, lane, !run_is_dense(nrun.len));
         }
         __syncthreads();
         ri = nri;
-        u0 = nu0;
+        pos = npos;
         run = nrun;
     }
 
@@ -1770,16 +1817,17 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
     }
 }
 
-// backward dk/dv, dense: lane owns INPUT longitude j of the tile.  For a run (ho, ws, len) the queries that see the
-// tile's keys are the len + 31 longitudes starting at w0 - ws - len + 1; query row r sees key j iff 0 <= r - j < len.
-// Per tile of 32 query rows:  S = Q K^T and G = dY V^T come out as [query][key] (a lane holds 16 queries of ITS key
-// column), P = exp2(S - lse_query) w, C = P (G - I_query), then dK^T += Q^T C and dV^T += dY^T P.
+// backward dk/dv: lane (j, half) owns INPUT longitude j of the tile, channels 8g + 4 half + e.  For a run (ho, ws, len)
+// the queries that see the tile's keys are the len + 31 longitudes starting at w0 - ws - len + 1; query row r sees key j
+// iff 0 <= r - j < len.  Matrix-core tile of 32 query rows:  S = Q K^T and G = dY V^T come out as [query][key] (a lane
+// holds 16 queries of ITS key column), P = exp2(S - lse_query) w, C = P (G - I_query), then dK^T += Q^T C and
+// dV^T += dY^T P.  Short runs: vector chunks of VC query rows starting at row pos, key j reads staged rows j + i.
 template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(const Args a)
 {
-    __shared__ float Qs[MT * MLK];
-    __shared__ float Gs[MT * MLK];
-    __shared__ float Ls[MT];
-    __shared__ float Is[MT];
+    __shared__ __attribute__((aligned(16))) float Qs[MR * MLK];
+    __shared__ __attribute__((aligned(16))) float Gs[MR * MLK];
+    __shared__ __attribute__((aligned(16))) float Ls[MR];
+    __shared__ __attribute__((aligned(16))) float Is[MR];
 
     S2_MFMA_IDS(a.Wi)
     const int hi = a.sorder[a.row_first + rowsel];
@@ -1792,14 +1840,14 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
 
     float kb[16], vb[16];
     {
-        const T *krow = static_cast<const T *>(a.k) + pt * ldk + (size_t)h * 32 + 16 * half;
-        const T *vrow = static_cast<const T *>(a.v) + pt * ldv + (size_t)h * 32 + 16 * half;
+        const T *krow = static_cast<const T *>(a.k) + pt * ldk + (size_t)h * 32 + 4 * half;
+        const T *vrow = static_cast<const T *>(a.v) + pt * ldv + (size_t)h * 32 + 4 * half;
 #pragma unroll
-        for (int c = 0; c < 16; c += 4) {
-            const float4 x = load4(krow + c);
-            const float4 z = load4(vrow + c);
-            kb[c] = x.x * LOG2E, kb[c + 1] = x.y * LOG2E, kb[c + 2] = x.z * LOG2E, kb[c + 3] = x.w * LOG2E;
-            vb[c] = z.x, vb[c + 1] = z.y, vb[c + 2] = z.z, vb[c + 3] = z.w;
+        for (int g = 0; g < 4; g++) {
+            const float4 x = load4(krow + 8 * g);
+            const float4 z = load4(vrow + 8 * g);
+            kb[4 * g] = x.x * LOG2E, kb[4 * g + 1] = x.y * LOG2E, kb[4 * g + 2] = x.z * LOG2E, kb[4 * g + 3] = x.w * LOG2E;
+            vb[4 * g] = z.x, vb[4 * g + 1] = z.y, vb[4 * g + 2] = z.z, vb[4 * g + 3] = z.w;
         }
     }
     f16v dkt, dvt;
@@ -1812,101 +1860,140 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
 
     int ri = a.soff[hi];
     const int rend = a.soff[hi + 1];
-    int r0 = 0;
+    int pos = 0;
     Run run = {0, 0, 0, 0};
-    Tile32<T> qt, gt;
+    Tile40<T> qt, gt;
     float2 st = make_float2(0.f, 0.f);
-    auto fetch = [&](const Run &rn, int r) {
-        int c0 = (w0 - rn.ws - rn.len + 1 + r) % a.Wo;
+    auto fetch = [&](const Run &rn, int p) {
+        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
-        qt.fetch(qy + (size_t)rn.lat * a.Wo * ldk, ldk, c0, a.Wo, lane);
-        gt.fetch(gy + (size_t)rn.lat * a.Wo * ldv, ldv, c0, a.Wo, lane);
-        int col = c0 + j;
+        const bool fifth = !run_is_dense(rn.len);
+        qt.fetch(qy + (size_t)rn.lat * a.Wo * ldk, ldk, c0, a.Wo, lane, fifth);
+        gt.fetch(gy + (size_t)rn.lat * a.Wo * ldv, ldv, c0, a.Wo, lane, fifth);
+        int col = c0 + lane; // lanes 0..39 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
-        st = stats[(size_t)rn.lat * a.Wo + col];
+        if (lane < MR) st = stats[(size_t)rn.lat * a.Wo + col];
     };
-    auto commit = [&]() {
-        qt.template commit<MLK>(Qs, lane);
-        gt.template commit<MLK>(Gs, lane);
-        if (half == 0) {
-            Ls[j] = st.x;
-            Is[j] = st.y;
+    auto commit = [&](bool fifth) {
+        qt.commit(Qs, lane, fifth);
+        gt.commit(Gs, lane, fifth);
+        if (lane < MR) {
+            Ls[lane] = st.x;
+            Is[lane] = st.y;
         }
     };
     if (ri < rend) {
         run = a.sruns[ri];
         fetch(run, 0);
-        commit();
+        commit(!run_is_dense(run.len));
     }
     __syncthreads();
 
     while (ri < rend) {
         const int len = run.len;
-        int nri = ri, nr0 = r0 + MT;
+        int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
-        if (nr0 >= len + MT - 1) {
+        if (run_done(len, npos)) {
             nri++;
-            nr0 = 0;
+            npos = 0;
             if (nri < rend) nrun = a.sruns[nri];
         }
         const bool more = nri < rend;
-        if (more) fetch(nrun, nr0);
+        if (more) fetch(nrun, npos);
 
-        f16v sc, gc;
+        const float *qq = Qs + j * MLK + 4 * half;
+        const float *gq = Gs + j * MLK + 4 * half;
+        if (run_is_dense(len)) {
+            const int r0 = pos;
+            f16v sc, gc;
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            sc[v] = 0.f;
-            gc[v] = 0.f;
-        }
-        {
-            const float *qr = Qs + j * MLK + 16 * half;
-            const float *gr = Gs + j * MLK + 16 * half;
-#pragma unroll
-            for (int c = 0; c < 16; c += 4) {
-                const float4 x = *reinterpret_cast<const float4 *>(qr + c);
-                const float4 z = *reinterpret_cast<const float4 *>(gr + c);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, kb[c + 0], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, vb[c + 0], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, kb[c + 1], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, vb[c + 1], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, kb[c + 2], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, vb[c + 2], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, kb[c + 3], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, vb[c + 3], gc, 0, 0, 0);
+            for (int v = 0; v < 16; v++) {
+                sc[v] = 0.f;
+                gc[v] = 0.f;
             }
-        }
-        const bool edge = (r0 < MT - 1) || (r0 + MT - 1 >= len);
 #pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 8 * g + 4 * half);
-            const float4 i4 = *reinterpret_cast<const float4 *>(Is + 8 * g + 4 * half);
-            const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
-            const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
+            for (int g = 0; g < 4; g++) {
+                const float4 x = *reinterpret_cast<const float4 *>(qq + 8 * g);
+                const float4 z = *reinterpret_cast<const float4 *>(gq + 8 * g);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, kb[4 * g + 0], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, vb[4 * g + 0], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, kb[4 * g + 1], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, vb[4 * g + 1], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, kb[4 * g + 2], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, vb[4 * g + 2], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, kb[4 * g + 3], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, vb[4 * g + 3], gc, 0, 0, 0);
+            }
+            const bool edge = (r0 < MT - 1) || (r0 + MT - 1 >= len);
 #pragma unroll
-            for (int e = 0; e < 4; e++) {
-                const int v = 4 * g + e;
-                float p = fast_exp2(sc[v] - lv[e]) * w;
-                if (edge) {
-                    const int t = r0 + kappa(v, half) - j;
-                    p = (t >= 0 && t < len) ? p : 0.f;
+            for (int g = 0; g < 4; g++) {
+                const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 8 * g + 4 * half);
+                const float4 i4 = *reinterpret_cast<const float4 *>(Is + 8 * g + 4 * half);
+                const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+                const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const int v = 4 * g + e;
+                    float p = fast_exp2(sc[v] - lv[e]) * w;
+                    if (edge) {
+                        const int t = r0 + kappa(v, half) - j;
+                        p = (t >= 0 && t < len) ? p : 0.f;
+                    }
+                    sc[v] = p;
+                    gc[v] = p * (gc[v] - iv[e]);
                 }
-                sc[v] = p;
-                gc[v] = p * (gc[v] - iv[e]);
             }
-        }
 #pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float x = Qs[kappa(v, half) * MLK + j];
-            const float z = Gs[kappa(v, half) * MLK + j];
-            dkt = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], dkt, 0, 0, 0);
-            dvt = __builtin_amdgcn_mfma_f32_32x32x2f32(z, sc[v], dvt, 0, 0, 0);
+            for (int v = 0; v < 16; v++) {
+                const float x = Qs[kappa(v, half) * MLK + j];
+                const float z = Gs[kappa(v, half) * MLK + j];
+                dkt = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], dkt, 0, 0, 0);
+                dvt = __builtin_amdgcn_mfma_f32_32x32x2f32(z, sc[v], dvt, 0, 0, 0);
+            }
+        } else {
+            const int L = min(VC, len - pos);
+#pragma unroll
+            for (int i = 0; i < VC; i++) {
+                if (i < L) {
+                    float4 xq[4], xg[4];
+                    float ps_ = 0.f, pg_ = 0.f;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        xq[g] = *reinterpret_cast<const float4 *>(qq + i * MLK + 8 * g);
+                        xg[g] = *reinterpret_cast<const float4 *>(gq + i * MLK + 8 * g);
+                        ps_ = fmaf(kb[4 * g], xq[g].x, ps_);
+                        ps_ = fmaf(kb[4 * g + 1], xq[g].y, ps_);
+                        ps_ = fmaf(kb[4 * g + 2], xq[g].z, ps_);
+                        ps_ = fmaf(kb[4 * g + 3], xq[g].w, ps_);
+                        pg_ = fmaf(vb[4 * g], xg[g].x, pg_);
+                        pg_ = fmaf(vb[4 * g + 1], xg[g].y, pg_);
+                        pg_ = fmaf(vb[4 * g + 2], xg[g].z, pg_);
+                        pg_ = fmaf(vb[4 * g + 3], xg[g].w, pg_);
+                    }
+                    const float s = ps_ + __shfl_xor(ps_, 32);
+                    const float gd = pg_ + __shfl_xor(pg_, 32);
+                    const float p = fast_exp2(s - Ls[j + i]) * w;
+                    const float coef = p * (gd - Is[j + i]);
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        dkt[4 * g] = fmaf(coef, xq[g].x, dkt[4 * g]);
+                        dkt[4 * g + 1] = fmaf(coef, xq[g].y, dkt[4 * g + 1]);
+                        dkt[4 * g + 2] = fmaf(coef, xq[g].z, dkt[4 * g + 2]);
+                        dkt[4 * g + 3] = fmaf(coef, xq[g].w, dkt[4 * g + 3]);
+                        dvt[4 * g] = fmaf(p, xg[g].x, dvt[4 * g]);
+                        dvt[4 * g + 1] = fmaf(p, xg[g].y, dvt[4 * g + 1]);
+                        dvt[4 * g + 2] = fmaf(p, xg[g].z, dvt[4 * g + 2]);
+                        dvt[4 * g + 3] = fmaf(p, xg[g].w, dvt[4 * g + 3]);
+                    }
+                }
+            }
         }
 
         __syncthreads();
-        if (more) commit();
+        if (more) commit(!run_is_dense(nrun.len));
         __syncthreads();
         ri = nri;
-        r0 = nr0;
+        pos = npos;
         run = nrun;
     }
 
@@ -2093,8 +2180,9 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
     const int nrows = which == DKDV ? a.Hi : a.Ho;
     int first = 0;
     if (dense_ok(which, a, vec)) {
-        // the forward kernel handles short runs itself (vector path inside), so it takes every latitude
-        const int take = which == FWD ? nrows : ndense;
+        // the dense kernels handle short runs themselves (vector path inside), so they take every latitude
+        (void)ndense;
+        const int take = nrows;
         const int rc = launch_dense<T>(which, a, take, stream);
         if (rc != S2ATTN_OK) return rc;
         first = take;
