@@ -1356,7 +1356,7 @@ __device__ inline int kappa(int v, int half) { return 8 * (v / 4) + 4 * half + (
 // 32 rows; the vector path for short runs uses all 40 (32 columns + up to 9 neighbors - 1).
 constexpr int MR = 40;  // rows of the LDS tile
 constexpr int VC = 9;   // neighbors per vector-path chunk (MT - 1 + VC <= MR)
-constexpr int LMIN = 20; // runs at least this long go through the matrix cores
+constexpr int LMIN = 32; // runs at least this long go through the matrix cores (measured optimum on cfg3: flat between 24 and 40)
 
 template <typename T> struct Tile40 {
     typedef typename Vec4<T>::type raw_t;
