@@ -33,6 +33,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
+FP32_MATRIX_PEAK_TFLOPS = 157.3  # dense fp32 MFMA: the unit the long-run (polar) part of the path runs on
 FP32_VALU_PEAK_TFLOPS = 78.6  # 157.3 TFLOP/s vector fp32 is quoted with packed FMA; these kernels are built without packed fp32
 
 CONFIGS = {
@@ -96,16 +97,16 @@ def make_workload(cfg, device, seed=333):
 def cpu_baseline(cfg, mod, k, v, q, dy):
     """
     Times the fp32 CPU port of the reference algorithm (oracle/s2attn_oracle.c, built with the reference's
-    release flags) forward + backward on a sample of the workload: the first two heads and every 12th output
+    release flags) forward + backward on a sample of the workload: the first four heads and every 6th output
     latitude (both pole rows included, so the reference backward's per-neighbor scratch is sized by the longest
     row, as in the full problem).  Throughput is neighbor pairs of the sample per second.
     """
     from oracle import cpu_attention as oracle
 
-    nh_s = min(2, cfg["nh"])
+    nh_s = min(4, cfg["nh"])
     ck, cv = mod.k_channels // cfg["nh"], mod.out_channels // cfg["nh"]
     Ho, Wo = cfg["out_shape"]
-    stride = 12 if Ho >= 120 else 1
+    stride = 6 if Ho >= 120 else 1
     rows = torch.arange(0, Ho, stride)
     if rows[-1] != Ho - 1:
         rows = torch.cat([rows, torch.tensor([Ho - 1])])
@@ -210,9 +211,9 @@ def main():
 
     nk, nv, nq, ny = k.numel(), v.numel(), q.numel(), y.numel()
     alg = {  # compulsory traffic of each kernel: every tensor it must read or write, once
-        "s2attn fwd_kernel": (esz * (nq + nk + nv + ny), t_fwd),
-        "s2attn dq_kernel": (esz * (nq + nk + nv + ny + nq), t_dq),
-        "s2attn dkdv_kernel": (esz * (nq + nk + nv + ny + nk + nv), t_dkdv),
+        "s2::fwd_mfma_kernel (forward)": (esz * (nq + nk + nv + ny), t_fwd),
+        "s2::dq_mfma_kernel (backward, dq + softmax statistics)": (esz * (nq + nk + nv + ny + nq), t_dq),
+        "s2::dkdv_mfma_kernel (backward, dk + dv)": (esz * (nq + nk + nv + ny + nk + nv), t_dkdv),
     }
     dom = max(alg, key=lambda n: alg[n][1])
     dom_bytes, dom_ms = alg[dom]
@@ -251,6 +252,7 @@ def main():
         },
         "kernel_ms": {"fwd": t_fwd, "dq": t_dq, "dkdv": t_dkdv},
         "step_hbm_frac": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "step_fp32_matrix_frac": flops_alg / (ms_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS,
         "step_fp32_valu_frac": flops_alg / (ms_step * 1e-3) / 1e12 / FP32_VALU_PEAK_TFLOPS,
     }
 
