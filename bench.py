@@ -217,6 +217,12 @@ def main():
     }
     dom = max(alg, key=lambda n: alg[n][1])
     dom_bytes, dom_ms = alg[dom]
+    # HBM bytes per launch measured with rocprofv3 counters on this workload (see profiles/); only valid for cfg3
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "cfg3_hbm_traffic.json")
+    if args.config == "cfg3" and os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(dom)
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
     step_bytes = esz * ((nq + nk + nv + ny) + (nq + nk + nv + ny + nq + nk + nv))
     d = k.shape[3] // nh
@@ -246,7 +252,7 @@ def main():
             "peak": HBM_PEAK_GBS,
             "unit": "GB/s",
             "frac": achieved / HBM_PEAK_GBS,
-            "traffic": None,
+            "traffic": traffic,
             "algorithmic_bytes": dom_bytes,
             "kernel_ms": dom_ms,
         },
