@@ -173,8 +173,8 @@ def main():
     esz = 4
 
     def step():
-        y = ops.forward(k, v, q, wq, ci, ro, nh, Wi, Ho, Wo)
-        return y, ops.backward(k, v, q, dy, wq, ci, ro, nh, Wi, Ho, Wo)
+        y, lse = ops.forward_lse(k, v, q, wq, ci, ro, nh, Wi, Ho, Wo)
+        return y, ops.backward_saved(k, v, q, dy, y, lse, wq, ci, ro, nh, Wi, Ho, Wo)
 
     for _ in range(args.warmup):
         step()
@@ -191,14 +191,20 @@ def main():
     y = torch.empty(q.shape[:3] + (v.shape[3],), device=dev)
     dk, dv, dq = torch.empty_like(k), torch.empty_like(v), torch.empty_like(q)
     ws = torch.empty(lib.s2attn_backward_workspace_bytes(ctypes.byref(shape)) // 4, device=dev)
+    lse = torch.empty((B, nh, Ho, Wo), device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     pl, sh = ctypes.byref(plan.struct), ctypes.byref(shape)
     ev = [[torch.cuda.Event(enable_timing=True) for _ in range(4)] for _ in range(args.steps)]
     for s in range(args.steps):
         ev[s][0].record()
-        _lib.check(lib.s2attn_forward(k.data_ptr(), v.data_ptr(), q.data_ptr(), wq.data_ptr(), y.data_ptr(), pl, sh, stream), "fwd")
+        _lib.check(lib.s2attn_forward_lse(k.data_ptr(), v.data_ptr(), q.data_ptr(), wq.data_ptr(), y.data_ptr(), lse.data_ptr(), pl, sh, stream), "fwd")
         ev[s][1].record()
-        _lib.check(lib.s2attn_backward_dq(k.data_ptr(), v.data_ptr(), q.data_ptr(), dy.data_ptr(), wq.data_ptr(), dq.data_ptr(), ws.data_ptr(), pl, sh, stream), "dq")
+        _lib.check(
+            lib.s2attn_backward_dq_saved(
+                k.data_ptr(), v.data_ptr(), q.data_ptr(), dy.data_ptr(), y.data_ptr(), lse.data_ptr(), wq.data_ptr(), dq.data_ptr(), ws.data_ptr(), pl, sh, stream
+            ),
+            "dq",
+        )
         ev[s][2].record()
         _lib.check(
             lib.s2attn_backward_dkdv(k.data_ptr(), v.data_ptr(), q.data_ptr(), dy.data_ptr(), wq.data_ptr(), dk.data_ptr(), dv.data_ptr(), ws.data_ptr(), pl, sh, stream), "dkdv"
@@ -209,11 +215,11 @@ def main():
     t_dq = sum(e[1].elapsed_time(e[2]) for e in ev) / args.steps
     t_dkdv = sum(e[2].elapsed_time(e[3]) for e in ev) / args.steps
 
-    nk, nv, nq, ny = k.numel(), v.numel(), q.numel(), y.numel()
+    nk, nv, nq, ny, nstat = k.numel(), v.numel(), q.numel(), y.numel(), lse.numel()
     alg = {  # compulsory traffic of each kernel: every tensor it must read or write, once
-        "s2::fwd_mfma_kernel (forward)": (esz * (nq + nk + nv + ny), t_fwd),
-        "s2::dq_mfma_kernel (backward, dq + softmax statistics)": (esz * (nq + nk + nv + ny + nq), t_dq),
-        "s2::dkdv_mfma_kernel (backward, dk + dv)": (esz * (nq + nk + nv + ny + nk + nv), t_dkdv),
+        "s2::fwd_mfma_kernel (forward)": (esz * (nq + nk + nv + ny) + 4 * nstat, t_fwd),
+        "s2::dq_saved_mfma_kernel (backward, dq)": (esz * (nq + nk + nv + ny + ny + nq) + 12 * nstat, t_dq),
+        "s2::dkdv_mfma_kernel (backward, dk + dv)": (esz * (nq + nk + nv + ny + nk + nv) + 8 * nstat, t_dkdv),
     }
     dom = max(alg, key=lambda n: alg[n][1])
     dom_bytes, dom_ms = alg[dom]
@@ -224,7 +230,8 @@ def main():
         with open(tpath) as f:
             traffic = json.load(f).get(dom)
     achieved = dom_bytes / (dom_ms * 1e-3) / 1e9
-    step_bytes = esz * ((nq + nk + nv + ny) + (nq + nk + nv + ny + nq + nk + nv))
+    # the step's own compulsory traffic: the backward counted as one pass (k, v, q, dy, y read once; dk, dv, dq written)
+    step_bytes = esz * ((nq + nk + nv + ny) + (nq + nk + nv + ny + ny + nq + nk + nv)) + 8 * nstat
     d = k.shape[3] // nh
     flops_alg = 14 * d * pairs
 

@@ -103,6 +103,15 @@ int s2attn_forward(const void *k, const void *v, const void *q, const float *qua
                    const s2attn_plan *plan, const s2attn_shape *shape, void *stream);
 
 /*
+ * Forward that also returns the softmax statistic lse[B, num_heads, nlat_out, nlon_out] (fp32, log2 of
+ * sum_j exp(q.k_j) quad_weights[hi_j], i.e. in the log2 domain the kernels work in) for s2attn_backward_saved.
+ * Same reference entry point as s2attn_forward; the reference saves only its inputs for backward
+ * (_attention_utils.py:94-100) and recomputes the statistics.
+ */
+int s2attn_forward_lse(const void *k, const void *v, const void *q, const float *quad_weights, void *y, float *lse,
+                       const s2attn_plan *plan, const s2attn_shape *shape, void *stream);
+
+/*
  * Backward.  Replaces attention_kernels::backward (attention_interface.cpp:117-119;
  * CUDA implementation s2_attention_bwd_dkvq_cuda, attention_cuda_bwd.cu:856-956).
  * Writes dk, dv, dq (every element; no pre-zeroing needed, no atomics).
@@ -128,6 +137,20 @@ int s2attn_backward_dq(const void *k, const void *v, const void *q, const void *
 int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
                          void *dk, void *dv, const void *workspace, const s2attn_plan *plan, const s2attn_shape *shape,
                          void *stream);
+
+/*
+ * Backward from saved forward results: y (the forward output) and lse (from s2attn_forward_lse) make the softmax
+ * final from the first neighbor on, which saves one of the four matrix products of the dq pass and all running-maximum
+ * bookkeeping.  Same outputs as s2attn_backward to rounding; same workspace.  Shapes outside the matrix-core kernels'
+ * domain (head dim != 32, nlon_in != nlon_out, nlon < 64) ignore y and lse and take the s2attn_backward path.
+ */
+int s2attn_backward_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
+                          const float *quad_weights, void *dk, void *dv, void *dq, void *workspace, const s2attn_plan *plan,
+                          const s2attn_shape *shape, void *stream);
+
+int s2attn_backward_dq_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
+                             const float *quad_weights, void *dq, void *workspace, const s2attn_plan *plan,
+                             const s2attn_shape *shape, void *stream);
 
 /*
  * Layout conversion.  Replace attention_kernels::permute_to_nhwc / permute_to_nchw

@@ -31,13 +31,17 @@ def _setup(name, heads=None, batch=None, seed=333):
     return c, (Hi, Wi, Ho, Wo, nh, d), col, roff, w, k, v, q, dy
 
 
-def _hip(k, v, q, dy, w, col, roff, nh, dims):
+def _hip(k, v, q, dy, w, col, roff, nh, dims, saved=False):
     from torch_harmonics_amd import ops
 
     Hi, Wi, Ho, Wo = dims
     kd, vd, qd, gd, wd, cd, rd = [t.to(DEV) for t in (k, v, q, dy, w, col, roff)]
-    y = ops.forward(kd, vd, qd, wd, cd, rd, nh, Wi, Ho, Wo)
-    dk, dv, dq = ops.backward(kd, vd, qd, gd, wd, cd, rd, nh, Wi, Ho, Wo)
+    if saved:  # backward from the forward's saved output and softmax normaliser
+        y, lse = ops.forward_lse(kd, vd, qd, wd, cd, rd, nh, Wi, Ho, Wo)
+        dk, dv, dq = ops.backward_saved(kd, vd, qd, gd, y, lse, wd, cd, rd, nh, Wi, Ho, Wo)
+    else:
+        y = ops.forward(kd, vd, qd, wd, cd, rd, nh, Wi, Ho, Wo)
+        dk, dv, dq = ops.backward(kd, vd, qd, gd, wd, cd, rd, nh, Wi, Ho, Wo)
     torch.cuda.synchronize()
     return y, dk, dv, dq
 
@@ -53,11 +57,12 @@ def _check_rows(name, rows_fwd, band, k, v, q, dy, w, col, roff, nh, y, dk, dv, 
     return dk64, dv64
 
 
-def test_cfg3_sampled_rows_two_heads():
+@pytest.mark.parametrize("saved", [False, True], ids=["recompute", "saved"])
+def test_cfg3_sampled_rows_two_heads(saved):
     """721x1440 self-attention, head_dim 32, cutoff 3 spacings; two of the eight heads so the float64 check of the
     5760-neighbor pole rows stays within seconds (heads are independent in this op)."""
     c, (Hi, Wi, Ho, Wo, nh, d), col, roff, w, k, v, q, dy = _setup("cfg3", heads=2)
-    y, dk, dv, dq = _hip(k, v, q, dy, w, col, roff, nh, (Hi, Wi, Ho, Wo))
+    y, dk, dv, dq = _hip(k, v, q, dy, w, col, roff, nh, (Hi, Wi, Ho, Wo), saved=saved)
     # equator: rows 352..368 -> input latitudes 355..364 are complete (band half-height 3)
     dk64, dv64 = _check_rows("cfg3", [0, 1, 4, 360, 719, 720], (352, 369), k, v, q, dy, w, col, roff, nh, y, dk, dv, dq, 3)
     assert_close("cfg3 dk equator", dk[:, 355:365].cpu(), dk64[:, 355:365], **TOL)

@@ -152,6 +152,8 @@ def test_opcheck(nh):
     q = torch.randn(2, 6, 12, 8, device=DEV, requires_grad=True)
     args = (k, v, q, m.quad_weights, m.psi_col_idx, m.psi_roff_idx, nh, 24, 6, 12)
     torch.library.opcheck(ops._neighborhood_s2_attention_optimized, args)
+    torch.library.opcheck(ops._neighborhood_s2_attention_saved, args)
+    torch.library.opcheck(ops.forward_lse, tuple(a.detach() if isinstance(a, torch.Tensor) else a for a in args))
     torch.library.opcheck(ops.forward, tuple(a.detach() if isinstance(a, torch.Tensor) else a for a in args))
     x = torch.randn(2, 3, 4, 5, device=DEV, requires_grad=True)
     torch.library.opcheck(ops.permute_to_nhwc, (x,))

@@ -152,3 +152,53 @@ def test_reduced_precision_storage(dtype, tol):
     for name, got, want in (("y", y, y64), ("dk", dk, dk64), ("dv", dv, dv64), ("dq", dq, dq64)):
         rms = want.pow(2).mean().sqrt().item()
         assert_close(name, got, want, rtol=tol, atol=tol * rms)
+
+
+SAVED_CASES = [
+    # matrix-core domain (head dim 32, nlon >= 64): the backward consumes the saved output and normaliser
+    (1, 2, 32, 32, (24, 96), (24, 96), "equiangular", "equiangular", 0.5),
+    (2, 1, 32, 32, (16, 128), (16, 128), "legendre-gauss", "legendre-gauss", 0.9),
+    (1, 1, 32, 32, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
+    # outside it the saved tensors are ignored and the result must still be right
+    (1, 2, 16, 16, (16, 32), (16, 32), "equiangular", "equiangular", 0.4),
+    (1, 1, 48, 40, (12, 24), (6, 12), "equiangular", "equiangular", 0.6),
+]
+
+
+@pytest.mark.parametrize("case", SAVED_CASES, ids=lambda c: f"B{c[0]}h{c[1]}ck{c[2]}cv{c[3]}_{c[4][0]}x{c[4][1]}to{c[5][0]}x{c[5][1]}_{c[6][:3]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_backward_from_saved_forward_results(case, dtype):
+    """forward_lse + backward_saved against the fp64 oracle; lse against the oracle's dense softmax normaliser."""
+    from torch_harmonics_amd import ops
+
+    B, nh, ck, cv, ins, outs, gi, go, tc = case
+    print(f"case {case} {dtype}", flush=True)
+    col_idx, row_off, quad = _psi(ins, outs, gi, go, tc)
+    k, v, q, dy = randn_inputs(B, ins[0], ins[1], outs[0], outs[1], nh, ck, cv, scale=0.5 if dtype != torch.float32 else 1.0)
+    k, v, q, dy = [t.to(dtype).float() for t in (k, v, q, dy)]
+    dev = torch.device("cuda", 0)
+    kd, vd, qd, gd = [t.to(device=dev, dtype=dtype) for t in (k, v, q, dy)]
+    wd, cd, rd = quad.to(dev), col_idx.to(dev), row_off.to(dev)
+    geo = (nh, ins[1], outs[0], outs[1])
+    y, lse = ops.forward_lse(kd, vd, qd, wd, cd, rd, *geo)
+    assert torch.equal(y, ops.forward(kd, vd, qd, wd, cd, rd, *geo))
+    dk, dv, dq = ops.backward_saved(kd, vd, qd, gd, y, lse, wd, cd, rd, *geo)
+    torch.cuda.synchronize()
+
+    # normaliser: log2 sum_j exp(q.k_j) w_j from the dense fp64 restatement
+    mask = oracle.dense_mask(col_idx, row_off, ins[0], ins[1], outs[0], outs[1])  # [Ho*Wo, Hi*Wi] bool
+    kh = k.double().view(B, ins[0] * ins[1], nh, ck)
+    qh = q.double().view(B, outs[0] * outs[1], nh, ck)
+    logw = quad.double().log().view(-1, 1).expand(ins[0], ins[1]).reshape(-1)
+    s = (torch.einsum("bxhc,bihc->bhxi", qh, kh) + logw).masked_fill(~mask[None, None], float("-inf"))
+    want_lse = (torch.logsumexp(s, dim=-1) / math.log(2.0)).float().view(B, nh, outs[0], outs[1])
+    assert_close("lse", lse, want_lse, rtol=1e-5, atol=2e-5)
+
+    y64 = oracle.forward_f64(k, v, q, quad, col_idx, row_off, nh)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, quad, col_idx, row_off, nh)
+    for name, got, want in (("y", y, y64), ("dk", dk, dk64), ("dv", dv, dv64), ("dq", dq, dq64)):
+        if dtype == torch.float32:
+            assert_close(name, got, want, **F32_TOL)
+        else:
+            rms = want.pow(2).mean().sqrt().item()
+            assert_close(name, got, want, rtol=2e-2, atol=2e-2 * rms)

@@ -8,12 +8,13 @@ from . import _lib
 from ._layout import to_nchw, to_nhwc
 from .attention import NeighborhoodAttentionS2
 from .neighborhood import precompute_neighborhood_s2
-from .ops import _neighborhood_s2_attention_optimized
+from .ops import _neighborhood_s2_attention_optimized, neighborhood_s2_attention
 from .quadrature import precompute_latitudes, precompute_longitudes
 
 __all__ = [
     "NeighborhoodAttentionS2",
     "_neighborhood_s2_attention_optimized",
+    "neighborhood_s2_attention",
     "to_nhwc",
     "to_nchw",
     "precompute_neighborhood_s2",

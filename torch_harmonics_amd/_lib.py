@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -57,6 +57,9 @@ SYMBOLS = {
     "s2attn_plan_count": (_i64, [_vp, _vp, _i64, _int, _int, _int, _int]),
     "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_forward_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_backward_saved": (_int, [_vp] * 11 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_backward_dq_saved": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
     "s2attn_backward": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_dq": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),

@@ -17,7 +17,7 @@ import torch.nn.functional as F
 from ._attention_utils import _check_dtypes_match, _check_extent, _check_ndim
 from ._layout import to_nchw, to_nhwc
 from .neighborhood import precompute_neighborhood_s2
-from .ops import _neighborhood_s2_attention_optimized
+from .ops import neighborhood_s2_attention
 from .quadrature import precompute_latitudes
 
 __all__ = ["NeighborhoodAttentionS2"]
@@ -138,7 +138,7 @@ class NeighborhoodAttentionS2(nn.Module):
         else:
             self.q_norm_weights = self.k_norm_weights = None
 
-        self.attention_handle = _neighborhood_s2_attention_optimized
+        self.attention_handle = neighborhood_s2_attention
 
     def extra_repr(self):
         return (

@@ -40,7 +40,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 2; }
+extern "C" int s2attn_abi_version(void) { return 3; }
 
 namespace s2 {
 
@@ -218,6 +218,8 @@ struct Args {
     const void *k, *v, *q, *dy;
     void *y, *dk, *dv, *dq;
     float2 *stats; // per (batch, head, ho, wo): (log2-sum-exp of the scaled scores, sum_j p_j <dy, v_j>)
+    float *lse;    // forward, optional: log2-sum-exp per (batch, head, ho, wo); backward with saved statistics: the same array
+    const void *ysaved; // backward with saved statistics: the forward output
     const float *quad_w;
     const int *goff, *gorder, *soff, *sorder;
     const Run *gruns, *sruns;
@@ -317,6 +319,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd
         }
     }
 
+    if (a.lse && lane < nvalid) a.lse[((long)bh * a.Ho + ho) * a.Wo + wo0 + lane] = m + fast_log2(S);
     const float inv = 1.0f / S;
     __syncthreads();
 #pragma unroll
@@ -683,6 +686,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
             }
         }
     }
+    if (a.lse && qi < nvalid && sl == 0) a.lse[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = m + fast_log2(S);
     const float inv = 1.0f / S;
     __syncthreads();
 #pragma unroll
@@ -1049,6 +1053,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kern
         run = nrun;
     }
 
+    if (a.lse && lane < nvalid) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + lane] = m + fast_log2(S);
     const float inv = 1.0f / S;
 #pragma unroll
     for (int c = 0; c < P; c += 4)
@@ -1587,6 +1592,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     }
 
     if (mine) {
+        if (a.lse && half == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + j] = m + fast_log2(S);
         const float inv = 1.0f / S;
         T *y = static_cast<T *>(a.y) + pt * ldv + (size_t)h * 32 + 4 * half;
 #pragma unroll
@@ -1816,6 +1822,174 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
                                            (Akg[4 * g + 2] - I * Ak[4 * g + 2]) * inv, (Akg[4 * g + 3] - I * Ak[4 * g + 3]) * inv));
     }
 }
+
+// backward dq from saved forward statistics: with lse = log2 sum_j a_j known per query and I = <dy, y>, the softmax is
+// final from the first neighbor on, p_j = exp2(s_j - lse) w_j, and dq = sum_j p_j (g_j - I) k_j needs three matrix
+// products per tile (S^T, G^T, dQ^T += K^T C^T) and no running maximum or rescaling.
+template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel(const Args a)
+{
+    __shared__ __attribute__((aligned(16))) float Ks[MR * MLK];
+    __shared__ __attribute__((aligned(16))) float Vs[MR * MLK];
+
+    S2_MFMA_IDS(a.Wo)
+    const int ho = a.gorder[a.row_first + rowsel];
+    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
+    const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
+    const bool mine = j < nvalid;
+    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+    const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+
+    float qb[16], gb[16];
+    float I = 0.f;
+    {
+        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 4 * half;
+        const T *grow = static_cast<const T *>(a.dy) + pt * ldv + (size_t)h * 32 + 4 * half;
+        const T *yrow = static_cast<const T *>(a.ysaved) + pt * ldv + (size_t)h * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float4 x = load4(qrow + 8 * g);
+            const float4 z = load4(grow + 8 * g);
+            const float4 yv = load4(yrow + 8 * g);
+            qb[4 * g] = x.x * LOG2E, qb[4 * g + 1] = x.y * LOG2E, qb[4 * g + 2] = x.z * LOG2E, qb[4 * g + 3] = x.w * LOG2E;
+            gb[4 * g] = z.x, gb[4 * g + 1] = z.y, gb[4 * g + 2] = z.z, gb[4 * g + 3] = z.w;
+            I = fmaf(z.x, yv.x, I);
+            I = fmaf(z.y, yv.y, I);
+            I = fmaf(z.z, yv.z, I);
+            I = fmaf(z.w, yv.w, I);
+        }
+        I += __shfl_xor(I, 32);
+    }
+    const float lse = a.lse[sidx];
+    if (mine && half == 0) a.stats[sidx] = make_float2(lse, I);
+    f16v dqt;
+#pragma unroll
+    for (int v = 0; v < 16; v++) dqt[v] = 0.f;
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int pos = 0;
+    Run run = {0, 0, 0, 0};
+    Tile40<T> kt, vt;
+    auto fetch = [&](const Run &rn, int p) {
+        const int c0 = (rn.ws + w0 + p) % a.Wi;
+        const bool fifth = !run_is_dense(rn.len);
+        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane, fifth);
+        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane, fifth);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+        kt.commit(Ks, lane, !run_is_dense(run.len));
+        vt.commit(Vs, lane, !run_is_dense(run.len));
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const float w = a.quad_w[run.lat];
+        const int len = run.len;
+        int nri = ri, npos = pos + run_stride(len);
+        Run nrun = run;
+        if (run_done(len, npos)) {
+            nri++;
+            npos = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, npos);
+
+        const float *kq = Ks + j * MLK + 4 * half;
+        const float *vq = Vs + j * MLK + 4 * half;
+        if (run_is_dense(len)) {
+            const int u0 = pos;
+            f16v sc, gc;
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                sc[v] = 0.f;
+                gc[v] = 0.f;
+            }
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const float4 x = *reinterpret_cast<const float4 *>(kq + 8 * g);
+                const float4 z = *reinterpret_cast<const float4 *>(vq + 8 * g);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[4 * g + 0], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, gb[4 * g + 0], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[4 * g + 1], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, gb[4 * g + 1], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[4 * g + 2], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, gb[4 * g + 2], gc, 0, 0, 0);
+                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[4 * g + 3], sc, 0, 0, 0);
+                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, gb[4 * g + 3], gc, 0, 0, 0);
+            }
+            const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
+            if (edge) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    const int t = u0 + kappa(v, half) - j;
+                    const float p = (t >= 0 && t < len) ? fast_exp2(sc[v] - lse) * w : 0.f;
+                    sc[v] = p * (gc[v] - I);
+                }
+            } else {
+#pragma unroll
+                for (int v = 0; v < 16; v++) sc[v] = fast_exp2(sc[v] - lse) * w * (gc[v] - I);
+            }
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float x = Ks[kappa(v, half) * MLK + j];
+                dqt = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], dqt, 0, 0, 0);
+            }
+        } else {
+            const int L = min(VC, len - pos);
+#pragma unroll
+            for (int t = 0; t < VC; t++) {
+                if (t < L) {
+                    float4 xk[4];
+                    float ps_ = 0.f, pg_ = 0.f;
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        xk[g] = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
+                        const float4 z = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
+                        ps_ = fmaf(qb[4 * g], xk[g].x, ps_);
+                        ps_ = fmaf(qb[4 * g + 1], xk[g].y, ps_);
+                        ps_ = fmaf(qb[4 * g + 2], xk[g].z, ps_);
+                        ps_ = fmaf(qb[4 * g + 3], xk[g].w, ps_);
+                        pg_ = fmaf(gb[4 * g], z.x, pg_);
+                        pg_ = fmaf(gb[4 * g + 1], z.y, pg_);
+                        pg_ = fmaf(gb[4 * g + 2], z.z, pg_);
+                        pg_ = fmaf(gb[4 * g + 3], z.w, pg_);
+                    }
+                    const float sv = ps_ + __shfl_xor(ps_, 32);
+                    const float gv = pg_ + __shfl_xor(pg_, 32);
+                    const float coef = fast_exp2(sv - lse) * w * (gv - I);
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        dqt[4 * g] = fmaf(coef, xk[g].x, dqt[4 * g]);
+                        dqt[4 * g + 1] = fmaf(coef, xk[g].y, dqt[4 * g + 1]);
+                        dqt[4 * g + 2] = fmaf(coef, xk[g].z, dqt[4 * g + 2]);
+                        dqt[4 * g + 3] = fmaf(coef, xk[g].w, dqt[4 * g + 3]);
+                    }
+                }
+            }
+        }
+
+        __syncthreads();
+        if (more) {
+            kt.commit(Ks, lane, !run_is_dense(nrun.len));
+            vt.commit(Vs, lane, !run_is_dense(nrun.len));
+        }
+        __syncthreads();
+        ri = nri;
+        pos = npos;
+        run = nrun;
+    }
+
+    if (mine) {
+        T *dq = static_cast<T *>(a.dq) + pt * ldk + (size_t)h * 32 + 4 * half;
+#pragma unroll
+        for (int g = 0; g < 4; g++) store4(dq + 8 * g, make_float4(dqt[4 * g], dqt[4 * g + 1], dqt[4 * g + 2], dqt[4 * g + 3]));
+    }
+}
+
 
 // backward dk/dv: lane (j, half) owns INPUT longitude j of the tile, channels 8g + 4 half + e.  For a run (ho, ws, len)
 // the queries that see the tile's keys are the len + 31 longitudes starting at w0 - ws - len + 1; query row r sees key j
@@ -2156,7 +2330,7 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
         kern = fwd_mfma_kernel<T>;
         nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
     } else if (which == DQ) {
-        kern = dq_mfma_kernel<T>;
+        kern = (a.ysaved && a.lse) ? dq_saved_mfma_kernel<T> : dq_mfma_kernel<T>;
         nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
     } else {
         kern = dkdv_mfma_kernel<T>;
@@ -2219,8 +2393,17 @@ void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const f
 
 } // namespace
 
+extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, const float *quad_weights, void *y, float *lse,
+                                  const s2attn_plan *plan, const s2attn_shape *shape, void *stream);
+
 extern "C" int s2attn_forward(const void *k, const void *v, const void *q, const float *quad_weights, void *y,
                               const s2attn_plan *plan, const s2attn_shape *shape, void *stream)
+{
+    return s2attn_forward_lse(k, v, q, quad_weights, y, nullptr, plan, shape, stream);
+}
+
+extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, const float *quad_weights, void *y, float *lse,
+                                  const s2attn_plan *plan, const s2attn_shape *shape, void *stream)
 {
     int rc = check_shape(shape);
     if (rc != S2ATTN_OK) return rc;
@@ -2230,6 +2413,7 @@ extern "C" int s2attn_forward(const void *k, const void *v, const void *q, const
     Args a = {};
     fill_args(a, plan, shape, quad_weights);
     a.k = k, a.v = v, a.q = q, a.y = y;
+    a.lse = lse;
     a.tile_rows = a.pscale * (TQ - 1) + TL;
     const size_t al = 4 * (size_t)esize(shape->dtype);
     const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(y, al);
@@ -2277,6 +2461,24 @@ extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, c
     return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
 }
 
+extern "C" int s2attn_backward_dq_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
+                                        const float *quad_weights, void *dq, void *workspace, const s2attn_plan *plan,
+                                        const s2attn_shape *shape, void *stream)
+{
+    Args a = {};
+    bool vec = false;
+    const int rc = backward_args(a, vec, k, v, q, dy, quad_weights, workspace, plan, shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!dq || !y || !lse) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    a.dq = dq;
+    a.ysaved = y;
+    a.lse = const_cast<float *>(lse);
+    const size_t al = 4 * (size_t)esize(shape->dtype);
+    vec = vec && aligned(dq, al) && aligned(y, al);
+    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
+}
+
 extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
                                     void *dk, void *dv, const void *workspace, const s2attn_plan *plan,
                                     const s2attn_shape *shape, void *stream)
@@ -2292,6 +2494,16 @@ extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q,
     a.tile_rows = (TQ - 1) / a.pscale + 1 + TL;
     if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile also stages the lane-owned k/v and dk/dv rows
     return launch(DKDV, a, shape->dtype, vec, plan->scatter_ndense, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2attn_backward_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
+                                     const float *quad_weights, void *dk, void *dv, void *dq, void *workspace, const s2attn_plan *plan,
+                                     const s2attn_shape *shape, void *stream)
+{
+    if (!dk || !dv || !dq) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    const int rc = s2attn_backward_dq_saved(k, v, q, dy, y, lse, quad_weights, dq, workspace, plan, shape, stream);
+    if (rc != S2ATTN_OK) return rc;
+    return s2attn_backward_dkdv(k, v, q, dy, quad_weights, dk, dv, workspace, plan, shape, stream);
 }
 
 extern "C" int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,

@@ -83,6 +83,36 @@ def _shape_struct(kx, vx, qy, num_heads) -> _lib.ShapeStruct:
     return _lib.ShapeStruct(B, num_heads, Hi, Wi, Ho, Wo, CK // num_heads, vx.shape[3] // num_heads, _DTYPE_CODE[qy.dtype])
 
 
+def _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, with_lse):
+    _validate(kx, vx, qy, None, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
+    for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
+        _require_gpu(t, name)
+    if qy.dtype == torch.float64:  # stored as fp64, computed in fp32 like the reference (attention_cuda_utils.cuh:185-190)
+        y, lse = _forward_impl(kx.float(), vx.float(), qy.float(), quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, with_lse)
+        return y.double(), lse
+    y = torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
+    lse = torch.empty((kx.shape[0], num_heads, nlat_out, nlon_out) if with_lse else (0,), dtype=torch.float32, device=kx.device)
+    if y.numel() == 0:
+        return y, lse
+    plan = get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out)
+    shape = _shape_struct(kx, vx, qy, num_heads)
+    qw = quad_weights.to(dtype=torch.float32).contiguous()
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_forward_lse(
+            kx.data_ptr(),
+            vx.data_ptr(),
+            qy.data_ptr(),
+            qw.data_ptr(),
+            y.data_ptr(),
+            lse.data_ptr() if with_lse else None,
+            ctypes.byref(plan.struct),
+            ctypes.byref(shape),
+            _stream_ptr(kx.device),
+        )
+    _lib.check(rc, "s2attn_forward_lse")
+    return y, lse
+
+
 @torch.library.custom_op("s2attn::forward", mutates_args=())
 def forward(
     kx: torch.Tensor,
@@ -96,28 +126,73 @@ def forward(
     nlat_out: int,
     nlon_out: int,
 ) -> torch.Tensor:
-    _validate(kx, vx, qy, None, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-    for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
-        _require_gpu(t, name)
-    if qy.dtype == torch.float64:  # stored as fp64, computed in fp32 like the reference (attention_cuda_utils.cuh:185-190)
-        return forward(kx.float(), vx.float(), qy.float(), quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out).double()
-    y = torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
-    if y.numel() == 0:
-        return y
-    plan = get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out)
-    shape = _shape_struct(kx, vx, qy, num_heads)
-    qw = quad_weights.to(dtype=torch.float32).contiguous()
-    with torch.cuda.device(kx.device):
-        rc = _lib.load().s2attn_forward(
-            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), qw.data_ptr(), y.data_ptr(), ctypes.byref(plan.struct), ctypes.byref(shape), _stream_ptr(kx.device)
-        )
-    _lib.check(rc, "s2attn_forward")
-    return y
+    return _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, False)[0]
 
 
 @forward.register_fake
 def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
     return torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
+
+
+@torch.library.custom_op("s2attn::forward_lse", mutates_args=())
+def forward_lse(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    num_heads: int,
+    nlon_in: int,
+    nlat_out: int,
+    nlon_out: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    """forward plus the fp32 log2-domain softmax normaliser [B, num_heads, nlat_out, nlon_out] that backward_saved takes."""
+    return _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, True)
+
+
+@forward_lse.register_fake
+def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
+    y = torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
+    return y, torch.empty((kx.shape[0], num_heads, nlat_out, nlon_out), dtype=torch.float32, device=kx.device)
+
+
+def _backward_impl(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
+    _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
+    for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("dy", dy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
+        _require_gpu(t, name)
+    saved = y is not None
+    if saved:
+        _require_gpu(y, "y")
+        _require_gpu(lse, "lse")
+        if y.shape != dy.shape or y.dtype != dy.dtype or not y.is_contiguous():
+            raise RuntimeError("y must be the contiguous forward output (shape and dtype of dy)")
+        if lse.shape != (kx.shape[0], num_heads, nlat_out, nlon_out) or lse.dtype != torch.float32 or not lse.is_contiguous():
+            raise RuntimeError("lse must be the contiguous fp32 (B, num_heads, nlat_out, nlon_out) tensor returned by forward_lse")
+    if qy.dtype == torch.float64:
+        dk, dv, dq = _backward_impl(
+            kx.float(), vx.float(), qy.float(), dy.float(), y.float() if saved else None, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out
+        )
+        return dk.double(), dv.double(), dq.double()
+    dk, dv, dq = torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
+    if qy.numel() == 0 or kx.numel() == 0:
+        return dk.zero_(), dv.zero_(), dq.zero_()
+    plan = get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out)
+    shape = _shape_struct(kx, vx, qy, num_heads)
+    lib = _lib.load()
+    nbytes = lib.s2attn_backward_workspace_bytes(ctypes.byref(shape))
+    _lib.check(nbytes, "s2attn_backward_workspace_bytes")
+    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=kx.device)
+    qw = quad_weights.to(dtype=torch.float32).contiguous()
+    head = (kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr())
+    tail = (qw.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), workspace.data_ptr(), ctypes.byref(plan.struct), ctypes.byref(shape), _stream_ptr(kx.device))
+    with torch.cuda.device(kx.device):
+        if saved:
+            rc = lib.s2attn_backward_saved(*head, y.data_ptr(), lse.data_ptr(), *tail)
+        else:
+            rc = lib.s2attn_backward(*head, *tail)
+    _lib.check(rc, "s2attn_backward_saved" if saved else "s2attn_backward")
+    return dk, dv, dq
 
 
 @torch.library.custom_op("s2attn::backward", mutates_args=())
@@ -134,43 +209,36 @@ def backward(
     nlat_out: int,
     nlon_out: int,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-    for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("dy", dy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
-        _require_gpu(t, name)
-    if qy.dtype == torch.float64:
-        dk, dv, dq = backward(kx.float(), vx.float(), qy.float(), dy.float(), quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-        return dk.double(), dv.double(), dq.double()
-    dk, dv, dq = torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
-    if qy.numel() == 0 or kx.numel() == 0:
-        return dk.zero_(), dv.zero_(), dq.zero_()
-    plan = get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out)
-    shape = _shape_struct(kx, vx, qy, num_heads)
-    lib = _lib.load()
-    nbytes = lib.s2attn_backward_workspace_bytes(ctypes.byref(shape))
-    _lib.check(nbytes, "s2attn_backward_workspace_bytes")
-    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=kx.device)
-    qw = quad_weights.to(dtype=torch.float32).contiguous()
-    with torch.cuda.device(kx.device):
-        rc = lib.s2attn_backward(
-            kx.data_ptr(),
-            vx.data_ptr(),
-            qy.data_ptr(),
-            dy.data_ptr(),
-            qw.data_ptr(),
-            dk.data_ptr(),
-            dv.data_ptr(),
-            dq.data_ptr(),
-            workspace.data_ptr(),
-            ctypes.byref(plan.struct),
-            ctypes.byref(shape),
-            _stream_ptr(kx.device),
-        )
-    _lib.check(rc, "s2attn_backward")
-    return dk, dv, dq
+    return _backward_impl(kx, vx, qy, dy, None, None, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
 
 
 @backward.register_fake
 def _(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
+    return torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
+
+
+@torch.library.custom_op("s2attn::backward_saved", mutates_args=())
+def backward_saved(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    dy: torch.Tensor,
+    y: torch.Tensor,
+    lse: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    num_heads: int,
+    nlon_in: int,
+    nlat_out: int,
+    nlon_out: int,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """backward with the (y, lse) pair of forward_lse, so that the softmax statistics are not recomputed."""
+    return _backward_impl(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
+
+
+@backward_saved.register_fake
+def _(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
     return torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
 
 
@@ -264,6 +332,53 @@ def _neighborhood_s2_attention_bwd_optimized(ctx, grad_output):
 _neighborhood_s2_attention_optimized.register_autograd(_neighborhood_s2_attention_bwd_optimized, setup_context=_setup_context_attention_backward)
 
 
+# Same op, but the forward also hands its output and softmax normaliser to the backward (the reference recomputes both,
+# attention_cuda_bwd.cu:856-956).  Two outputs, so it cannot carry the reference's one-tensor signature; the module
+# calls it through neighborhood_s2_attention below.
+@torch.library.custom_op("s2attn::_neighborhood_s2_attention_saved", mutates_args=())
+def _neighborhood_s2_attention_saved(
+    kw: torch.Tensor,
+    vw: torch.Tensor,
+    qw: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    nh: int,
+    nlon_in: int,
+    nlat_out: int,
+    nlon_out: int,
+) -> Tuple[torch.Tensor, torch.Tensor]:
+    return forward_lse(kw.contiguous(), vw.contiguous(), qw.contiguous(), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out)
+
+
+@_neighborhood_s2_attention_saved.register_fake
+def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
+    y = torch.empty((kw.shape[0], nlat_out, nlon_out, vw.shape[3]), dtype=kw.dtype, device=kw.device)
+    return y, torch.empty((kw.shape[0], nh, nlat_out, nlon_out), dtype=torch.float32, device=kw.device)
+
+
+def _setup_context_saved(ctx, inputs, output):
+    _setup_context_attention_backward(ctx, inputs, output)
+    ctx.y, ctx.lse = output[0].detach(), output[1].detach()
+    ctx.mark_non_differentiable(output[1])
+
+
+def _neighborhood_s2_attention_bwd_saved(ctx, grad_output, grad_lse):
+    col_idx, row_off, quad_weights, kw, vw, qw = ctx.saved_tensors
+    dkw, dvw, dqw = backward_saved(
+        kw.contiguous(), vw.contiguous(), qw.contiguous(), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in, ctx.nlat_out, ctx.nlon_out
+    )
+    return dkw, dvw, dqw, None, None, None, None, None, None, None
+
+
+_neighborhood_s2_attention_saved.register_autograd(_neighborhood_s2_attention_bwd_saved, setup_context=_setup_context_saved)
+
+
+def neighborhood_s2_attention(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
+    """Differentiable attention on NHWC heads-packed tensors; what NeighborhoodAttentionS2.forward calls."""
+    return _neighborhood_s2_attention_saved(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out)[0]
+
+
 # Autocast: k, v, q are brought to the active autocast dtype and the op re-entered with autocast off;
 # quad_weights and the index tensors pass through (attention_optimized.py:310-322).
 def _make_autocast_impl(device_type: str):
@@ -276,5 +391,16 @@ def _make_autocast_impl(device_type: str):
     return _
 
 
-_make_autocast_impl("cuda")
-_make_autocast_impl("cpu")
+def _make_autocast_impl_saved(device_type: str):
+    @torch.library.impl("s2attn::_neighborhood_s2_attention_saved", f"Autocast{device_type.upper()}")
+    def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
+        cast_dtype = torch.get_autocast_dtype(device_type)
+        with torch.amp.autocast(device_type, enabled=False):
+            return _neighborhood_s2_attention_saved(kw.to(cast_dtype), vw.to(cast_dtype), qw.to(cast_dtype), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out)
+
+    return _
+
+
+for _device_type in ("cuda", "cpu"):
+    _make_autocast_impl(_device_type)
+    _make_autocast_impl_saved(_device_type)
