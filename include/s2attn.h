@@ -155,7 +155,7 @@ int s2attn_backward_dq_saved(const void *k, const void *v, const void *q, const 
 /*
  * Layout conversion.  Replace attention_kernels::permute_to_nhwc / permute_to_nchw
  * (attention_interface.cpp:85-86; CUDA kernels attention_cuda_utils.cuh:417-576).
- * Pure element moves; elem_size is 2 or 4 bytes.  dst must not alias src.
+ * Pure element moves; elem_size is 2, 4 or 8 bytes.  dst must not alias src.
  *   to_nhwc: src [B, C, H, W] -> dst [B, H, W, C]
  *   to_nchw: src [B, H, W, C] -> dst [B, C, H, W]
  */
