@@ -162,11 +162,17 @@ SAVED_CASES = [
     # outside it the saved tensors are ignored and the result must still be right
     (1, 2, 16, 16, (16, 32), (16, 32), "equiangular", "equiangular", 0.4),
     (1, 1, 48, 40, (12, 24), (6, 12), "equiangular", "equiangular", 0.6),
+    # head dim 64: with 16-bit storage the 16-bit matrix-core kernels (16-longitude tiles, nlon >= 32); ragged last tile,
+    # full-circle runs longer than the grid is wide minus a tile, several heads and batches
+    (1, 2, 64, 64, (16, 48), (16, 48), "legendre-gauss", "legendre-gauss", 0.4),
+    (2, 1, 64, 64, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
+    (1, 1, 64, 64, (8, 40), (8, 40), "equiangular", "equiangular", 7.0),
+    (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
 ]
 
 
 @pytest.mark.parametrize("case", SAVED_CASES, ids=lambda c: f"B{c[0]}h{c[1]}ck{c[2]}cv{c[3]}_{c[4][0]}x{c[4][1]}to{c[5][0]}x{c[5][1]}_{c[6][:3]}")
-@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "fp16"])
 def test_backward_from_saved_forward_results(case, dtype):
     """forward_lse + backward_saved against the fp64 oracle; lse against the oracle's dense softmax normaliser."""
     from torch_harmonics_amd import ops

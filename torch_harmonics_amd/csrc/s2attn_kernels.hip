@@ -22,6 +22,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <type_traits>
 
 #include "s2attn_internal.h"
 
@@ -2182,6 +2183,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     }
 }
 
+#include "s2attn_h16.hpp"
+
 // ---------------------------------------------------------------------------------
 // layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
 // ---------------------------------------------------------------------------------
@@ -2343,6 +2346,46 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
     return S2ATTN_OK;
 }
 
+// 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
+// dq pass exists only in the form that takes the forward's y and lse.
+template <typename T, int D> int launch_h16(Which which, const Args &a0, hipStream_t stream)
+{
+    if constexpr (std::is_same<T, float>::value) {
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "16-bit kernels asked for fp32 storage");
+    } else {
+        Args a = a0;
+        a.row_first = 0;
+        void (*kern)(const Args) = nullptr;
+        long nblocks = 0;
+        if (which == FWD) {
+            kern = fwd_h16_kernel<T, D>;
+            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+        } else if (which == DQ) {
+            kern = dq_h16_kernel<T, D>;
+            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+        } else {
+            kern = dkdv_h16_kernel<T, D>;
+            nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
+        }
+        if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+        return S2ATTN_OK;
+    }
+}
+
+template <typename T> bool h16_ok(Which which, const Args &a)
+{
+    if (std::is_same<T, float>::value) return false;
+    if (a.pscale != 1 || a.dk_ != a.dv_ || a.dk_ != 64 || a.Wi < HK) return false;
+    if (which == DQ && !(a.ysaved && a.lse)) return false;
+    const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
+    for (const void *p : ptrs)
+        if (p && !aligned(p, 16)) return false;
+    return true;
+}
+
 bool dense_ok(Which which, const Args &a, bool vec)
 {
     (void)which;
@@ -2353,6 +2396,7 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
 {
     const int nrows = which == DKDV ? a.Hi : a.Ho;
     int first = 0;
+    if (h16_ok<T>(which, a)) return launch_h16<T, 64>(which, a, stream);
     if (dense_ok(which, a, vec)) {
         // the dense kernels handle short runs themselves (vector path inside), so they take every latitude
         (void)ndense;
