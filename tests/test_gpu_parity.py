@@ -168,6 +168,7 @@ SAVED_CASES = [
     (2, 1, 64, 64, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
     (1, 1, 64, 64, (8, 40), (8, 40), "equiangular", "equiangular", 7.0),
     (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
+    (1, 1, 128, 128, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
 ]
 
 

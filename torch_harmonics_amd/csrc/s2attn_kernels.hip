@@ -2378,7 +2378,7 @@ template <typename T, int D> int launch_h16(Which which, const Args &a0, hipStre
 template <typename T> bool h16_ok(Which which, const Args &a)
 {
     if (std::is_same<T, float>::value) return false;
-    if (a.pscale != 1 || a.dk_ != a.dv_ || a.dk_ != 64 || a.Wi < HK) return false;
+    if (a.pscale != 1 || a.dk_ != a.dv_ || (a.dk_ != 32 && a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
     if (which == DQ && !(a.ysaved && a.lse)) return false;
     const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
     for (const void *p : ptrs)
@@ -2396,7 +2396,11 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
 {
     const int nrows = which == DKDV ? a.Hi : a.Ho;
     int first = 0;
-    if (h16_ok<T>(which, a)) return launch_h16<T, 64>(which, a, stream);
+    if (h16_ok<T>(which, a)) {
+        if (a.dk_ == 32) return launch_h16<T, 32>(which, a, stream);
+        if (a.dk_ == 64) return launch_h16<T, 64>(which, a, stream);
+        return launch_h16<T, 128>(which, a, stream);
+    }
     if (dense_ok(which, a, vec)) {
         // the dense kernels handle short runs themselves (vector path inside), so they take every latitude
         (void)ndense;
@@ -2464,11 +2468,26 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     return launch(FWD, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
 }
 
+namespace {
+// Shapes of the 16-bit matrix-core kernels.  Their dq pass consumes the forward's output and normaliser; a backward
+// that is not handed them (s2attn_backward, s2attn_backward_dq) first recomputes both into the tail of the workspace.
+bool h16_shape(const s2attn_shape *sh)
+{
+    return sh->dtype != S2ATTN_F32 && sh->ck == sh->cv && (sh->ck == 32 || sh->ck == 64 || sh->ck == 128) && sh->nlon_in == sh->nlon_out
+        && sh->nlon_in >= HK;
+}
+int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
+int64_t round16(int64_t n) { return (n + 15) / 16 * 16; }
+} // namespace
+
 extern "C" int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape)
 {
     const int rc = check_shape(shape);
     if (rc != S2ATTN_OK) return rc;
-    return (int64_t)shape->batch * shape->num_heads * shape->nlat_out * shape->nlon_out * (int64_t)sizeof(float2);
+    const int64_t n = stat_points(shape);
+    int64_t bytes = round16(n * (int64_t)sizeof(float2));
+    if (h16_shape(shape)) bytes += round16(n * 4) + n * shape->cv * 2; // lse, y
+    return bytes;
 }
 
 namespace {
@@ -2502,6 +2521,17 @@ extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, c
     a.dq = dq;
     vec = vec && aligned(dq, 4 * (size_t)esize(shape->dtype));
     a.tile_rows = a.pscale * (TQ - 1) + TL;
+    if (h16_shape(shape) && aligned(workspace, 16)) {
+        const int64_t n = stat_points(shape);
+        char *ws = static_cast<char *>(workspace);
+        float *lse = reinterpret_cast<float *>(ws + round16(n * (int64_t)sizeof(float2)));
+        void *y = ws + round16(n * (int64_t)sizeof(float2)) + round16(n * 4);
+        Args f = a;
+        f.y = y, f.lse = lse, f.dq = nullptr, f.dy = nullptr;
+        const int rc2 = launch(FWD, f, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
+        if (rc2 != S2ATTN_OK) return rc2;
+        a.ysaved = y, a.lse = lse;
+    }
     return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
 }
 
