@@ -47,22 +47,28 @@ int s2attn_abi_version(void);
  * attention_cuda_bwd.cu:792).  This library instead converts the CSR once, on the
  * host, into runs of consecutive longitudes:
  *
- *   run = (lat, ws, len, 0)   four int32
+ *   run = (lat, ws, len, aux)   four int32
  *
- * gather runs   grouped by output latitude ho:  lat = hi, neighbors (hi, (ws + t + pscale*wo) mod nlon_in), t in [0, len)
- * scatter runs  the same runs grouped by input latitude hi: lat = ho
+ * With ps = nlon_in / nlon_out > 1 query column wo sees input columns ws + t + ps * wo.  The plan removes that stride:
+ * input latitude hi is split into ps "virtual latitudes" hi * ps + par, the columns {par, par + ps, ...}, each with
+ * nlon_out columns, and every CSR run into one run per column class it touches.  On virtual latitudes the
+ * neighborhood has unit stride in wo for any ps, and that is the only form the kernels implement.  (ps = 1: virtual
+ * and real latitudes coincide.)
+ *
+ * gather runs   grouped by output latitude ho:  lat = virtual input latitude, aux = real input latitude;
+ *               neighbors are its columns (ws + t + wo) mod nlon_out, t in [0, len)
+ * scatter runs  the same runs grouped by virtual input latitude: lat = ho, aux = 0
  *
  * plus, for each grouping, the group offsets and a launch order of the groups.  The order lists first the
- * latitudes whose runs are long enough for the dense matrix-core kernels (ndense of them, most work first) and
- * then the others for the vector kernels (most work first); starting the longest latitudes first is the load
- * balancing for the ~200:1 spread of row lengths between the poles and the equator.
- * Any CSR is representable (worst case every entry is its own run).
+ * latitudes whose runs are long (ndense of them, most work first) and then the others (most work first); starting
+ * the longest latitudes first is the load balancing for the ~200:1 spread of row lengths between the poles and
+ * the equator.  Any CSR is representable (worst case every entry is its own run).
  *
  * s2attn_plan_count   number of runs the CSR decomposes into, or a negative error.
  * s2attn_plan_build   fills caller-allocated host arrays:
- *     gather_off  [nlat_out+1]   gather_runs  [4*nruns]   gather_order  [nlat_out]
- *     scatter_off [nlat_in+1]    scatter_runs [4*nruns]   scatter_order [nlat_in]
- *     ndense [2]  number of dense latitudes at the front of gather_order and of scatter_order
+ *     gather_off  [nlat_out+1]      gather_runs  [4*nruns]   gather_order  [nlat_out]
+ *     scatter_off [nlat_in*ps+1]    scatter_runs [4*nruns]   scatter_order [nlat_in*ps]
+ *     ndense [2]  number of long-run latitudes at the front of gather_order and of scatter_order
  * The caller copies the six arrays to the device and passes them, with the two counts, in s2attn_plan.
  */
 int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
@@ -77,9 +83,9 @@ typedef struct s2attn_plan {
     const int32_t *gather_off;    /* device, [nlat_out+1] */
     const int32_t *gather_runs;   /* device, [4*nruns]    */
     const int32_t *gather_order;  /* device, [nlat_out]   */
-    const int32_t *scatter_off;   /* device, [nlat_in+1]  (backward only) */
-    const int32_t *scatter_runs;  /* device, [4*nruns]    (backward only) */
-    const int32_t *scatter_order; /* device, [nlat_in]    (backward only) */
+    const int32_t *scatter_off;   /* device, [nlat_in*ps+1]  (backward only) */
+    const int32_t *scatter_runs;  /* device, [4*nruns]       (backward only) */
+    const int32_t *scatter_order; /* device, [nlat_in*ps]    (backward only) */
     int64_t nruns;
     int32_t gather_ndense;  /* leading entries of gather_order that go to the dense kernels  */
     int32_t scatter_ndense; /* leading entries of scatter_order that go to the dense kernels */

@@ -70,27 +70,25 @@ def _pairs_from_csr(col, roff, Wi, Wo):
 
 
 def _pairs_from_plan(arrays, Hi, Wi, Ho, Wo):
-    """Expands both run groupings back into (ho, wo, hi, wi) pairs the way the kernels index them."""
+    """Expands both run groupings back into (ho, wo, hi, wi) pairs the way the kernels index them: runs live on
+    virtual input latitudes hi * ps + par (the columns par, par + ps, ... of latitude hi, Wo of them), where query
+    column wo sees virtual columns (ws + t + wo) mod Wo."""
     goff, gruns, gorder, soff, sruns, sorder = [a.numpy() for a in arrays]
     ps = Wi // Wo
     gather, scatter = Counter(), Counter()
     for ho in range(Ho):
         for ri in range(goff[ho], goff[ho + 1]):
-            hi, ws, ln, _ = (int(x) for x in gruns[ri])
+            vlat, ws, ln, hi = (int(x) for x in gruns[ri])
+            assert hi == vlat // ps and 0 <= ws < Wo and 1 <= ln <= Wo
             for wo in range(Wo):
                 for t in range(ln):
-                    gather[(ho, wo, hi, (ws + t + ps * wo) % Wi)] += 1
-    for hi in range(Hi):
-        for ri in range(soff[hi], soff[hi + 1]):
+                    gather[(ho, wo, hi, ((ws + t + wo) % Wo) * ps + vlat % ps)] += 1
+    for vlat in range(Hi * ps):
+        for ri in range(soff[vlat], soff[vlat + 1]):
             ho, ws, ln, _ = (int(x) for x in sruns[ri])
-            for wi in range(Wi):
-                delta = (wi - ws) % Wi
-                t = delta % ps
-                u = 0
-                while t < ln:
-                    scatter[(ho, (delta // ps - u) % Wo, hi, wi)] += 1
-                    u += 1
-                    t += ps
+            for j in range(Wo):  # virtual column j of this virtual latitude is seen by wo = j - ws - t
+                for t in range(ln):
+                    scatter[(ho, (j - ws - t) % Wo, vlat // ps, j * ps + vlat % ps)] += 1
     return gather, scatter, gorder, sorder
 
 
@@ -111,7 +109,7 @@ def test_plan_covers_exactly_the_csr_pairs(ins, outs, gi, go, tc):
     ref = _pairs_from_csr(col, roff, ins[1], outs[1])
     gather, scatter, gorder, sorder = _pairs_from_plan(arrays, ins[0], ins[1], outs[0], outs[1])
     assert gather == ref and scatter == ref
-    assert sorted(gorder.tolist()) == list(range(outs[0])) and sorted(sorder.tolist()) == list(range(ins[0]))
+    assert sorted(gorder.tolist()) == list(range(outs[0])) and sorted(sorder.tolist()) == list(range(ins[0] * (ins[1] // outs[1])))
     lens = (roff[1:] - roff[:-1]).tolist()
     assert all(lens[gorder[i]] >= lens[gorder[i + 1]] for i in range(outs[0] - 1)), "rows must be ordered longest first"
     assert nruns <= col.numel()
@@ -135,7 +133,7 @@ def test_plan_merges_wrapping_intervals_into_one_circular_run():
     roff = torch.tensor([0, 7])
     arrays, nruns, ndense = build_host_plan(col, roff, 2, Wi, 1, Wi)
     assert nruns == 2
-    assert arrays[1][:2].tolist() == [[0, 14, 5, 0], [1, 5, 2, 0]]
+    assert arrays[1][:2].tolist() == [[0, 14, 5, 0], [1, 5, 2, 1]]
 
 
 def test_plan_builder_rejects_malformed_csr():

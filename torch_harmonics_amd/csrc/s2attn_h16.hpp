@@ -70,15 +70,20 @@ template <int D> struct HTile {
     static constexpr int NIT = HK / RPI;     // iterations
     static constexpr int PITCH = 2 * D + 16; // bytes; 16-byte reads of 8 consecutive rows fall in distinct banks
     u4v raw[NIT];
-    __device__ inline void fetch(const char *src, unsigned ldb, int c0, int W, int lane)
+    // Byte offsets of this lane's pieces inside one latitude of one (batch, head) slice; the same for every tensor of
+    // a step (k and v, or q and dy).  lane_off = (lane / CPR) * ldb + 16 * (lane % CPR).
+    static __device__ inline void offsets(unsigned (&off)[NIT], unsigned lane_off, int lane, int c0, int W, unsigned ldb)
     {
-        const int r0 = lane / CPR, cb = 16 * (lane % CPR);
+        const int r0 = lane / CPR;
+        const int lim = W - c0; // staged rows from lim on wrap around the circle
+        const unsigned base = (unsigned)c0 * ldb + lane_off;
 #pragma unroll
-        for (int it = 0; it < NIT; it++) {
-            int col = c0 + r0 + it * RPI;
-            col -= (col >= W) ? W : 0;
-            raw[it] = *reinterpret_cast<const u4v *>(src + (size_t)col * ldb + cb);
-        }
+        for (int it = 0; it < NIT; it++) off[it] = base + (unsigned)(it * RPI) * ldb - ((r0 >= lim - it * RPI) ? (unsigned)W * ldb : 0u);
+    }
+    __device__ inline void fetch(const char *src, const unsigned (&off)[NIT])
+    {
+#pragma unroll
+        for (int it = 0; it < NIT; it++) raw[it] = *reinterpret_cast<const u4v *>(src + off[it]);
     }
     __device__ inline void commit(char *dst, int lane) const
     {
@@ -180,10 +185,15 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
     int pos = 0;
     Run run = {0, 0, 0, 0};
     Tile kt, vt;
+    const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldb, ldb, c0, a.Wi, lane);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldb, ldb, c0, a.Wi, lane);
+        unsigned off[Tile::NIT];
+        Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
+        const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
+        kt.fetch(kx + lat_off, off);
+        vt.fetch(vx + lat_off, off);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -194,7 +204,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
     __syncthreads();
 
     while (ri < rend) {
-        const float lw = fast_log2(a.quad_w[run.lat]);
+        const float lw = fast_log2(a.quad_w[run.pad]);
         const int len = run.len;
         int nri = ri, npos = pos + HK;
         Run nrun = run;
@@ -213,20 +223,20 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
 #pragma unroll
             for (int s = 0; s < NS; s++) sc[kb] = M::mfma(h16_read_row<PITCH>(Ks, kb, s, c, qd), qop[s], sc[kb]);
         }
+        // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
         const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
-        float mx = NEG_BIG;
+        float mx = -INFINITY;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 const unsigned t = (unsigned)(tb + 16 * kb + v);
-                const float x = (t < (unsigned)len) ? fmaf(sc[kb][v], LOG2E, lw) : NEG_BIG;
-                sc[kb][v] = x;
-                mx = fmaxf(mx, x);
+                sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
+                mx = fmaxf(mx, sc[kb][v]);
             }
         }
         mx = h16_quarter_max(mx);
-        const float mn = fmaxf(m, mx);
+        const float mn = fmaxf(m, fmaf(mx, LOG2E, lw)); // m starts finite, so mn is finite
         if (__any(mn > m)) {
             const float corr = fast_exp2(m - mn);
             S *= corr;
@@ -234,17 +244,16 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
             for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
         }
         m = mn;
-        float rs = 0.f;
+        const float sh = lw - mn;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float p = (sc[kb][v] == NEG_BIG) ? 0.f : fast_exp2(sc[kb][v] - mn);
+                const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // masked: exp2(-inf) = 0
                 sc[kb][v] = p;
-                rs += p;
+                S += p; // this lane's share; the four lanes of a column are added up at the end
             }
         }
-        S += h16_quarter_sum(rs);
         const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++) acc[cb] = M::mfma(h16_read_transposed<PITCH>(Vs, cb, c, qd), pop, acc[cb]);
@@ -260,6 +269,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
         run = nrun;
     }
 
+    S = h16_quarter_sum(S);
     if (mine) {
         if (a.lse && qd == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + c] = m + fast_log2(S);
         const float inv = 1.0f / S;
@@ -320,10 +330,15 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
     int pos = 0;
     Run run = {0, 0, 0, 0};
     Tile kt, vt;
+    const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldb, ldb, c0, a.Wi, lane);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldb, ldb, c0, a.Wi, lane);
+        unsigned off[Tile::NIT];
+        Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
+        const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
+        kt.fetch(kx + lat_off, off);
+        vt.fetch(vx + lat_off, off);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -334,7 +349,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
     __syncthreads();
 
     while (ri < rend) {
-        const float lwl = fast_log2(a.quad_w[run.lat]) - lse;
+        const float lwl = fast_log2(a.quad_w[run.pad]) - lse;
         const int len = run.len;
         int nri = ri, npos = pos + HK;
         Run nrun = run;
@@ -411,7 +426,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
     const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 2);
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = c < nvalid;
-    const size_t pt = (size_t)(b * a.Hi + hi) * a.Wi + w0 + (mine ? c : 0);
+    const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? c : 0)) * a.kps;
 
     uint4 kop[NS], vop[NS]; // B operands: channels 32 s + 8 qd .. + 8 of key c
     {
@@ -428,7 +443,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
         dkt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
         dvt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
     }
-    const float lw = fast_log2(a.quad_w[hi]);
+    const float lw = fast_log2(a.quad_w[hi / a.kps]);
 
     int ri = a.soff[hi];
     const int rend = a.soff[hi + 1];
@@ -436,11 +451,15 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
     Run run = {0, 0, 0, 0};
     Tile qt, gt;
     float2 st = make_float2(0.f, 0.f);
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldb + 16u * (lane % Tile::CPR);
     auto fetch = [&](const Run &rn, int p) {
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
-        qt.fetch(qy + (size_t)rn.lat * a.Wo * ldb, ldb, c0, a.Wo, lane);
-        gt.fetch(gy + (size_t)rn.lat * a.Wo * ldb, ldb, c0, a.Wo, lane);
+        unsigned off[Tile::NIT];
+        Tile::offsets(off, lane_off, lane, c0, a.Wo, ldb);
+        const size_t lat_off = (size_t)rn.lat * a.Wo * ldb;
+        qt.fetch(qy + lat_off, off);
+        gt.fetch(gy + lat_off, off);
         int col = c0 + lane; // lanes 0..31 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
         if (lane < HK) st = stats[(size_t)rn.lat * a.Wo + col];

@@ -41,7 +41,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 3; }
+extern "C" int s2attn_abi_version(void) { return 4; }
 
 namespace s2 {
 
@@ -225,9 +225,22 @@ struct Args {
     const int *goff, *gorder, *soff, *sorder;
     const Run *gruns, *sruns;
     int B, nh, Hi, Wi, Ho, Wo, dk_, dv_, pscale;
+    int kps; // real longitude ratio nlon_in / nlon_out; see key_point()
     int tile_rows; // LDS rows per staged band
     int row_first; // first entry of gorder / sorder this launch covers (dense rows come first, see s2attn_plan_split)
 };
+
+// Key-side addressing.  With nlon_in = kps * nlon_out, query column wo sees input columns ws + t + kps * wo: on the
+// sub-lattice {par, par + kps, ...} of a real input latitude that is a unit-stride problem.  The plan therefore lists
+// neighborhoods over Hi = nlat_in * kps "virtual" latitudes (real latitude * kps + par) of Wi = nlon_out columns each,
+// every kernel works as if nlon_in == nlon_out (pscale == 1), and only the address of a virtual grid point differs:
+// key_point() is the real point index of column 0 of a virtual latitude, consecutive columns lie kps points apart.
+// Gather runs carry the real latitude in Run::pad (also the index of the quadrature weight).
+__device__ inline long key_point(const Args &a, int b, int vlat, int rlat)
+{
+    return ((long)b * a.Hi + (long)rlat * a.kps) * a.Wi + (vlat - rlat * a.kps);
+}
+__device__ inline long key_row(const Args &a, int vlat, int rlat) { return (long)rlat * a.kps * a.Wi + (vlat - rlat * a.kps); }
 
 // ---------------------------------------------------------------------------------
 // forward:  y = sum_j a_j v_j / sum_j a_j
@@ -271,16 +284,16 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd
 
     for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
         const Run run = a.gruns[ri];
-        const float w = a.quad_w[run.lat];
-        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
-        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        const float w = a.quad_w[run.pad];
+        const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
+        const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
         for (int t0 = 0; t0 < run.len; t0 += TL) {
             const int L = min(TL, run.len - t0);
             const int c0 = (run.ws + t0 + ps * wo0) % a.Wi;
             const int nrows = ps * (nvalid - 1) + L;
             __syncthreads();
-            stage_rows<T, P, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
-            stage_rows<T, P, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            stage_rows<T, P, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, P, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
             __syncthreads();
 
             const float *krow = Ks + (ps * lane) * LS;
@@ -377,16 +390,16 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dq_
 
     for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
         const Run run = a.gruns[ri];
-        const float w = a.quad_w[run.lat];
-        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
-        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        const float w = a.quad_w[run.pad];
+        const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
+        const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
         for (int t0 = 0; t0 < run.len; t0 += TL) {
             const int L = min(TL, run.len - t0);
             const int c0 = (run.ws + t0 + ps * wo0) % a.Wi;
             const int nrows = ps * (nvalid - 1) + L;
             __syncthreads();
-            stage_rows<T, P, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
-            stage_rows<T, P, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            stage_rows<T, P, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, P, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
             __syncthreads();
 
             const float *krow = Ks + (ps * lane) * LS;
@@ -486,8 +499,8 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
     T *dk = static_cast<T *>(a.dk);
     T *dv = static_cast<T *>(a.dv);
 
-    stage_rows<T, P, VEC>(Qs, kx + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, ldk, a.dk_, wi0, a.Wi, nvalid, lane);
-    stage_rows<T, P, VEC>(Gs, vx + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, ldv, a.dv_, wi0, a.Wi, nvalid, lane);
+    stage_rows<T, P, VEC>(Qs, kx + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, ldk * a.kps, a.dk_, wi0, a.Wi, nvalid, lane);
+    stage_rows<T, P, VEC>(Gs, vx + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, ldv * a.kps, a.dv_, wi0, a.Wi, nvalid, lane);
     __syncthreads();
     float kr[P], vr[P], dkr[P], dvr[P];
 #pragma unroll
@@ -497,7 +510,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
         dkr[c] = 0.f;
         dvr[c] = 0.f;
     }
-    const float w = a.quad_w[hi];
+    const float w = a.quad_w[hi / a.kps];
 
     for (int ri = a.soff[hi]; ri < a.soff[hi + 1]; ri++) {
         const Run run = a.sruns[ri];
@@ -579,8 +592,8 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
         *reinterpret_cast<float4 *>(Gs + lane * LS + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
     }
     __syncthreads();
-    unstage_rows<T, P, VEC>(dk + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, Qs, ldk, a.dk_, wi0, nvalid, lane);
-    unstage_rows<T, P, VEC>(dv + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, Gs, ldv, a.dv_, wi0, nvalid, lane);
+    unstage_rows<T, P, VEC>(dk + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, Qs, ldk * a.kps, a.dk_, wi0, nvalid, lane);
+    unstage_rows<T, P, VEC>(dv + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, Gs, ldv * a.kps, a.dv_, wi0, nvalid, lane);
 }
 
 
@@ -640,16 +653,16 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
 
     for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
         const Run run = a.gruns[ri];
-        const float w = a.quad_w[run.lat];
-        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
-        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        const float w = a.quad_w[run.pad];
+        const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
+        const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
         for (int t0 = 0; t0 < run.len; t0 += TL) {
             const int L = min(TL, run.len - t0);
             const int c0 = (run.ws + t0 + ps * w0) % a.Wi;
             const int nrows = ps * (nvalid - 1) + L;
             __syncthreads();
-            stage_rows<T, PT, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
-            stage_rows<T, PT, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
             __syncthreads();
             const float *krow = Ks + (ps * qi) * LS + sl * 32;
             const float *vrow = Vs + (ps * qi) * LS + sl * 32;
@@ -725,16 +738,16 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
 
     for (int ri = a.goff[ho]; ri < a.goff[ho + 1]; ri++) {
         const Run run = a.gruns[ri];
-        const float w = a.quad_w[run.lat];
-        const T *kl = kx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldk + (long)h * a.dk_;
-        const T *vl = vx + ((long)(b * a.Hi + run.lat) * a.Wi) * ldv + (long)h * a.dv_;
+        const float w = a.quad_w[run.pad];
+        const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
+        const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
         for (int t0 = 0; t0 < run.len; t0 += TL) {
             const int L = min(TL, run.len - t0);
             const int c0 = (run.ws + t0 + ps * w0) % a.Wi;
             const int nrows = ps * (nvalid - 1) + L;
             __syncthreads();
-            stage_rows<T, PT, VEC>(Ks, kl, ldk, a.dk_, c0, a.Wi, nrows, lane);
-            stage_rows<T, PT, VEC>(Vs, vl, ldv, a.dv_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
             __syncthreads();
             const float *krow = Ks + (ps * qi) * LS + sl * 32;
             const float *vrow = Vs + (ps * qi) * LS + sl * 32;
@@ -812,8 +825,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
     T *dk = static_cast<T *>(a.dk);
     T *dv = static_cast<T *>(a.dv);
 
-    stage_rows<T, PT, VEC>(Qs, kx + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, ldk, a.dk_, w0, a.Wi, nvalid, lane);
-    stage_rows<T, PT, VEC>(Gs, vx + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, ldv, a.dv_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, PT, VEC>(Qs, kx + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, ldk * a.kps, a.dk_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, PT, VEC>(Gs, vx + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, ldv * a.kps, a.dv_, w0, a.Wi, nvalid, lane);
     __syncthreads();
     float kr[32], vr[32], dkr[32], dvr[32];
 #pragma unroll
@@ -823,7 +836,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
         dkr[c] = 0.f;
         dvr[c] = 0.f;
     }
-    const float w = a.quad_w[hi];
+    const float w = a.quad_w[hi / a.kps];
 
     for (int ri = a.soff[hi]; ri < a.soff[hi + 1]; ri++) {
         const Run run = a.sruns[ri];
@@ -889,8 +902,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
         *reinterpret_cast<float4 *>(Gs + qi * LS + sl * 32 + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
     }
     __syncthreads();
-    unstage_rows<T, PT, VEC>(dk + ((long)(b * a.Hi + hi) * a.Wi) * ldk + (long)h * a.dk_, Qs, ldk, a.dk_, w0, nvalid, lane);
-    unstage_rows<T, PT, VEC>(dv + ((long)(b * a.Hi + hi) * a.Wi) * ldv + (long)h * a.dv_, Gs, ldv, a.dv_, w0, nvalid, lane);
+    unstage_rows<T, PT, VEC>(dk + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, Qs, ldk * a.kps, a.dk_, w0, nvalid, lane);
+    unstage_rows<T, PT, VEC>(dv + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, Gs, ldv * a.kps, a.dv_, w0, nvalid, lane);
 }
 
 // ---------------------------------------------------------------------------------
@@ -980,8 +993,8 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kern
         int c0 = rn.ws + t + w0;
         c0 -= (c0 >= a.Wi) ? a.Wi : 0;
         c0 -= (c0 >= a.Wi) ? a.Wi : 0;
-        kb.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, r0, cb);
-        vb.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, r0, cb);
+        kb.fetch(kx + (size_t)key_row(a, rn.lat, rn.pad) * ldk, ldk * a.kps, c0, a.Wi, r0, cb);
+        vb.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, r0, cb);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -996,7 +1009,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kern
 
     while (ri < rend) {
         const int L = min(TL, run.len - t0);
-        const float w = a.quad_w[run.lat];
+        const float w = a.quad_w[run.pad];
         int nri = ri, nt0 = t0 + TL;
         Run nrun = run;
         if (nt0 >= run.len) {
@@ -1106,8 +1119,8 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kerne
         int c0 = rn.ws + t + w0;
         c0 -= (c0 >= a.Wi) ? a.Wi : 0;
         c0 -= (c0 >= a.Wi) ? a.Wi : 0;
-        kb.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, r0, cb);
-        vb.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, r0, cb);
+        kb.fetch(kx + (size_t)key_row(a, rn.lat, rn.pad) * ldk, ldk * a.kps, c0, a.Wi, r0, cb);
+        vb.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, r0, cb);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -1122,7 +1135,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kerne
 
     while (ri < rend) {
         const int L = min(TL, run.len - t0);
-        const float w = a.quad_w[run.lat];
+        const float w = a.quad_w[run.pad];
         int nri = ri, nt0 = t0 + TL;
         Run nrun = run;
         if (nt0 >= run.len) {
@@ -1221,16 +1234,17 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
     const unsigned ldk = a.nh * a.dk_, ldv = a.nh * a.dv_;
     const int r0 = lane / BandT::V4, cb = 4 * (lane % BandT::V4);
 
-    const T *kx = static_cast<const T *>(a.k) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldk + (size_t)h * a.dk_;
-    const T *vx = static_cast<const T *>(a.v) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldv + (size_t)h * a.dv_;
+    const size_t kpt = (size_t)key_point(a, b, hi, hi / a.kps);
+    const T *kx = static_cast<const T *>(a.k) + kpt * ldk + (size_t)h * a.dk_;
+    const T *vx = static_cast<const T *>(a.v) + kpt * ldv + (size_t)h * a.dv_;
     const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldk + (size_t)h * a.dk_;
     const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * a.dv_;
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
-    T *dk = static_cast<T *>(a.dk) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldk + (size_t)h * a.dk_;
-    T *dv = static_cast<T *>(a.dv) + ((size_t)(b * a.Hi + hi) * a.Wi) * ldv + (size_t)h * a.dv_;
+    T *dk = static_cast<T *>(a.dk) + kpt * ldk + (size_t)h * a.dk_;
+    T *dv = static_cast<T *>(a.dv) + kpt * ldv + (size_t)h * a.dv_;
 
-    stage_rows<T, P, true>(Qs, kx, ldk, a.dk_, w0, a.Wi, nvalid, lane);
-    stage_rows<T, P, true>(Gs, vx, ldv, a.dv_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, P, true>(Qs, kx, ldk * a.kps, a.dk_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, P, true>(Gs, vx, ldv * a.kps, a.dv_, w0, a.Wi, nvalid, lane);
     __syncthreads();
     float kr[P], vr[P], dkr[P], dvr[P];
 #pragma unroll
@@ -1240,7 +1254,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
         dkr[c] = 0.f;
         dvr[c] = 0.f;
     }
-    const float w = a.quad_w[hi];
+    const float w = a.quad_w[hi / a.kps];
 
     int ri = a.soff[hi];
     const int rend = a.soff[hi + 1];
@@ -1332,8 +1346,8 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
         *reinterpret_cast<float4 *>(Gs + lane * LS + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
     }
     __syncthreads();
-    unstage_rows<T, P, true>(dk, Qs, ldk, a.dk_, w0, nvalid, lane);
-    unstage_rows<T, P, true>(dv, Gs, ldv, a.dv_, w0, nvalid, lane);
+    unstage_rows<T, P, true>(dk, Qs, ldk * a.kps, a.dk_, w0, nvalid, lane);
+    unstage_rows<T, P, true>(dv, Gs, ldv * a.kps, a.dv_, w0, nvalid, lane);
 }
 
 
@@ -1449,8 +1463,8 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         const bool fifth = !run_is_dense(rn.len);
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane, fifth);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane, fifth);
+        kt.fetch(kx + (size_t)key_row(a, rn.lat, rn.pad) * ldk, ldk * a.kps, c0, a.Wi, lane, fifth);
+        vt.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, lane, fifth);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -1461,7 +1475,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     __syncthreads();
 
     while (ri < rend) {
-        const float w = a.quad_w[run.lat];
+        const float w = a.quad_w[run.pad];
         const int len = run.len;
         int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
@@ -1646,8 +1660,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         const bool fifth = !run_is_dense(rn.len);
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane, fifth);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane, fifth);
+        kt.fetch(kx + (size_t)key_row(a, rn.lat, rn.pad) * ldk, ldk * a.kps, c0, a.Wi, lane, fifth);
+        vt.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, lane, fifth);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -1658,7 +1672,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
     __syncthreads();
 
     while (ri < rend) {
-        const float w = a.quad_w[run.lat];
+        const float w = a.quad_w[run.pad];
         const int len = run.len;
         int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
@@ -1875,8 +1889,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         const bool fifth = !run_is_dense(rn.len);
-        kt.fetch(kx + (size_t)rn.lat * a.Wi * ldk, ldk, c0, a.Wi, lane, fifth);
-        vt.fetch(vx + (size_t)rn.lat * a.Wi * ldv, ldv, c0, a.Wi, lane, fifth);
+        kt.fetch(kx + (size_t)key_row(a, rn.lat, rn.pad) * ldk, ldk * a.kps, c0, a.Wi, lane, fifth);
+        vt.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, lane, fifth);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -1887,7 +1901,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     __syncthreads();
 
     while (ri < rend) {
-        const float w = a.quad_w[run.lat];
+        const float w = a.quad_w[run.pad];
         const int len = run.len;
         int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
@@ -2011,7 +2025,7 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * 32;
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = j < nvalid;
-    const size_t pt = (size_t)(b * a.Hi + hi) * a.Wi + w0 + (mine ? j : 0);
+    const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? j : 0)) * a.kps;
 
     float kb[16], vb[16];
     {
@@ -2031,7 +2045,7 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
         dkt[v] = 0.f;
         dvt[v] = 0.f;
     }
-    const float w = a.quad_w[hi];
+    const float w = a.quad_w[hi / a.kps];
 
     int ri = a.soff[hi];
     const int rend = a.soff[hi + 1];
@@ -2430,13 +2444,14 @@ void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const f
     a.sorder = plan->scatter_order;
     a.B = sh->batch;
     a.nh = sh->num_heads;
-    a.Hi = sh->nlat_in;
-    a.Wi = sh->nlon_in;
+    a.kps = sh->nlon_in / sh->nlon_out;
+    a.Hi = sh->nlat_in * a.kps; // virtual input latitudes, see key_point()
+    a.Wi = sh->nlon_out;        // columns of a virtual latitude
     a.Ho = sh->nlat_out;
     a.Wo = sh->nlon_out;
     a.dk_ = sh->ck;
     a.dv_ = sh->cv;
-    a.pscale = sh->nlon_in / sh->nlon_out;
+    a.pscale = 1;
 }
 
 } // namespace
@@ -2473,8 +2488,7 @@ namespace {
 // that is not handed them (s2attn_backward, s2attn_backward_dq) first recomputes both into the tail of the workspace.
 bool h16_shape(const s2attn_shape *sh)
 {
-    return sh->dtype != S2ATTN_F32 && sh->ck == sh->cv && (sh->ck == 32 || sh->ck == 64 || sh->ck == 128) && sh->nlon_in == sh->nlon_out
-        && sh->nlon_in >= HK;
+    return sh->dtype != S2ATTN_F32 && sh->ck == sh->cv && (sh->ck == 32 || sh->ck == 64 || sh->ck == 128) && sh->nlon_out >= HK;
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
 int64_t round16(int64_t n) { return (n + 15) / 16 * 16; }

@@ -17,7 +17,7 @@
 namespace {
 
 struct HostRun {
-    int32_t ho, hi, ws, len;
+    int32_t ho, hi, ws, len; // after decompose(): hi is the virtual latitude (real latitude * ps + parity class)
 };
 
 // Splits the CSR into maximal runs of consecutive longitudes inside one input
@@ -37,6 +37,7 @@ int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int n
                            (long long)row_off[0], (long long)row_off[nlat_out]);
 
     const int64_t ncol = (int64_t)nlat_in * nlon_in;
+    const int ps = nlon_in / nlon_out;
     int64_t total = 0;
     std::vector<HostRun> row;
     for (int ho = 0; ho < nlat_out; ho++) {
@@ -66,10 +67,18 @@ int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int n
             }
             i = j + 1;
         }
+        // Longitude ratio ps = nlon_in / nlon_out > 1: query wo sees columns ws + t + ps * wo.  Split every run by
+        // column parity class: on the sub-lattice {par, par + ps, par + 2 ps, ...} of latitude hi (a "virtual latitude"
+        // hi * ps + par with nlon_out columns) the same neighbors are the run (ws', len') with unit stride in wo.
         for (const HostRun &r : row) {
             if (r.len == 0) continue;
-            total++;
-            if (out) out->push_back(r);
+            for (int par = 0; par < ps; par++) {
+                const int t0 = ((par - r.ws) % ps + ps) % ps; // first neighbor of the run in this class
+                if (t0 >= r.len) continue;
+                const int first = (r.ws + t0) % nlon_in;
+                total++;
+                if (out) out->push_back({ho, r.hi * ps + par, (first - par) / ps, (r.len - t0 + ps - 1) / ps});
+            }
         }
     }
     *count = total;
@@ -129,27 +138,28 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
     if (rc != S2ATTN_OK) return rc;
     if (n != nruns) return s2attn_fail(S2ATTN_E_INVALID, "nruns = %lld does not match the CSR (%lld runs)", (long long)nruns, (long long)n);
 
-    const int pscale = nlon_in / nlon_out;
+    const int ps = nlon_in / nlon_out;
+    const int nvlat = nlat_in * ps; // virtual input latitudes
 
     // gather side: runs are already grouped by ho, in CSR order
-    std::vector<RowCost> gcost(nlat_out), scost(nlat_in);
+    std::vector<RowCost> gcost(nlat_out), scost(nvlat);
     std::fill(gather_off, gather_off + nlat_out + 1, 0);
     for (int64_t i = 0; i < n; i++) {
         const HostRun &r = runs[i];
         gather_runs[4 * i + 0] = r.hi;
         gather_runs[4 * i + 1] = r.ws;
         gather_runs[4 * i + 2] = r.len;
-        gather_runs[4 * i + 3] = 0;
+        gather_runs[4 * i + 3] = r.hi / ps; // real latitude: quadrature weight index, row address
         gather_off[r.ho + 1]++;
         gcost[r.ho].add(r.len);
     }
     for (int ho = 0; ho < nlat_out; ho++) gather_off[ho + 1] += gather_off[ho];
 
     // scatter side: stable counting sort by hi keeps ho ascending inside a group
-    std::fill(scatter_off, scatter_off + nlat_in + 1, 0);
+    std::fill(scatter_off, scatter_off + nvlat + 1, 0);
     for (int64_t i = 0; i < n; i++) scatter_off[runs[i].hi + 1]++;
-    for (int hi = 0; hi < nlat_in; hi++) scatter_off[hi + 1] += scatter_off[hi];
-    std::vector<int32_t> cursor(scatter_off, scatter_off + nlat_in);
+    for (int hi = 0; hi < nvlat; hi++) scatter_off[hi + 1] += scatter_off[hi];
+    std::vector<int32_t> cursor(scatter_off, scatter_off + nvlat);
     for (int64_t i = 0; i < n; i++) {
         const HostRun &r = runs[i];
         const int32_t s = cursor[r.hi]++;
@@ -157,7 +167,7 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
         scatter_runs[4 * s + 1] = r.ws;
         scatter_runs[4 * s + 2] = r.len;
         scatter_runs[4 * s + 3] = 0;
-        scost[r.hi].add((r.len + pscale - 1) / pscale);
+        scost[r.hi].add(r.len);
     }
 
     ndense[0] = order_rows(gcost, gather_order);
