@@ -15,6 +15,7 @@ Reported alongside the throughput:
                 around every launch of it inside the timed region
   cpu_baseline  the CPU port of the reference algorithm (oracle/, reference release flags, OpenMP)
                 on a bounded sample of the same workload, on this machine's host cores
+  other_configs op-level forward and backward times of the other four benchmark configurations
 """
 
 import argparse
@@ -34,6 +35,7 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E
 FP32_MATRIX_PEAK_TFLOPS = 157.3  # dense fp32 MFMA: the unit the long-run (polar) part of the path runs on
+BF16_MATRIX_PEAK_TFLOPS = 2500.0  # dense bf16 MFMA
 FP32_VALU_PEAK_TFLOPS = 78.6  # 157.3 TFLOP/s vector fp32 is quoted with packed FMA; these kernels are built without packed fp32
 
 CONFIGS = {
@@ -41,6 +43,9 @@ CONFIGS = {
     "cfg2": dict(in_shape=(128, 256), out_shape=(128, 256), grid_in="equiangular", grid_out="equiangular", B=4, C=64, nh=4, theta_cutoff=4 * math.pi / 127),
     "cfg3": dict(in_shape=(721, 1440), out_shape=(721, 1440), grid_in="equiangular", grid_out="equiangular", B=1, C=256, nh=8, theta_cutoff=3 * math.pi / 720),
     "cfg4": dict(in_shape=(721, 1440), out_shape=(360, 720), grid_in="equiangular", grid_out="legendre-gauss", B=2, C=128, nh=4, theta_cutoff=2 * math.pi / 359),
+    "cfg5": dict(
+        in_shape=(361, 720), out_shape=(361, 720), grid_in="legendre-gauss", grid_out="legendre-gauss", B=4, C=1024, nh=16, theta_cutoff=8 * math.pi / 360, dtype="bf16"
+    ),
 }
 
 
@@ -94,6 +99,44 @@ def make_workload(cfg, device, seed=333):
     return mod, x_in, x_out, k, v, q, dy
 
 
+def time_other_config(name, device, steps=3):
+    """Op-level forward + backward (ms) of another benchmark configuration on N(0,1)-type inputs in its own storage
+    dtype (cfg5: 0.5 * N(0,1) in bf16), psi and quadrature weights from the package's geometry code."""
+    from torch_harmonics_amd import ops
+    from torch_harmonics_amd.neighborhood import precompute_neighborhood_s2
+    from torch_harmonics_amd.quadrature import precompute_latitudes
+
+    cfg = CONFIGS[name]
+    (Hi, Wi), (Ho, Wo) = cfg["in_shape"], cfg["out_shape"]
+    nh, B, d = cfg["nh"], cfg["B"], cfg["C"] // cfg["nh"]
+    dt = torch.bfloat16 if cfg.get("dtype") == "bf16" else torch.float32
+    col, roff, _ = precompute_neighborhood_s2(cfg["in_shape"], cfg["out_shape"], cfg["grid_in"], cfg["grid_out"], cfg["theta_cutoff"])
+    w = (2.0 * torch.pi * precompute_latitudes(Hi, cfg["grid_in"])[1].float() / Wi).contiguous().to(device)
+    col, roff = col.to(device), roff.to(device)
+    gen = torch.Generator(device=device).manual_seed(333)
+    scale = 0.5 if dt == torch.bfloat16 else 1.0
+    k = (scale * torch.randn(B, Hi, Wi, nh * d, device=device, generator=gen)).to(dt)
+    v = (scale * torch.randn(B, Hi, Wi, nh * d, device=device, generator=gen)).to(dt)
+    q = (scale * torch.randn(B, Ho, Wo, nh * d, device=device, generator=gen) / math.sqrt(d)).to(dt)
+    dy = (scale * torch.randn(B, Ho, Wo, nh * d, device=device, generator=gen)).to(dt)
+    geo = (w, col, roff, nh, Wi, Ho, Wo)
+    pairs = B * nh * Wo * col.numel()
+
+    def run(f):
+        f()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            f()
+        torch.cuda.synchronize()
+        return 1e3 * (time.perf_counter() - t0) / steps
+
+    y, lse = ops.forward_lse(k, v, q, *geo)
+    t_fwd = run(lambda: ops.forward_lse(k, v, q, *geo))
+    t_bwd = run(lambda: ops.backward_saved(k, v, q, dy, y, lse, *geo))
+    return {"fwd_ms": t_fwd, "bwd_ms": t_bwd, "pairs": pairs, "pairs_per_s": pairs / ((t_fwd + t_bwd) * 1e-3), "dtype": "bf16" if dt == torch.bfloat16 else "f32"}
+
+
 def cpu_baseline(cfg, mod, k, v, q, dy):
     """
     Times the fp32 CPU port of the reference algorithm (oracle/s2attn_oracle.c, built with the reference's
@@ -115,11 +158,11 @@ def cpu_baseline(cfg, mod, k, v, q, dy):
     ro_s = torch.zeros(len(rows) + 1, dtype=torch.int64)
     ro_s[1:] = torch.cumsum(lens, 0)
     col_s = torch.cat([col[ro[r] : ro[r + 1]] for r in rows.tolist()])
-    ks = k[..., : nh_s * ck].cpu().contiguous()
-    vs = v[..., : nh_s * cv].cpu().contiguous()
-    qs = q[:, rows][..., : nh_s * ck].cpu().contiguous()
-    gs = dy[:, rows][..., : nh_s * cv].cpu().contiguous()
-    w = mod.quad_weights.cpu()
+    ks = k[..., : nh_s * ck].float().cpu().contiguous()
+    vs = v[..., : nh_s * cv].float().cpu().contiguous()
+    qs = q[:, rows][..., : nh_s * ck].float().cpu().contiguous()
+    gs = dy[:, rows][..., : nh_s * cv].float().cpu().contiguous()
+    w = mod.quad_weights.float().cpu()
     pairs = cfg["B"] * nh_s * Wo * int(lens.sum())
     scratch_gb = 2 * cfg["B"] * nh_s * len(rows) * Wo * int(lens.max()) * 4 / 1e9
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
@@ -146,6 +189,7 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the op-level timings of the other benchmark configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true", help="skip the module-level (projections + permutes) timing")
     args = ap.parse_args()
@@ -170,7 +214,14 @@ def main():
     nnz = mod.psi_col_idx.numel()
     pairs = B * nh * Wo * nnz
     wq, ci, ro = mod.quad_weights, mod.psi_col_idx, mod.psi_roff_idx
-    esz = 4
+    bf16 = cfg.get("dtype") == "bf16"
+    esz = 2 if bf16 else 4
+    if bf16:  # 16-bit storage configuration: inputs scaled by 0.5 and stored as bf16, module in bf16
+        mod = mod.to(torch.bfloat16)
+        mod.quad_weights = wq  # the quadrature weights stay fp32
+        x_in, x_out = (0.5 * x_in).to(torch.bfloat16), (0.5 * x_out).to(torch.bfloat16) if x_out is not x_in else None
+        x_out = x_in if x_out is None else x_out
+        k, v, q, dy = [(0.5 * t).to(torch.bfloat16).contiguous() for t in (k, v, q, dy)]
 
     def step():
         y, lse = ops.forward_lse(k, v, q, wq, ci, ro, nh, Wi, Ho, Wo)
@@ -187,8 +238,8 @@ def main():
 
     # ---- per-kernel durations: events on the launch stream around each launch, same K steps ----
     plan = get_plan(ci, ro, Hi, Wi, Ho, Wo)
-    shape = _lib.ShapeStruct(B, nh, Hi, Wi, Ho, Wo, k.shape[3] // nh, v.shape[3] // nh, _lib.S2ATTN_F32)
-    y = torch.empty(q.shape[:3] + (v.shape[3],), device=dev)
+    shape = _lib.ShapeStruct(B, nh, Hi, Wi, Ho, Wo, k.shape[3] // nh, v.shape[3] // nh, _lib.S2ATTN_BF16 if bf16 else _lib.S2ATTN_F32)
+    y = torch.empty(q.shape[:3] + (v.shape[3],), device=dev, dtype=k.dtype)
     dk, dv, dq = torch.empty_like(k), torch.empty_like(v), torch.empty_like(q)
     ws = torch.empty(lib.s2attn_backward_workspace_bytes(ctypes.byref(shape)) // 4, device=dev)
     lse = torch.empty((B, nh, Ho, Wo), device=dev)
@@ -219,11 +270,13 @@ def main():
     d = k.shape[3] // nh
     # per launch: compulsory traffic (every tensor the kernel must read or write, once), algorithmic flops
     # (2*d per contraction per pair: forward q.k, p.v; dq pass q.k, dy.v, dq; dk/dv pass q.k, dy.v, dk, dv), time
+    kname = ("fwd_h16_kernel", "dq_h16_kernel", "dkdv_h16_kernel") if bf16 else ("fwd_mfma_kernel", "dq_saved_mfma_kernel", "dkdv_mfma_kernel")
     alg = {
-        "s2::fwd_mfma_kernel (forward)": (esz * (nq + nk + nv + ny) + 4 * nstat, 4 * d * pairs, t_fwd),
-        "s2::dq_saved_mfma_kernel (backward, dq)": (esz * (nq + nk + nv + ny + ny + nq) + 12 * nstat, 6 * d * pairs, t_dq),
-        "s2::dkdv_mfma_kernel (backward, dk + dv)": (esz * (nq + nk + nv + ny + nk + nv) + 8 * nstat, 8 * d * pairs, t_dkdv),
+        f"s2::{kname[0]} (forward)": (esz * (nq + nk + nv + ny) + 4 * nstat, 4 * d * pairs, t_fwd),
+        f"s2::{kname[1]} (backward, dq)": (esz * (nq + nk + nv + ny + ny + nq) + 12 * nstat, 6 * d * pairs, t_dq),
+        f"s2::{kname[2]} (backward, dk + dv)": (esz * (nq + nk + nv + ny + nk + nv) + 8 * nstat, 8 * d * pairs, t_dkdv),
     }
+    matrix_peak = BF16_MATRIX_PEAK_TFLOPS if bf16 else FP32_MATRIX_PEAK_TFLOPS
     dom = max(alg, key=lambda n: alg[n][2])
     dom_bytes, dom_flops, dom_ms = alg[dom]
     # HBM bytes per launch measured with rocprofv3 counters on this workload (see profiles/); only valid for cfg3
@@ -249,10 +302,10 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f32",
+        "dtype": "bf16" if bf16 else "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.config}: {cfg['grid_in']} {Hi}x{Wi} -> {cfg['grid_out']} {Ho}x{Wo}, B={B}, C={cfg['C']}, heads={nh}, fp32, theta_cutoff={cfg['theta_cutoff']}, nnz={nnz}, pairs={pairs}",
+            "workload": f"{args.config}: {cfg['grid_in']} {Hi}x{Wi} -> {cfg['grid_out']} {Ho}x{Wo}, B={B}, C={cfg['C']}, heads={nh}, {'bf16' if bf16 else 'fp32'}, theta_cutoff={cfg['theta_cutoff']}, nnz={nnz}, pairs={pairs}",
             "level": "op (s2attn forward + backward through the C ABI); module-level time in module_ms_per_step",
         },
         # 44 flop per compulsory byte puts this workload above the fp32 ridge (157.3 TFLOP/s / 8 TB/s = 20): the fp32
@@ -261,9 +314,9 @@ def main():
             "bound": "mfma",
             "kernel": dom,
             "achieved": achieved_tf,
-            "peak": FP32_MATRIX_PEAK_TFLOPS,
+            "peak": matrix_peak,
             "unit": "TFLOP/s",
-            "frac": achieved_tf / FP32_MATRIX_PEAK_TFLOPS,
+            "frac": achieved_tf / matrix_peak,
             "traffic": traffic,
             "algorithmic_flops": dom_flops,
             "kernel_ms": dom_ms,
@@ -281,7 +334,7 @@ def main():
         },
         "kernel_ms": {"fwd": t_fwd, "dq": t_dq, "dkdv": t_dkdv},
         "step_hbm_frac": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
-        "step_fp32_matrix_frac": flops_alg / (ms_step * 1e-3) / 1e12 / FP32_MATRIX_PEAK_TFLOPS,
+        "step_matrix_frac": flops_alg / (ms_step * 1e-3) / 1e12 / matrix_peak,
         "step_fp32_valu_frac": flops_alg / (ms_step * 1e-3) / 1e12 / FP32_VALU_PEAK_TFLOPS,
     }
 
@@ -289,7 +342,7 @@ def main():
         xq = x_out.clone().requires_grad_(True)
         same = x_in is x_out
         xk = None if same else x_in.clone().requires_grad_(True)
-        gout = torch.randn(B, mod.out_channels, Ho, Wo, device=dev)
+        gout = torch.randn(B, mod.out_channels, Ho, Wo, device=dev).to(x_out.dtype)
 
         def mstep():
             o = mod(xq) if same else mod(xq, xk, xk)
@@ -308,6 +361,9 @@ def main():
             mstep()
         torch.cuda.synchronize()
         out["module_ms_per_step"] = 1e3 * (time.perf_counter() - t0) / nm
+
+    if not args.no_other_configs:
+        out["other_configs"] = {name: time_other_config(name, dev) for name in sorted(CONFIGS) if name != args.config}
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy)

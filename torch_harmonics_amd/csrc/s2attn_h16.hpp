@@ -68,7 +68,9 @@ template <int D> struct HTile {
     static constexpr int CPR = D / 8;        // 16-byte pieces per row
     static constexpr int RPI = 64 / CPR;     // rows per iteration
     static constexpr int NIT = HK / RPI;     // iterations
-    static constexpr int PITCH = 2 * D + 16; // bytes; 16-byte reads of 8 consecutive rows fall in distinct banks
+    static constexpr int PITCH = 2 * D + 32; // bytes.  Measured with SQ_LDS_BANK_CONFLICT: row pitches of 32 or 96 bytes modulo 128
+                                             // are free of bank conflicts for all three access patterns (16-byte row pieces by lanes
+                                             // (c, qd), transposing 8-byte reads, 16-byte writes); 2 D + 16 costs both reads 2x
     u4v raw[NIT];
     // Byte offsets of this lane's pieces inside one latitude of one (batch, head) slice; the same for every tensor of
     // a step (k and v, or q and dy).  lane_off = (lane / CPR) * ldb + 16 * (lane % CPR).
