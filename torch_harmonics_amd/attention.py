@@ -146,10 +146,10 @@ class NeighborhoodAttentionS2(nn.Module):
             f"out_channels={self.out_channels}, k_channels={self.k_channels}, theta_cutoff={self.theta_cutoff}"
         )
 
-    def _head_rms_norm(self, x: torch.Tensor, gain: torch.Tensor) -> torch.Tensor:
+    def _head_rms_norm(self, x: torch.Tensor, gain: torch.Tensor, scale=None) -> torch.Tensor:
         B, H, W, C = x.shape
         x = x.reshape(B, H, W, self.num_heads, -1)
-        x = F.rms_norm(x, normalized_shape=gain.shape, weight=1 + gain)
+        x = F.rms_norm(x, normalized_shape=gain.shape, weight=1 + gain if scale is None else (1 + gain) * scale)
         return x.reshape(B, H, W, C)
 
     def forward(self, query: torch.Tensor, key: Optional[torch.Tensor] = None, value: Optional[torch.Tensor] = None) -> torch.Tensor:
@@ -179,17 +179,22 @@ class NeighborhoodAttentionS2(nn.Module):
         key = query if key_is_query else to_nhwc(key)
         value = query if value_is_query else (key if value_is_key else to_nhwc(value))
 
-        query = F.linear(query, self.q_weights.view(self.q_weights.shape[0], -1), self.q_bias)
+        # the softmax scale rides on the q projection (or on the q gain when the q/k RMS norm is on): no pass of its own
+        normed = self.q_norm_weights is not None
+        wq = self.q_weights.view(self.q_weights.shape[0], -1)
+        if normed:
+            query = F.linear(query, wq, self.q_bias)
+        else:
+            query = F.linear(query, wq * self.scale, None if self.q_bias is None else self.q_bias * self.scale)
         key = F.linear(key, self.k_weights.view(self.k_weights.shape[0], -1), self.k_bias)
         value = F.linear(value, self.v_weights.view(self.v_weights.shape[0], -1), self.v_bias)
 
-        if self.q_norm_weights is not None:
-            query = self._head_rms_norm(query, self.q_norm_weights)
-        if self.k_norm_weights is not None:
+        if normed:
+            query = self._head_rms_norm(query, self.q_norm_weights, self.scale)
             key = self._head_rms_norm(key, self.k_norm_weights)
 
         out = self.attention_handle(
-            key, value, query * self.scale, self.quad_weights, self.psi_col_idx, self.psi_roff_idx, self.num_heads, self.nlon_in, self.nlat_out, self.nlon_out
+            key, value, query, self.quad_weights, self.psi_col_idx, self.psi_roff_idx, self.num_heads, self.nlon_in, self.nlat_out, self.nlon_out
         )
 
         out = F.linear(out, self.proj_weights.view(self.proj_weights.shape[0], -1), self.proj_bias)
