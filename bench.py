@@ -99,7 +99,7 @@ def make_workload(cfg, device, seed=333):
     return mod, x_in, x_out, k, v, q, dy
 
 
-def time_other_config(name, device, steps=3):
+def time_other_config(name, device, steps=3, cpu=False):
     """Op-level forward + backward (ms) of another benchmark configuration on N(0,1)-type inputs in its own storage
     dtype (cfg5: 0.5 * N(0,1) in bf16), psi and quadrature weights from the package's geometry code."""
     from torch_harmonics_amd import ops
@@ -134,7 +134,19 @@ def time_other_config(name, device, steps=3):
     y, lse = ops.forward_lse(k, v, q, *geo)
     t_fwd = run(lambda: ops.forward_lse(k, v, q, *geo))
     t_bwd = run(lambda: ops.backward_saved(k, v, q, dy, y, lse, *geo))
-    return {"fwd_ms": t_fwd, "bwd_ms": t_bwd, "pairs": pairs, "pairs_per_s": pairs / ((t_fwd + t_bwd) * 1e-3), "dtype": "bf16" if dt == torch.bfloat16 else "f32"}
+    res = {"fwd_ms": t_fwd, "bwd_ms": t_bwd, "pairs": pairs, "pairs_per_s": pairs / ((t_fwd + t_bwd) * 1e-3), "dtype": "bf16" if dt == torch.bfloat16 else "f32"}
+    if cpu and dt == torch.float32:
+        # the whole configuration on the CPU port of the reference algorithm (its backward scratch is 2*B*nh*Ho*Wo*max_row floats)
+        from oracle import cpu_attention as oracle
+
+        hk, hv, hq, hg, hw, hc, hr = [t.cpu() for t in (k, v, q, dy, w, col, roff)]
+        t0 = time.perf_counter()
+        oracle.forward_f32(hk, hv, hq, hw, hc, hr, nh, fast=True)
+        t1 = time.perf_counter()
+        oracle.backward_f32(hk, hv, hq, hg, hw, hc, hr, nh, fast=True)
+        t2 = time.perf_counter()
+        res["cpu_port_fwd_ms"], res["cpu_port_bwd_ms"] = 1e3 * (t1 - t0), 1e3 * (t2 - t1)
+    return res
 
 
 def cpu_baseline(cfg, mod, k, v, q, dy):
@@ -363,7 +375,10 @@ def main():
         out["module_ms_per_step"] = 1e3 * (time.perf_counter() - t0) / nm
 
     if not args.no_other_configs:
-        out["other_configs"] = {name: time_other_config(name, dev) for name in sorted(CONFIGS) if name != args.config}
+        # cfg1 and cfg2 are small enough for the reference's CPU algorithm in full: timed beside the GPU when the CPU leg is on
+        out["other_configs"] = {
+            name: time_other_config(name, dev, cpu=(not args.no_cpu_baseline) and name in ("cfg1", "cfg2")) for name in sorted(CONFIGS) if name != args.config
+        }
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy)
