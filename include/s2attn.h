@@ -13,7 +13,11 @@
  *   q  [B, nlat_out, nlon_out, num_heads*ck]   y, dy [B, nlat_out, nlon_out, num_heads*cv]
  * physical NHWC, contiguous, heads packed along the channel axis, one storage
  * dtype for all activations; quad_weights [nlat_in] fp32; q arrives already
- * multiplied by the softmax scale.  nlon_in must be a multiple of nlon_out.
+ * multiplied by the softmax scale.  Either nlon_in is a multiple of nlon_out
+ * (self-attention and down-sampling, "gather" direction) or nlon_out is a
+ * proper multiple of nlon_in (up-sampling, "scatter" direction); the two
+ * directions are told apart by the longitude counts, as in the reference
+ * (attention.py:337).
  */
 #ifndef S2ATTN_H
 #define S2ATTN_H
@@ -40,24 +44,27 @@ const char *s2attn_last_error(void);
 int s2attn_abi_version(void);
 
 /*
- * Neighborhood plan.  The reference kernels walk the CSR neighborhood
- * (row_off[nlat_out+1], col_idx[nnz], col = hi*nlon_in + wi at output longitude 0)
- * entry by entry and re-sort its rows by length on every call
- * (attention_cuda_utils.cu:74-113, called from attention_cuda_fwd.cu:476 and
- * attention_cuda_bwd.cu:792).  This library instead converts the CSR once, on the
- * host, into runs of consecutive longitudes:
+ * Neighborhood plan.  The reference kernels walk the CSR neighborhood entry by entry and re-sort its rows by length
+ * on every call (attention_cuda_utils.cu:74-113, called from attention_cuda_fwd.cu:476 and attention_cuda_bwd.cu:792).
+ *   gather direction:  row_off[nlat_out+1], col = hi*nlon_in + wi: the input points output point (ho, 0) attends to;
+ *                      output column wo sees them shifted by (nlon_in/nlon_out)*wo      (attention_torch.py:97-104)
+ *   scatter direction: row_off[nlat_in+1],  col = ho*nlon_out + wo: the output points that attend to input point
+ *                      (hi, 0); input column wi is seen by them shifted by (nlon_out/nlon_in)*wi (attention_torch.py:613-621)
+ * This library converts either CSR once, on the host, into runs of consecutive longitudes:
  *
  *   run = (lat, ws, len, aux)   four int32
  *
- * With ps = nlon_in / nlon_out > 1 query column wo sees input columns ws + t + ps * wo.  The plan removes that stride:
- * input latitude hi is split into ps "virtual latitudes" hi * ps + par, the columns {par, par + ps, ...}, each with
- * nlon_out columns, and every CSR run into one run per column class it touches.  On virtual latitudes the
- * neighborhood has unit stride in wo for any ps, and that is the only form the kernels implement.  (ps = 1: virtual
- * and real latitudes coincide.)
+ * The longitude ratio ps > 1 is removed in the plan, not in the kernels: every latitude of the FINER grid is split into
+ * ps "virtual latitudes" (real latitude * ps + column class par: its columns par, par + ps, ...), each with
+ * W = min(nlon_in, nlon_out) columns, and every CSR run into one run per column class it touches.  On virtual latitudes
+ * all neighborhoods have unit stride: query column j of virtual output latitude vo sees columns (ws + t + j) mod W of
+ * virtual input latitude vi, t in [0, len); that is the only form the kernels implement.  (The coarser grid's virtual
+ * latitudes are its real ones; with nlon_in == nlon_out nothing is split.)
+ *   nvin = nlat_in * (nlon_in / W),  nvout = nlat_out * (nlon_out / W)
  *
- * gather runs   grouped by output latitude ho:  lat = virtual input latitude, aux = real input latitude;
- *               neighbors are its columns (ws + t + wo) mod nlon_out, t in [0, len)
- * scatter runs  the same runs grouped by virtual input latitude: lat = ho, aux = 0
+ * gather runs   grouped by virtual output latitude:  lat = virtual input latitude, aux = real input latitude
+ * scatter runs  the same runs grouped by virtual input latitude: lat = virtual output latitude, aux = real output latitude;
+ *               key column j is seen by query columns (j - ws - t) mod W
  *
  * plus, for each grouping, the group offsets and a launch order of the groups.  The order lists first the
  * latitudes whose runs are long (ndense of them, most work first) and then the others (most work first); starting
@@ -66,8 +73,8 @@ int s2attn_abi_version(void);
  *
  * s2attn_plan_count   number of runs the CSR decomposes into, or a negative error.
  * s2attn_plan_build   fills caller-allocated host arrays:
- *     gather_off  [nlat_out+1]      gather_runs  [4*nruns]   gather_order  [nlat_out]
- *     scatter_off [nlat_in*ps+1]    scatter_runs [4*nruns]   scatter_order [nlat_in*ps]
+ *     gather_off  [nvout+1]   gather_runs  [4*nruns]   gather_order  [nvout]
+ *     scatter_off [nvin+1]    scatter_runs [4*nruns]   scatter_order [nvin]
  *     ndense [2]  number of long-run latitudes at the front of gather_order and of scatter_order
  * The caller copies the six arrays to the device and passes them, with the two counts, in s2attn_plan.
  */
@@ -80,12 +87,12 @@ int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nn
                       int32_t *ndense);
 
 typedef struct s2attn_plan {
-    const int32_t *gather_off;    /* device, [nlat_out+1] */
-    const int32_t *gather_runs;   /* device, [4*nruns]    */
-    const int32_t *gather_order;  /* device, [nlat_out]   */
-    const int32_t *scatter_off;   /* device, [nlat_in*ps+1]  (backward only) */
-    const int32_t *scatter_runs;  /* device, [4*nruns]       (backward only) */
-    const int32_t *scatter_order; /* device, [nlat_in*ps]    (backward only) */
+    const int32_t *gather_off;    /* device, [nvout+1]  */
+    const int32_t *gather_runs;   /* device, [4*nruns]  */
+    const int32_t *gather_order;  /* device, [nvout]    */
+    const int32_t *scatter_off;   /* device, [nvin+1]   (backward only) */
+    const int32_t *scatter_runs;  /* device, [4*nruns]  (backward only) */
+    const int32_t *scatter_order; /* device, [nvin]     (backward only) */
     int64_t nruns;
     int32_t gather_ndense;  /* leading entries of gather_order that go to the dense kernels  */
     int32_t scatter_ndense; /* leading entries of scatter_order that go to the dense kernels */
@@ -101,7 +108,8 @@ typedef struct s2attn_shape {
 
 /*
  * Forward.  Replaces attention_kernels::forward (attention_interface.cpp:114-116;
- * CUDA implementation s2_attention_fwd_cuda, attention_cuda_fwd.cu:539-633).
+ * CUDA implementations s2_attention_fwd_cuda, attention_cuda_fwd.cu:539-633, and the up-sampling
+ * kernels of attention_cuda_fwd_upsample.cu:70-289).
  *   y = sum_j a_j v_j / sum_j a_j,  a_j = exp(q.k_j - max) * quad_weights[hi_j]
  * y must not alias an input.
  */

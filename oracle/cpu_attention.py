@@ -60,7 +60,7 @@ def _dims(k, v, q, nh):
     B, Hi, Wi, CK = k.shape
     _, Ho, Wo, _ = q.shape
     CV = v.shape[3]
-    assert CK % nh == 0 and CV % nh == 0 and Wi % Wo == 0
+    assert CK % nh == 0 and CV % nh == 0 and (Wi % Wo == 0 or Wo % Wi == 0)
     return B, Hi, Wi, Ho, Wo, CK // nh, CV // nh
 
 
@@ -128,13 +128,34 @@ def dense_mask(col_idx, row_off, Hi, Wi, Ho, Wo):
     return M.reshape(Ho * Wo, Hi * Wi)
 
 
+def dense_mask_upsample(col_idx, row_off, Hi, Wi, Ho, Wo):
+    """Boolean [Ho*Wo, Hi*Wi] mask of the up-sampling (scatter) direction: psi row hi lists output points (ho, wo) seen from
+    input column 0; input column wi sees them shifted by (Wo / Wi) * wi in longitude (attention_torch.py:613-621)."""
+    ps = Wo // Wi
+    M = torch.zeros((Ho, Wo, Hi, Wi), dtype=torch.bool)
+    ci, ro = _i64(col_idx), _i64(row_off)
+    for hi in range(Hi):
+        cols = ci[ro[hi] : ro[hi + 1]]
+        ho = cols // Wo
+        wo = cols % Wo
+        for wi in range(Wi):
+            M[ho, (wo + ps * wi) % Wo, hi, wi] = True
+    return M.reshape(Ho * Wo, Hi * Wi)
+
+
+def is_upsample(Wi, Wo):
+    """Direction rule of the reference (attention.py:337): scatter iff nlon_out is a proper multiple of nlon_in."""
+    return Wo % Wi == 0 and Wi % Wo != 0
+
+
 def dense_attention_f64(k, v, q, quad_weights, col_idx, row_off, nh):
     """
     Textbook formulation, differentiable: softmax over the masked neighborhood of
-    q.k + log(quad weight), times v, in float64.  Small grids only (dense mask).
+    q.k + log(quad weight), times v, in float64.  Small grids only (dense mask).  Serves both
+    directions: the mask is the only thing that differs (attention_torch.py:74-125 and 582-650).
     """
     B, Hi, Wi, Ho, Wo, Ck, Cv = _dims(k, v, q, nh)
-    M = dense_mask(col_idx, row_off, Hi, Wi, Ho, Wo)
+    M = (dense_mask_upsample if is_upsample(Wi, Wo) else dense_mask)(col_idx, row_off, Hi, Wi, Ho, Wo)
     kd = k.to(torch.float64).reshape(B, Hi * Wi, nh, Ck).permute(0, 2, 1, 3)
     vd = v.to(torch.float64).reshape(B, Hi * Wi, nh, Cv).permute(0, 2, 1, 3)
     qd = q.to(torch.float64).reshape(B, Ho * Wo, nh, Ck).permute(0, 2, 1, 3)

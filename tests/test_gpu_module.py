@@ -41,7 +41,7 @@ def _reference_module_forward(m, xq, xk, xv):
 
 
 MODULE_CASES = [
-    # B, C, Cout, heads, in_shape, out_shape, grid_in, grid_out, qknorm   (gather rows of tests/test_attention.py:89-110,126-146)
+    # B, C, Cout, heads, in_shape, out_shape, grid_in, grid_out, qknorm   (rows of tests/test_attention.py:89-110,126-146)
     (4, 4, 4, 1, (6, 12), (6, 12), "equiangular", "equiangular", False),
     (4, 4, 4, 2, (6, 12), (6, 12), "equiangular", "equiangular", False),
     (4, 4, 8, 4, (6, 12), (6, 12), "equiangular", "equiangular", False),
@@ -56,6 +56,11 @@ MODULE_CASES = [
     (4, 4, 4, 2, (6, 12), (6, 12), "equiangular", "equiangular", True),
     (4, 8, 4, 4, (12, 24), (6, 12), "equiangular", "equiangular", True),
     (2, 64, 64, 4, (24, 48), (24, 48), "equiangular", "equiangular", False),
+    # up-sampling rows (nlon_out a multiple of nlon_in): psi keyed by input latitude, default radius from the input grid
+    (4, 4, 4, 1, (6, 12), (12, 24), "equiangular", "equiangular", False),
+    (4, 8, 4, 4, (6, 12), (12, 24), "equiangular", "equiangular", False),
+    (2, 4, 4, 2, (3, 6), (12, 24), "legendre-gauss", "equiangular", True),
+    (2, 4, 8, 1, (5, 4), (9, 12), "equiangular", "equiangular", False),
 ]
 
 

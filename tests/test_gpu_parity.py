@@ -209,3 +209,54 @@ def test_backward_from_saved_forward_results(case, dtype):
         else:
             rms = want.pow(2).mean().sqrt().item()
             assert_close(name, got, want, rtol=2e-2, atol=2e-2 * rms)
+
+
+# (B, nh, ck, cv, in_shape, out_shape, grid_in, grid_out, theta_cutoff): up-sampling (scatter) direction, the reference's own
+# shape matrix for it (tests/test_attention.py, rows with nlon_out > nlon_in) plus wide grids for every kernel family
+UPSAMPLE_CASES = [
+    (2, 1, 4, 4, (6, 12), (12, 24), "equiangular", "equiangular", None),
+    (2, 2, 2, 2, (6, 12), (6, 24), "equiangular", "equiangular", None),
+    (1, 1, 4, 4, (3, 6), (12, 24), "equiangular", "equiangular", None),
+    (1, 2, 3, 5, (5, 4), (9, 12), "equiangular", "equiangular", 0.9),
+    (1, 1, 4, 4, (6, 12), (12, 24), "legendre-gauss", "legendre-gauss", None),
+    (1, 2, 8, 8, (10, 100), (10, 200), "equiangular", "equiangular", 0.35),
+    (1, 1, 32, 32, (12, 70), (24, 140), "equiangular", "equiangular", 0.4),
+    (1, 1, 48, 40, (6, 12), (12, 24), "equiangular", "equiangular", 0.7),
+    (1, 2, 64, 64, (8, 40), (16, 80), "legendre-gauss", "equiangular", 0.6),
+]
+
+
+@pytest.mark.parametrize("case", UPSAMPLE_CASES, ids=lambda c: f"B{c[0]}h{c[1]}ck{c[2]}cv{c[3]}_{c[4][0]}x{c[4][1]}to{c[5][0]}x{c[5][1]}_{c[6][:3]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_upsampling_direction(case, dtype):
+    """nlon_out a multiple of nlon_in: psi keyed by input latitude; y and all gradients against the dense float64 softmax over the
+    scatter-direction mask, through both backward entry points."""
+    from torch_harmonics_amd import ops
+
+    B, nh, ck, cv, ins, outs, gi, go, tc = case
+    print(f"case {case} {dtype}", flush=True)
+    tc = math.pi / (ins[0] - 1) if tc is None else tc
+    col_idx, row_off = ogeo.neighborhood_csr(outs, ins, go, gi, tc)  # grids swapped: rows index the input grid
+    quad = ogeo.attention_quad_weights(ins[0], ins[1], gi)
+    k, v, q, dy = randn_inputs(B, ins[0], ins[1], outs[0], outs[1], nh, ck, cv, scale=0.5 if dtype != torch.float32 else 1.0)
+    k, v, q, dy = [t.to(dtype).float() for t in (k, v, q, dy)]
+
+    kr, vr, qr = [t.double().requires_grad_(True) for t in (k, v, q)]
+    y64 = oracle.dense_attention_f64(kr, vr, qr, quad, col_idx, row_off, nh)
+    y64.backward(dy.double())
+    want = (y64.detach(), kr.grad, vr.grad, qr.grad)
+
+    dev = torch.device("cuda", 0)
+    kd, vd, qd, gd = [t.to(device=dev, dtype=dtype) for t in (k, v, q, dy)]
+    wd, cd, rd = quad.to(dev), col_idx.to(dev), row_off.to(dev)
+    geo = (nh, ins[1], outs[0], outs[1])
+    y, lse = ops.forward_lse(kd, vd, qd, wd, cd, rd, *geo)
+    assert torch.equal(y, ops.forward(kd, vd, qd, wd, cd, rd, *geo))
+    for name, grads in (("saved", ops.backward_saved(kd, vd, qd, gd, y, lse, wd, cd, rd, *geo)), ("recompute", ops.backward(kd, vd, qd, gd, wd, cd, rd, *geo))):
+        torch.cuda.synchronize()
+        for tname, got, w in zip(("y", "dk", "dv", "dq"), (y,) + tuple(grads), want):
+            if dtype == torch.float32:
+                assert_close(f"{tname} ({name})", got, w, **F32_TOL)
+            else:
+                rms = w.pow(2).mean().sqrt().item()
+                assert_close(f"{tname} ({name})", got, w, rtol=2e-2, atol=2e-2 * rms)

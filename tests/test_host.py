@@ -59,36 +59,46 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
 
 
 def _pairs_from_csr(col, roff, Wi, Wo):
-    ps = Wi // Wo
+    """(ho, wo, hi, wi) pairs of a CSR.  Gather direction (Wi = ps Wo): rows are ho, entries (hi, wi) at wo = 0, shifted by
+    ps per output column (attention_torch.py:97-104).  Scatter direction (Wo = ps Wi, ps > 1): rows are hi, entries (ho, wo)
+    at wi = 0, shifted by ps per input column (attention_torch.py:613-621)."""
     ref = Counter()
-    for ho in range(len(roff) - 1):
-        for z in range(int(roff[ho]), int(roff[ho + 1])):
-            hi, wi = divmod(int(col[z]), Wi)
-            for wo in range(Wo):
-                ref[(ho, wo, hi, (wi + ps * wo) % Wi)] += 1
+    up = Wo % Wi == 0 and Wo != Wi
+    for r in range(len(roff) - 1):
+        for z in range(int(roff[r]), int(roff[r + 1])):
+            if up:
+                ho, wo = divmod(int(col[z]), Wo)
+                for wi in range(Wi):
+                    ref[(ho, (wo + (Wo // Wi) * wi) % Wo, r, wi)] += 1
+            else:
+                hi, wi = divmod(int(col[z]), Wi)
+                for wo in range(Wo):
+                    ref[(r, wo, hi, (wi + (Wi // Wo) * wo) % Wi)] += 1
     return ref
 
 
 def _pairs_from_plan(arrays, Hi, Wi, Ho, Wo):
     """Expands both run groupings back into (ho, wo, hi, wi) pairs the way the kernels index them: runs live on
-    virtual input latitudes hi * ps + par (the columns par, par + ps, ... of latitude hi, Wo of them), where query
-    column wo sees virtual columns (ws + t + wo) mod Wo."""
+    virtual latitudes (real latitude * ps + column class, W = min(Wi, Wo) columns each) of the finer grid, where query
+    column j sees key columns (ws + t + j) mod W and key column j is seen by query columns (j - ws - t) mod W."""
     goff, gruns, gorder, soff, sruns, sorder = [a.numpy() for a in arrays]
-    ps = Wi // Wo
+    up = Wo % Wi == 0 and Wo != Wi
+    psk, psq, W = (1, Wo // Wi, Wi) if up else (Wi // Wo, 1, Wo)
     gather, scatter = Counter(), Counter()
-    for ho in range(Ho):
-        for ri in range(goff[ho], goff[ho + 1]):
-            vlat, ws, ln, hi = (int(x) for x in gruns[ri])
-            assert hi == vlat // ps and 0 <= ws < Wo and 1 <= ln <= Wo
-            for wo in range(Wo):
+    for vo in range(Ho * psq):
+        for ri in range(goff[vo], goff[vo + 1]):
+            vi, ws, ln, hi = (int(x) for x in gruns[ri])
+            assert hi == vi // psk and 0 <= ws < W and 1 <= ln <= W
+            for j in range(W):
                 for t in range(ln):
-                    gather[(ho, wo, hi, ((ws + t + wo) % Wo) * ps + vlat % ps)] += 1
-    for vlat in range(Hi * ps):
-        for ri in range(soff[vlat], soff[vlat + 1]):
-            ho, ws, ln, _ = (int(x) for x in sruns[ri])
-            for j in range(Wo):  # virtual column j of this virtual latitude is seen by wo = j - ws - t
+                    gather[(vo // psq, j * psq + vo % psq, hi, ((ws + t + j) % W) * psk + vi % psk)] += 1
+    for vi in range(Hi * psk):
+        for ri in range(soff[vi], soff[vi + 1]):
+            vo, ws, ln, ho = (int(x) for x in sruns[ri])
+            assert ho == vo // psq
+            for j in range(W):
                 for t in range(ln):
-                    scatter[(ho, (j - ws - t) % Wo, vlat // ps, j * ps + vlat % ps)] += 1
+                    scatter[(ho, ((j - ws - t) % W) * psq + vo % psq, vi // psk, j * psk + vi % psk)] += 1
     return gather, scatter, gorder, sorder
 
 
@@ -101,17 +111,27 @@ def _pairs_from_plan(arrays, Hi, Wi, Ho, Wo):
         ((9, 12), (5, 4), "equiangular", "equiangular", None),
         ((12, 24), (6, 12), "legendre-gauss", "legendre-gauss", 0.7),
         ((6, 12), (6, 12), "equiangular", "equiangular", 7.0),
+        # scatter direction (up-sampling): psi keyed by input latitude
+        ((6, 12), (12, 24), "equiangular", "equiangular", None),
+        ((5, 4), (9, 12), "equiangular", "equiangular", None),
+        ((6, 8), (12, 24), "legendre-gauss", "equiangular", 0.9),
     ],
 )
 def test_plan_covers_exactly_the_csr_pairs(ins, outs, gi, go, tc):
-    col, roff, _ = precompute_neighborhood_s2(ins, outs, gi, go, tc)
+    up = outs[1] % ins[1] == 0 and outs[1] != ins[1]
+    if up:  # rows index the (coarser) input grid, columns the output grid (attention.py:372-387)
+        col, roff, _ = precompute_neighborhood_s2(outs, ins, go, gi, tc if tc is not None else math.pi / (ins[0] - 1))
+    else:
+        col, roff, _ = precompute_neighborhood_s2(ins, outs, gi, go, tc)
     arrays, nruns, ndense = build_host_plan(col, roff, ins[0], ins[1], outs[0], outs[1])
     ref = _pairs_from_csr(col, roff, ins[1], outs[1])
     gather, scatter, gorder, sorder = _pairs_from_plan(arrays, ins[0], ins[1], outs[0], outs[1])
     assert gather == ref and scatter == ref
-    assert sorted(gorder.tolist()) == list(range(outs[0])) and sorted(sorder.tolist()) == list(range(ins[0] * (ins[1] // outs[1])))
-    lens = (roff[1:] - roff[:-1]).tolist()
-    assert all(lens[gorder[i]] >= lens[gorder[i + 1]] for i in range(outs[0] - 1)), "rows must be ordered longest first"
+    psk, psq = (1, outs[1] // ins[1]) if up else (ins[1] // outs[1], 1)
+    assert sorted(gorder.tolist()) == list(range(outs[0] * psq)) and sorted(sorder.tolist()) == list(range(ins[0] * psk))
+    if not up:
+        lens = (roff[1:] - roff[:-1]).tolist()
+        assert all(lens[gorder[i]] >= lens[gorder[i + 1]] for i in range(outs[0] - 1)), "rows must be ordered longest first"
     assert nruns <= col.numel()
 
 
@@ -228,9 +248,17 @@ def test_module_constructor_errors():
     with pytest.raises(ValueError, match="positive"):
         tha.NeighborhoodAttentionS2(4, (6, 12), (6, 12), theta_cutoff=0.0)
     with pytest.raises(NotImplementedError):
-        tha.NeighborhoodAttentionS2(4, (6, 12), (12, 24))  # upsampling
-    with pytest.raises(NotImplementedError):
         tha.NeighborhoodAttentionS2(4, (6, 12), (6, 12), optimized_kernel=False)
+
+
+def test_module_upsampling_direction_state():
+    """Up-sampling keys psi by input latitude and takes its default radius from the coarser (input) grid (attention.py:337-356,372-387)."""
+    m = tha.NeighborhoodAttentionS2(4, (6, 12), (12, 24))
+    assert m.upsample and m.psi_roff_idx.shape == (7,)
+    assert m.theta_cutoff == pytest.approx(math.pi / 5)
+    assert int(m.psi_col_idx.max()) < 12 * 24 and m.quad_weights.shape == (6,)
+    col, roff = ogeo.neighborhood_csr((12, 24), (6, 12), "equiangular", "equiangular", math.pi / 5)
+    assert torch.equal(m.psi_col_idx, col) and torch.equal(m.psi_roff_idx, roff)
 
 
 def test_module_forward_checks_shapes_and_has_no_cpu_path():
@@ -289,5 +317,5 @@ def test_operator_argument_errors():
         ops.forward(k, v, q, *psi, 2, 24, 6, 12)
     with pytest.raises(RuntimeError, match="only run on a ROCm GPU"):
         ops.permute_to_nhwc(torch.randn(1, 2, 3, 4))
-    with pytest.raises(NotImplementedError):
-        ops.forward(q, q[..., :4].contiguous(), k, *psi, 2, 12, 12, 24)  # upsampling direction
+    with pytest.raises(RuntimeError, match="integer multiple"):
+        ops.forward(k[:, :, :10].contiguous(), v[:, :, :10].contiguous(), q, *psi, 2, 10, 6, 12)

@@ -139,3 +139,47 @@ def test_restricted_row_range_accumulates_only_those_queries():
     y = o.forward_f64(k, v, q, w, col, roff, nh, ho_range=(2, 5))
     assert torch.equal(y[:, :2], torch.zeros_like(y[:, :2])) and torch.equal(y[:, 5:], torch.zeros_like(y[:, 5:]))
     assert torch.allclose(y[:, 2:5], o.forward_f64(k, v, q, w, col, roff, nh)[:, 2:5])
+
+
+# ---- up-sampling (scatter) direction: only the mask differs from the gather direction ---------------------------------
+
+
+def _geodesic_mask(in_shape, out_shape, grid_in, grid_out, cutoff):
+    """[Ho*Wo, Hi*Wi] from first principles: great-circle distance (haversine) between every output and input point."""
+    (Hi, Wi), (Ho, Wo) = in_shape, out_shape
+    th_i = g.colatitudes_and_weights(Hi, grid_in)[0].double()
+    th_o = g.colatitudes_and_weights(Ho, grid_out)[0].double()
+    lat_i = (math.pi / 2 - th_i).view(1, 1, Hi, 1)
+    lat_o = (math.pi / 2 - th_o).view(Ho, 1, 1, 1)
+    lon_i = (2 * math.pi * torch.arange(Wi, dtype=torch.float64) / Wi).view(1, 1, 1, Wi)
+    lon_o = (2 * math.pi * torch.arange(Wo, dtype=torch.float64) / Wo).view(1, Wo, 1, 1)
+    hav = torch.sin((lat_i - lat_o) / 2) ** 2 + torch.cos(lat_i) * torch.cos(lat_o) * torch.sin((lon_i - lon_o) / 2) ** 2
+    dist = 2 * torch.asin(hav.clamp(0, 1).sqrt())
+    return (dist <= 1.001 * cutoff).reshape(Ho * Wo, Hi * Wi)
+
+
+@pytest.mark.parametrize(
+    "ins,outs,gi,go,tc",
+    [
+        ((6, 12), (12, 24), "equiangular", "equiangular", math.pi / 5),
+        ((5, 4), (9, 12), "equiangular", "equiangular", 0.9),
+        ((6, 8), (12, 24), "legendre-gauss", "equiangular", 0.7),
+        ((4, 6), (7, 24), "lobatto", "legendre-gauss", 1.1),
+    ],
+)
+def test_upsampling_mask_is_the_geodesic_disk_and_the_transpose_of_the_swapped_gather_mask(ins, outs, gi, go, tc):
+    """The scatter-direction psi (rows = input latitude, built with the grids swapped, attention.py:372-387) expanded by
+    dense_mask_upsample must be (a) the set of pairs closer than the cutoff and (b) the transpose of the gather mask of
+    the swapped problem, in which the coarse grid queries the fine one."""
+    col, roff = g.neighborhood_csr(outs, ins, go, gi, tc)  # swapped call: rows index the input grid
+    M = o.dense_mask_upsample(col, roff, ins[0], ins[1], outs[0], outs[1])
+    assert torch.equal(M, _geodesic_mask(ins, outs, gi, go, tc))
+    Mswapped = o.dense_mask(col, roff, outs[0], outs[1], ins[0], ins[1])  # [Hi*Wi (queries), Ho*Wo (keys)]
+    assert torch.equal(M, Mswapped.t())
+    assert o.is_upsample(ins[1], outs[1]) and not o.is_upsample(outs[1], ins[1]) and not o.is_upsample(12, 12)
+
+
+def test_gather_mask_is_the_geodesic_disk_too():
+    ins, outs, tc = (12, 24), (6, 8), 0.6
+    col, roff = g.neighborhood_csr(ins, outs, "equiangular", "legendre-gauss", tc)
+    assert torch.equal(o.dense_mask(col, roff, 12, 24, 6, 8), _geodesic_mask(ins, outs, "equiangular", "legendre-gauss", tc))

@@ -41,7 +41,8 @@ class NeighborhoodAttentionS2(nn.Module):
     in_channels : int
         channels of the input signal
     in_shape, out_shape : (nlat, nlon)
-        input (key/value) and output (query) grids; ``nlon_in`` must be a multiple of ``nlon_out``
+        input (key/value) and output (query) grids; ``nlon_in`` must be a multiple of ``nlon_out`` (self-attention,
+        down-sampling) or ``nlon_out`` a multiple of ``nlon_in`` (up-sampling)
     grid_in, grid_out : str
         ``"equiangular"``, ``"legendre-gauss"``, ``"lobatto"`` or ``"equiangular-trapezoidal"``
     num_heads : int
@@ -84,8 +85,6 @@ class NeighborhoodAttentionS2(nn.Module):
         self.upsample = (self.nlon_out % self.nlon_in == 0) and (self.nlon_in % self.nlon_out != 0)
         if not (self.nlon_in % self.nlon_out == 0 or self.upsample):
             raise ValueError(f"either nlon_in ({self.nlon_in}) must be an integer multiple of nlon_out ({self.nlon_out}), or vice versa, for the attention p-shift to be exact")
-        if self.upsample:
-            raise NotImplementedError("upsampling attention (nlon_out > nlon_in) is not implemented by the HIP kernels")
         if not optimized_kernel:
             raise NotImplementedError("optimized_kernel=False selects a pure-PyTorch loop in the reference; this package ships the HIP kernels only")
         self.optimized_kernel = True
@@ -95,7 +94,11 @@ class NeighborhoodAttentionS2(nn.Module):
         self.k_channels = in_channels if k_channels is None else k_channels
         self.out_channels = in_channels if out_channels is None else out_channels
 
-        self.theta_cutoff = torch.pi / float(self.nlat_out - 1) if theta_cutoff is None else theta_cutoff
+        # default radius: one latitude spacing of the coarser grid (the input grid when up-sampling, attention.py:352-356)
+        if theta_cutoff is None:
+            self.theta_cutoff = torch.pi / float((self.nlat_in if self.upsample else self.nlat_out) - 1)
+        else:
+            self.theta_cutoff = theta_cutoff
         if self.theta_cutoff <= 0.0:
             raise ValueError("Error, theta_cutoff has to be positive.")
 
@@ -108,7 +111,12 @@ class NeighborhoodAttentionS2(nn.Module):
         _, wgl = precompute_latitudes(self.nlat_in, grid=grid_in)
         self.register_buffer("quad_weights", 2.0 * torch.pi * wgl.to(dtype=torch.float32) / self.nlon_in, persistent=False)
 
-        col_idx, row_off, row_idx = precompute_neighborhood_s2(in_shape, out_shape, grid_in=grid_in, grid_out=grid_out, theta_cutoff=self.theta_cutoff)
+        # Up-sampling keys psi by the (coarser) input latitude: rows hi, columns ho * nlon_out + wo of the output points inside
+        # the disk around input point (hi, 0) -- the same construction with the two grids swapped (attention.py:372-387).
+        if self.upsample:
+            col_idx, row_off, row_idx = precompute_neighborhood_s2(out_shape, in_shape, grid_in=grid_out, grid_out=grid_in, theta_cutoff=self.theta_cutoff)
+        else:
+            col_idx, row_off, row_idx = precompute_neighborhood_s2(in_shape, out_shape, grid_in=grid_in, grid_out=grid_out, theta_cutoff=self.theta_cutoff)
         self.register_buffer("psi_row_idx", row_idx, persistent=False)
         self.register_buffer("psi_col_idx", col_idx, persistent=False)
         self.register_buffer("psi_roff_idx", row_off, persistent=False)

@@ -169,7 +169,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
     const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
     const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
     const bool mine = c < nvalid;
-    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
 
     uint4 qop[NS]; // B operand of S^T = K Q^T: channels 32 s + 8 qd .. + 8 of column c
     {
@@ -298,7 +298,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
     const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
     const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
     const bool mine = c < nvalid;
-    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
     const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
 
     uint4 qop[NS], gop[NS];
@@ -453,13 +453,14 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
     Run run = {0, 0, 0, 0};
     Tile qt, gt;
     float2 st = make_float2(0.f, 0.f);
-    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldb + 16u * (lane % Tile::CPR);
+    const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbq + 16u * (lane % Tile::CPR);
     auto fetch = [&](const Run &rn, int p) {
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
         unsigned off[Tile::NIT];
-        Tile::offsets(off, lane_off, lane, c0, a.Wo, ldb);
-        const size_t lat_off = (size_t)rn.lat * a.Wo * ldb;
+        Tile::offsets(off, lane_off, lane, c0, a.Wo, ldbq);
+        const size_t lat_off = (size_t)query_row(a, rn.lat, rn.pad) * ldb;
         qt.fetch(qy + lat_off, off);
         gt.fetch(gy + lat_off, off);
         int col = c0 + lane; // lanes 0..31 fetch the statistics of the staged rows

@@ -41,7 +41,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 4; }
+extern "C" int s2attn_abi_version(void) { return 5; }
 
 namespace s2 {
 
@@ -225,7 +225,8 @@ struct Args {
     const int *goff, *gorder, *soff, *sorder;
     const Run *gruns, *sruns;
     int B, nh, Hi, Wi, Ho, Wo, dk_, dv_, pscale;
-    int kps; // real longitude ratio nlon_in / nlon_out; see key_point()
+    int kps; // nlon_in / nlon_out when the input grid is the finer one, else 1; see key_point()
+    int qps; // nlon_out / nlon_in when the output grid is the finer one, else 1; see query_point()
     int tile_rows; // LDS rows per staged band
     int row_first; // first entry of gorder / sorder this launch covers (dense rows come first, see s2attn_plan_split)
 };
@@ -241,6 +242,14 @@ __device__ inline long key_point(const Args &a, int b, int vlat, int rlat)
     return ((long)b * a.Hi + (long)rlat * a.kps) * a.Wi + (vlat - rlat * a.kps);
 }
 __device__ inline long key_row(const Args &a, int vlat, int rlat) { return (long)rlat * a.kps * a.Wi + (vlat - rlat * a.kps); }
+// The same on the query side for the up-sampling direction (nlon_out = qps * nlon_in): Ho = nlat_out * qps virtual output
+// latitudes of Wo = nlon_in columns; scatter runs carry the real output latitude in Run::pad.  The per-point statistics
+// (lse, stats) are private to the library and simply indexed by virtual coordinates.
+__device__ inline long query_point(const Args &a, int b, int vlat, int rlat)
+{
+    return ((long)b * a.Ho + (long)rlat * a.qps) * a.Wo + (vlat - rlat * a.qps);
+}
+__device__ inline long query_row(const Args &a, int vlat, int rlat) { return (long)rlat * a.qps * a.Wo + (vlat - rlat * a.qps); }
 
 // ---------------------------------------------------------------------------------
 // forward:  y = sum_j a_j v_j / sum_j a_j
@@ -272,7 +281,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd
     T *y = static_cast<T *>(a.y);
 
     // q for this lane, pre-multiplied by log2(e)
-    stage_rows<T, P, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, wo0, a.Wo, nvalid, lane);
+    stage_rows<T, P, VEC>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, wo0, a.Wo, nvalid, lane);
     __syncthreads();
     float qr[P], acc[P];
 #pragma unroll
@@ -340,7 +349,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd
     for (int c = 0; c < P; c += 4)
         *reinterpret_cast<float4 *>(Ks + lane * LS + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
     __syncthreads();
-    unstage_rows<T, P, VEC>(y + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, Ks, ldv, a.dv_, wo0, nvalid, lane);
+    unstage_rows<T, P, VEC>(y + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, Ks, ldv * a.qps, a.dv_, wo0, nvalid, lane);
 }
 
 // ---------------------------------------------------------------------------------
@@ -375,8 +384,8 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dq_
     const T *gy = static_cast<const T *>(a.dy);
     T *dq = static_cast<T *>(a.dq);
 
-    stage_rows<T, P, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, wo0, a.Wo, nvalid, lane);
-    stage_rows<T, P, VEC>(Vs, gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, ldv, a.dv_, wo0, a.Wo, nvalid, lane);
+    stage_rows<T, P, VEC>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, wo0, a.Wo, nvalid, lane);
+    stage_rows<T, P, VEC>(Vs, gy + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, ldv * a.qps, a.dv_, wo0, a.Wo, nvalid, lane);
     __syncthreads();
     float qr[P], gr[P], Ak[P], Akg[P];
 #pragma unroll
@@ -461,7 +470,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dq_
             = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
                           (Akg[c + 3] - I * Ak[c + 3]) * inv);
     __syncthreads();
-    unstage_rows<T, P, VEC>(dq + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, Ks, ldk, a.dk_, wo0, nvalid, lane);
+    unstage_rows<T, P, VEC>(dq + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, Ks, ldk * a.qps, a.dk_, wo0, nvalid, lane);
 }
 
 // ---------------------------------------------------------------------------------
@@ -529,8 +538,8 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
         const int a0 = d0 / ps;
         const int span = (d0 + nvalid - 1) / ps - a0; // al of the last valid lane
         const int U = (run.len + ps - 1) / ps;
-        const T *ql = qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_;
-        const T *gl = gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_;
+        const T *ql = qy + query_point(a, b, ho, run.pad) * ldk + (long)h * a.dk_;
+        const T *gl = gy + query_point(a, b, ho, run.pad) * ldv + (long)h * a.dv_;
         const float2 *sl = a.stats + ((long)bh * a.Ho + ho) * a.Wo;
 
         for (int u0 = 0; u0 < U; u0 += TL) {
@@ -539,8 +548,8 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
             if (c0 < 0) c0 += a.Wo;
             const int nrows = span + UL;
             __syncthreads();
-            stage_rows<T, P, VEC>(Qs, ql, ldk, a.dk_, c0, a.Wo, nrows, lane);
-            stage_rows<T, P, VEC>(Gs, gl, ldv, a.dv_, c0, a.Wo, nrows, lane);
+            stage_rows<T, P, VEC>(Qs, ql, ldk * a.qps, a.dk_, c0, a.Wo, nrows, lane);
+            stage_rows<T, P, VEC>(Gs, gl, ldv * a.qps, a.dv_, c0, a.Wo, nrows, lane);
             for (int r = lane; r < nrows; r += TQ) {
                 int col = c0 + r;
                 while (col >= a.Wo) col -= a.Wo;
@@ -641,7 +650,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
     const T *qy = static_cast<const T *>(a.q);
     T *y = static_cast<T *>(a.y);
 
-    stage_rows<T, PT, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, PT, VEC>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, lane);
     __syncthreads();
     float qr[32], acc[32];
 #pragma unroll
@@ -707,7 +716,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
     for (int c = 0; c < 32; c += 4)
         *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
     __syncthreads();
-    unstage_rows<T, PT, VEC>(y + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, Ks, ldv, a.dv_, w0, nvalid, lane);
+    unstage_rows<T, PT, VEC>(y + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, Ks, ldv * a.qps, a.dv_, w0, nvalid, lane);
 }
 
 template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void dq_wide_kernel(const Args a)
@@ -723,8 +732,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
     const T *gy = static_cast<const T *>(a.dy);
     T *dq = static_cast<T *>(a.dq);
 
-    stage_rows<T, PT, VEC>(Ks, qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, ldk, a.dk_, w0, a.Wo, nvalid, lane);
-    stage_rows<T, PT, VEC>(Vs, gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_, ldv, a.dv_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, PT, VEC>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, PT, VEC>(Vs, gy + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, ldv * a.qps, a.dv_, w0, a.Wo, nvalid, lane);
     __syncthreads();
     float qr[32], gr[32], Ak[32], Akg[32];
 #pragma unroll
@@ -807,7 +816,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
             = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
                           (Akg[c + 3] - I * Ak[c + 3]) * inv);
     __syncthreads();
-    unstage_rows<T, PT, VEC>(dq + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_, Ks, ldk, a.dk_, w0, nvalid, lane);
+    unstage_rows<T, PT, VEC>(dq + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, Ks, ldk * a.qps, a.dk_, w0, nvalid, lane);
 }
 
 template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void dkdv_wide_kernel(const Args a)
@@ -848,8 +857,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
         const int a0 = d0 / ps;
         const int span = (d0 + nvalid - 1) / ps - a0;
         const int U = (run.len + ps - 1) / ps;
-        const T *ql = qy + ((long)(b * a.Ho + ho) * a.Wo) * ldk + (long)h * a.dk_;
-        const T *gl = gy + ((long)(b * a.Ho + ho) * a.Wo) * ldv + (long)h * a.dv_;
+        const T *ql = qy + query_point(a, b, ho, run.pad) * ldk + (long)h * a.dk_;
+        const T *gl = gy + query_point(a, b, ho, run.pad) * ldv + (long)h * a.dv_;
         const float2 *sl2 = a.stats + ((long)bh * a.Ho + ho) * a.Wo;
         for (int u0 = 0; u0 < U; u0 += TL) {
             const int UL = min(TL, U - u0);
@@ -857,8 +866,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
             if (c0 < 0) c0 += a.Wo;
             const int nrows = span + UL;
             __syncthreads();
-            stage_rows<T, PT, VEC>(Qs, ql, ldk, a.dk_, c0, a.Wo, nrows, lane);
-            stage_rows<T, PT, VEC>(Gs, gl, ldv, a.dv_, c0, a.Wo, nrows, lane);
+            stage_rows<T, PT, VEC>(Qs, ql, ldk * a.qps, a.dk_, c0, a.Wo, nrows, lane);
+            stage_rows<T, PT, VEC>(Gs, gl, ldv * a.qps, a.dv_, c0, a.Wo, nrows, lane);
             for (int r = lane; r < nrows; r += TQ) {
                 int col = c0 + r;
                 while (col >= a.Wo) col -= a.Wo;
@@ -971,10 +980,10 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kern
 
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * a.dk_;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * a.dv_;
-    const T *qy = static_cast<const T *>(a.q) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldk + (size_t)h * a.dk_;
-    T *y = static_cast<T *>(a.y) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldv + (size_t)h * a.dv_;
+    const T *qy = static_cast<const T *>(a.q) + (size_t)query_point(a, b, ho, ho / a.qps) * ldk + (size_t)h * a.dk_;
+    T *y = static_cast<T *>(a.y) + (size_t)query_point(a, b, ho, ho / a.qps) * ldv + (size_t)h * a.dv_;
 
-    stage_rows<T, P, true>(Ks, qy, ldk, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, P, true>(Ks, qy, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, lane);
     __syncthreads();
     float qr[P], acc[P];
 #pragma unroll
@@ -1073,7 +1082,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void fwd_fast_kern
     for (int c = 0; c < P; c += 4)
         *reinterpret_cast<float4 *>(Ks + lane * LS + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
     __syncthreads();
-    unstage_rows<T, P, true>(y, Ks, ldv, a.dv_, w0, nvalid, lane);
+    unstage_rows<T, P, true>(y, Ks, ldv * a.qps, a.dv_, w0, nvalid, lane);
 }
 
 // backward dq + statistics, fast path
@@ -1093,12 +1102,12 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kerne
 
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * a.dk_;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * a.dv_;
-    const T *qy = static_cast<const T *>(a.q) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldk + (size_t)h * a.dk_;
-    const T *gy = static_cast<const T *>(a.dy) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldv + (size_t)h * a.dv_;
-    T *dq = static_cast<T *>(a.dq) + ((size_t)(b * a.Ho + ho) * a.Wo) * ldk + (size_t)h * a.dk_;
+    const T *qy = static_cast<const T *>(a.q) + (size_t)query_point(a, b, ho, ho / a.qps) * ldk + (size_t)h * a.dk_;
+    const T *gy = static_cast<const T *>(a.dy) + (size_t)query_point(a, b, ho, ho / a.qps) * ldv + (size_t)h * a.dv_;
+    T *dq = static_cast<T *>(a.dq) + (size_t)query_point(a, b, ho, ho / a.qps) * ldk + (size_t)h * a.dk_;
 
-    stage_rows<T, P, true>(Ks, qy, ldk, a.dk_, w0, a.Wo, nvalid, lane);
-    stage_rows<T, P, true>(Vs, gy, ldv, a.dv_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, P, true>(Ks, qy, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, P, true>(Vs, gy, ldv * a.qps, a.dv_, w0, a.Wo, nvalid, lane);
     __syncthreads();
     float qr[P], gr[P], Ak[P], Akg[P];
 #pragma unroll
@@ -1214,7 +1223,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kerne
             = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
                           (Akg[c + 3] - I * Ak[c + 3]) * inv);
     __syncthreads();
-    unstage_rows<T, P, true>(dq, Ks, ldk, a.dk_, w0, nvalid, lane);
+    unstage_rows<T, P, true>(dq, Ks, ldk * a.qps, a.dk_, w0, nvalid, lane);
 }
 
 // backward dk/dv, fast path (pscale == 1: the queries that see input longitude wi through run (ho, ws, len)
@@ -1268,8 +1277,8 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_ker
         c0 += (c0 < 0) ? a.Wo : 0;
         c0 += (c0 < 0) ? a.Wo : 0;
         const int nrows = nvalid - 1 + UL;
-        qb.fetch(qy + (size_t)rn.lat * a.Wo * ldk, ldk, c0, a.Wo, r0, cb);
-        gb.fetch(gy + (size_t)rn.lat * a.Wo * ldv, ldv, c0, a.Wo, r0, cb);
+        qb.fetch(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldk, ldk * a.qps, c0, a.Wo, r0, cb);
+        gb.fetch(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldv, ldv * a.qps, c0, a.Wo, r0, cb);
         const float2 *sl = stats + (size_t)rn.lat * a.Wo;
 #pragma unroll
         for (int it = 0; it < 2; it++) {
@@ -1439,7 +1448,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
     const bool mine = j < nvalid;
-    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? j : 0)) * a.qps;
 
     float qb[16];
     {
@@ -1630,7 +1639,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
     const bool mine = j < nvalid;
-    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? j : 0)) * a.qps;
 
     float qb[16], gb[16];
     {
@@ -1852,7 +1861,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
     const bool mine = j < nvalid;
-    const size_t pt = (size_t)(b * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? j : 0)) * a.qps;
     const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
 
     float qb[16], gb[16];
@@ -2057,8 +2066,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
         const bool fifth = !run_is_dense(rn.len);
-        qt.fetch(qy + (size_t)rn.lat * a.Wo * ldk, ldk, c0, a.Wo, lane, fifth);
-        gt.fetch(gy + (size_t)rn.lat * a.Wo * ldv, ldv, c0, a.Wo, lane, fifth);
+        qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldk, ldk * a.qps, c0, a.Wo, lane, fifth);
+        gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldv, ldv * a.qps, c0, a.Wo, lane, fifth);
         int col = c0 + lane; // lanes 0..39 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
         if (lane < MR) st = stats[(size_t)rn.lat * a.Wo + col];
@@ -2235,8 +2244,8 @@ int check_shape(const s2attn_shape *sh)
         return s2attn_fail(S2ATTN_E_INVALID, "batch and grid extents must be positive");
     if (sh->num_heads < 1) return s2attn_fail(S2ATTN_E_INVALID, "num_heads must be positive, got %d", sh->num_heads);
     if (sh->ck < 1 || sh->cv < 1) return s2attn_fail(S2ATTN_E_INVALID, "per-head channel counts must be positive");
-    if (sh->nlon_in % sh->nlon_out != 0)
-        return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d)", sh->nlon_in, sh->nlon_out);
+    if (sh->nlon_in % sh->nlon_out != 0 && sh->nlon_out % sh->nlon_in != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d), or the other way round", sh->nlon_in, sh->nlon_out);
     if (sh->dtype != S2ATTN_F32 && sh->dtype != S2ATTN_BF16 && sh->dtype != S2ATTN_F16)
         return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
     if (sh->ck > 128 || sh->cv > 128)
@@ -2444,11 +2453,12 @@ void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const f
     a.sorder = plan->scatter_order;
     a.B = sh->batch;
     a.nh = sh->num_heads;
-    a.kps = sh->nlon_in / sh->nlon_out;
-    a.Hi = sh->nlat_in * a.kps; // virtual input latitudes, see key_point()
-    a.Wi = sh->nlon_out;        // columns of a virtual latitude
-    a.Ho = sh->nlat_out;
-    a.Wo = sh->nlon_out;
+    const bool up = sh->nlon_out % sh->nlon_in == 0 && sh->nlon_out != sh->nlon_in;
+    a.kps = up ? 1 : sh->nlon_in / sh->nlon_out;
+    a.qps = up ? sh->nlon_out / sh->nlon_in : 1;
+    a.Hi = sh->nlat_in * a.kps;  // virtual input latitudes, see key_point()
+    a.Ho = sh->nlat_out * a.qps; // virtual output latitudes, see query_point()
+    a.Wi = a.Wo = up ? sh->nlon_in : sh->nlon_out; // columns of a virtual latitude
     a.dk_ = sh->ck;
     a.dv_ = sh->cv;
     a.pscale = 1;
@@ -2488,7 +2498,8 @@ namespace {
 // that is not handed them (s2attn_backward, s2attn_backward_dq) first recomputes both into the tail of the workspace.
 bool h16_shape(const s2attn_shape *sh)
 {
-    return sh->dtype != S2ATTN_F32 && sh->ck == sh->cv && (sh->ck == 32 || sh->ck == 64 || sh->ck == 128) && sh->nlon_out >= HK;
+    const int w = sh->nlon_out < sh->nlon_in ? sh->nlon_out : sh->nlon_in; // columns of a virtual latitude
+    return sh->dtype != S2ATTN_F32 && sh->ck == sh->cv && (sh->ck == 32 || sh->ck == 64 || sh->ck == 128) && w >= HK;
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
 int64_t round16(int64_t n) { return (n + 15) / 16 * 16; }

@@ -17,12 +17,54 @@
 namespace {
 
 struct HostRun {
-    int32_t ho, hi, ws, len; // after decompose(): hi is the virtual latitude (real latitude * ps + parity class)
+    int32_t ho, hi, ws, len; // virtual output latitude, virtual input latitude, first column, length (see include/s2attn.h)
 };
 
-// Splits the CSR into maximal runs of consecutive longitudes inside one input
-// latitude, then joins a run that ends at nlon_in-1 with a run of the same
-// latitude that starts at 0 into a single circular run.
+// One CSR row -> maximal runs of consecutive columns inside one latitude of the OTHER grid (nlon columns per latitude);
+// a run that ends at nlon - 1 is joined with a run of the same latitude that starts at 0 into one circular run.
+struct RawRun {
+    int32_t lat, ws, len;
+};
+int row_runs(const int64_t *col_idx, int64_t z0, int64_t z1, int nlat, int nlon, std::vector<RawRun> &row)
+{
+    const int64_t ncol = (int64_t)nlat * nlon;
+    row.clear();
+    for (int64_t z = z0; z < z1; z++) {
+        const int64_t col = col_idx[z];
+        if (col < 0 || col >= ncol)
+            return s2attn_fail(S2ATTN_E_INVALID, "col_idx[%lld] = %lld outside [0, %lld)", (long long)z, (long long)col, (long long)ncol);
+        const int32_t lat = (int32_t)(col / nlon), w = (int32_t)(col % nlon);
+        if (!row.empty() && row.back().lat == lat && row.back().ws + row.back().len == w && row.back().len < nlon) {
+            row.back().len++;
+        } else {
+            row.push_back({lat, w, 1});
+        }
+    }
+    size_t i = 0;
+    while (i < row.size()) {
+        size_t j = i;
+        while (j + 1 < row.size() && row[j + 1].lat == row[i].lat) j++;
+        if (j > i && row[i].ws == 0 && row[j].ws + row[j].len == nlon && row[i].len + row[j].len <= nlon) {
+            row[j].len += row[i].len;
+            row[i].len = 0; // dropped
+        }
+        i = j + 1;
+    }
+    return S2ATTN_OK;
+}
+
+// Converts the CSR into runs on virtual latitudes.  Two directions, told apart by the longitude counts:
+//
+// gather (nlon_in = ps * nlon_out): rows are output latitudes ho, columns hi * nlon_in + wi; query column wo sees input
+//   columns ws + t + ps * wo.  Every run is split by column class par = column mod ps: on the sub-lattice
+//   {par, par + ps, ...} of latitude hi (virtual input latitude hi * ps + par, nlon_out columns) the same neighbors are
+//   a run (ws', len') with unit stride in wo.
+// scatter (nlon_out = ps * nlon_in, ps > 1): rows are INPUT latitudes hi, columns ho * nlon_out + wo; input column wi is
+//   seen by output columns ws + t + ps * wi.  Split by output column class: on virtual output latitude ho * ps + par
+//   (nlon_in columns j) input column wi is seen by j = us + u + wi, u in [0, len'), i.e. query column j sees the input
+//   columns (j - us - len' + 1) + t', t' in [0, len'): the run (ws'' = -us - len' + 1 mod nlon_in, len').
+// Either way the result reads: query column j of virtual output latitude `ho` sees columns (ws + t + j) mod W of virtual
+// input latitude `hi`, t in [0, len), W = min(nlon_in, nlon_out).
 int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in, int nlat_out,
               int nlon_out, std::vector<HostRun> *out, int64_t *count)
 {
@@ -30,54 +72,39 @@ int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int n
     if (!row_off) return s2attn_fail(S2ATTN_E_INVALID, "row_off is null");
     if (nlat_in < 1 || nlon_in < 1 || nlat_out < 1 || nlon_out < 1)
         return s2attn_fail(S2ATTN_E_INVALID, "grid extents must be positive");
-    if (nlon_in % nlon_out != 0)
-        return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d)", nlon_in, nlon_out);
-    if (row_off[0] != 0 || row_off[nlat_out] != nnz)
+    const bool up = nlon_out % nlon_in == 0 && nlon_out != nlon_in;
+    if (!up && nlon_in % nlon_out != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d), or the other way round", nlon_in, nlon_out);
+    const int nrow = up ? nlat_in : nlat_out;
+    if (row_off[0] != 0 || row_off[nrow] != nnz)
         return s2attn_fail(S2ATTN_E_INVALID, "row_off must start at 0 and end at nnz (%lld), got %lld..%lld", (long long)nnz,
-                           (long long)row_off[0], (long long)row_off[nlat_out]);
+                           (long long)row_off[0], (long long)row_off[nrow]);
 
-    const int64_t ncol = (int64_t)nlat_in * nlon_in;
-    const int ps = nlon_in / nlon_out;
+    const int ps = up ? nlon_out / nlon_in : nlon_in / nlon_out;
+    const int W = up ? nlon_in : nlon_out;             // columns of a virtual latitude
+    const int nlat_other = up ? nlat_out : nlat_in;    // grid the CSR columns live on
+    const int nlon_other = up ? nlon_out : nlon_in;
     int64_t total = 0;
-    std::vector<HostRun> row;
-    for (int ho = 0; ho < nlat_out; ho++) {
-        const int64_t z0 = row_off[ho], z1 = row_off[ho + 1];
-        if (z1 < z0) return s2attn_fail(S2ATTN_E_INVALID, "row_off decreases at row %d", ho);
-        row.clear();
-        for (int64_t z = z0; z < z1; z++) {
-            const int64_t col = col_idx[z];
-            if (col < 0 || col >= ncol)
-                return s2attn_fail(S2ATTN_E_INVALID, "col_idx[%lld] = %lld outside [0, %lld)", (long long)z, (long long)col,
-                                   (long long)ncol);
-            const int32_t hi = (int32_t)(col / nlon_in), wi = (int32_t)(col % nlon_in);
-            if (!row.empty() && row.back().hi == hi && row.back().ws + row.back().len == wi && row.back().len < nlon_in) {
-                row.back().len++;
-            } else {
-                row.push_back({ho, hi, wi, 1});
-            }
-        }
-        // circular join inside each group of runs that share a latitude
-        size_t i = 0;
-        while (i < row.size()) {
-            size_t j = i;
-            while (j + 1 < row.size() && row[j + 1].hi == row[i].hi) j++;
-            if (j > i && row[i].ws == 0 && row[j].ws + row[j].len == nlon_in && row[i].len + row[j].len <= nlon_in) {
-                row[j].len += row[i].len;
-                row[i].len = 0; // dropped
-            }
-            i = j + 1;
-        }
-        // Longitude ratio ps = nlon_in / nlon_out > 1: query wo sees columns ws + t + ps * wo.  Split every run by
-        // column parity class: on the sub-lattice {par, par + ps, par + 2 ps, ...} of latitude hi (a "virtual latitude"
-        // hi * ps + par with nlon_out columns) the same neighbors are the run (ws', len') with unit stride in wo.
-        for (const HostRun &r : row) {
-            if (r.len == 0) continue;
+    std::vector<RawRun> row;
+    for (int r = 0; r < nrow; r++) {
+        const int64_t z0 = row_off[r], z1 = row_off[r + 1];
+        if (z1 < z0) return s2attn_fail(S2ATTN_E_INVALID, "row_off decreases at row %d", r);
+        const int rc = row_runs(col_idx, z0, z1, nlat_other, nlon_other, row);
+        if (rc != S2ATTN_OK) return rc;
+        for (const RawRun &rr : row) {
+            if (rr.len == 0) continue;
             for (int par = 0; par < ps; par++) {
-                const int t0 = ((par - r.ws) % ps + ps) % ps; // first neighbor of the run in this class
-                if (t0 >= r.len) continue;
-                const int first = (r.ws + t0) % nlon_in;
+                const int t0 = ((par - rr.ws) % ps + ps) % ps; // first entry of the run in this column class
+                if (t0 >= rr.len) continue;
+                const int first = (rr.ws + t0) % nlon_other;
+                const int us = (first - par) / ps, len = (rr.len - t0 + ps - 1) / ps;
                 total++;
-                if (out) out->push_back({ho, r.hi * ps + par, (first - par) / ps, (r.len - t0 + ps - 1) / ps});
+                if (!out) continue;
+                if (up) {
+                    out->push_back({rr.lat * ps + par, r, ((-us - len + 1) % W + W) % W, len});
+                } else {
+                    out->push_back({r, rr.lat * ps + par, us, len});
+                }
             }
         }
     }
@@ -138,35 +165,33 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
     if (rc != S2ATTN_OK) return rc;
     if (n != nruns) return s2attn_fail(S2ATTN_E_INVALID, "nruns = %lld does not match the CSR (%lld runs)", (long long)nruns, (long long)n);
 
-    const int ps = nlon_in / nlon_out;
-    const int nvlat = nlat_in * ps; // virtual input latitudes
+    const bool up = nlon_out % nlon_in == 0 && nlon_out != nlon_in;
+    const int psk = up ? 1 : nlon_in / nlon_out, psq = up ? nlon_out / nlon_in : 1;
+    const int nvin = nlat_in * psk, nvout = nlat_out * psq; // virtual latitudes
 
-    // gather side: runs are already grouped by ho, in CSR order
-    std::vector<RowCost> gcost(nlat_out), scost(nvlat);
-    std::fill(gather_off, gather_off + nlat_out + 1, 0);
+    // both groupings by stable counting sort (entries keep the CSR's order inside a group)
+    std::vector<RowCost> gcost(nvout), scost(nvin);
+    std::fill(gather_off, gather_off + nvout + 1, 0);
+    std::fill(scatter_off, scatter_off + nvin + 1, 0);
     for (int64_t i = 0; i < n; i++) {
-        const HostRun &r = runs[i];
-        gather_runs[4 * i + 0] = r.hi;
-        gather_runs[4 * i + 1] = r.ws;
-        gather_runs[4 * i + 2] = r.len;
-        gather_runs[4 * i + 3] = r.hi / ps; // real latitude: quadrature weight index, row address
-        gather_off[r.ho + 1]++;
-        gcost[r.ho].add(r.len);
+        gather_off[runs[i].ho + 1]++;
+        scatter_off[runs[i].hi + 1]++;
     }
-    for (int ho = 0; ho < nlat_out; ho++) gather_off[ho + 1] += gather_off[ho];
-
-    // scatter side: stable counting sort by hi keeps ho ascending inside a group
-    std::fill(scatter_off, scatter_off + nvlat + 1, 0);
-    for (int64_t i = 0; i < n; i++) scatter_off[runs[i].hi + 1]++;
-    for (int hi = 0; hi < nvlat; hi++) scatter_off[hi + 1] += scatter_off[hi];
-    std::vector<int32_t> cursor(scatter_off, scatter_off + nvlat);
+    for (int r = 0; r < nvout; r++) gather_off[r + 1] += gather_off[r];
+    for (int r = 0; r < nvin; r++) scatter_off[r + 1] += scatter_off[r];
+    std::vector<int32_t> gcur(gather_off, gather_off + nvout), scur(scatter_off, scatter_off + nvin);
     for (int64_t i = 0; i < n; i++) {
         const HostRun &r = runs[i];
-        const int32_t s = cursor[r.hi]++;
-        scatter_runs[4 * s + 0] = r.ho;
-        scatter_runs[4 * s + 1] = r.ws;
-        scatter_runs[4 * s + 2] = r.len;
-        scatter_runs[4 * s + 3] = 0;
+        const int32_t g = gcur[r.ho]++, sidx = scur[r.hi]++;
+        gather_runs[4 * g + 0] = r.hi;
+        gather_runs[4 * g + 1] = r.ws;
+        gather_runs[4 * g + 2] = r.len;
+        gather_runs[4 * g + 3] = r.hi / psk; // real input latitude: quadrature weight index, row address
+        scatter_runs[4 * sidx + 0] = r.ho;
+        scatter_runs[4 * sidx + 1] = r.ws;
+        scatter_runs[4 * sidx + 2] = r.len;
+        scatter_runs[4 * sidx + 3] = r.ho / psq; // real output latitude: row address
+        gcost[r.ho].add(r.len);
         scost[r.hi].add(r.len);
     }
 

@@ -11,8 +11,9 @@ Operator set and signatures follow the reference:
                                                 (attention_optimized.py:230-322)
 Argument order is (k, v, q, ...), outputs of backward are (dk, dv, dq), as there.
 
-Only the gather direction (nlon_in a multiple of nlon_out) is implemented, and only for
-tensors on a ROCm device: there is no CPU implementation behind these operators.
+Both directions are served: nlon_in a multiple of nlon_out (self-attention, down-sampling; psi keyed by output latitude) and
+nlon_out a multiple of nlon_in (up-sampling; psi keyed by input latitude, attention_torch.py:582-592), told apart by the two
+longitude counts as in the reference.  Tensors must live on a ROCm device: there is no CPU implementation behind these operators.
 """
 
 import ctypes
@@ -42,8 +43,6 @@ def _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in
     upsample = nlon_out % nlon_in == 0
     if not (downsample or upsample):
         raise RuntimeError(f"either nlon_in ({nlon_in}) must be an integer multiple of nlon_out ({nlon_out}), or vice versa")
-    if not downsample:
-        raise NotImplementedError(f"upsampling attention (nlon_out {nlon_out} > nlon_in {nlon_in}) is not implemented by the HIP kernels")
     if num_heads < 1:
         raise RuntimeError(f"num_heads must be positive, got {num_heads}")
     for name, t in (("kx", kx), ("vx", vx), ("qy", qy)) + ((("dy", dy),) if dy is not None else ()):

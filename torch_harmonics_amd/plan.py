@@ -48,25 +48,29 @@ def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, 
     Runs the library's host builder on CPU copies of the CSR.  Returns
     ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns, (gather_ndense, scatter_ndense))
     as CPU int32 tensors; gather_runs has shape (nruns, 4) = (virtual input latitude, ws, len, real input latitude),
-    scatter_runs (output latitude, ws, len, 0), grouped by virtual input latitude (nlat_in * nlon_in / nlon_out of them:
-    real latitude * ratio + column class); the first *_ndense entries of each order are the latitudes with long runs.
+    grouped by virtual output latitude; scatter_runs (virtual output latitude, ws, len, real output latitude), grouped by
+    virtual input latitude.  Virtual latitude = real latitude * ratio + column class on the finer of the two grids (see
+    include/s2attn.h); the first *_ndense entries of each order are the latitudes with long runs.
     """
     lib = _lib.load()
     ci = col_idx.detach().to(device="cpu", dtype=torch.int64).contiguous()
     ro = row_off.detach().to(device="cpu", dtype=torch.int64).contiguous()
-    if ro.numel() != nlat_out + 1:
-        raise RuntimeError(f"row_off must have nlat_out + 1 = {nlat_out + 1} entries, got {ro.numel()}")
+    up = nlon_out % max(nlon_in, 1) == 0 and nlon_out != nlon_in  # scatter direction: the CSR is keyed by input latitude
+    nrow = nlat_in if up else nlat_out
+    if ro.numel() != nrow + 1:
+        raise RuntimeError(f"row_off must have {'nlat_in' if up else 'nlat_out'} + 1 = {nrow + 1} entries, got {ro.numel()}")
     nnz = ci.numel()
-    nvlat = nlat_in * max(nlon_in // max(nlon_out, 1), 1)
+    nvin = nlat_in * (1 if up else max(nlon_in // max(nlon_out, 1), 1))
+    nvout = nlat_out * (nlon_out // nlon_in if up else 1)
     nruns = lib.s2attn_plan_count(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out)
     _lib.check(nruns, "s2attn_plan_count")
     arrays = [
-        torch.zeros(nlat_out + 1, dtype=torch.int32),
+        torch.zeros(nvout + 1, dtype=torch.int32),
         torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
-        torch.zeros(nlat_out, dtype=torch.int32),
-        torch.zeros(nvlat + 1, dtype=torch.int32),
+        torch.zeros(nvout, dtype=torch.int32),
+        torch.zeros(nvin + 1, dtype=torch.int32),
         torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
-        torch.zeros(nvlat, dtype=torch.int32),
+        torch.zeros(nvin, dtype=torch.int32),
     ]
     ndense = torch.zeros(2, dtype=torch.int32)
     rc = lib.s2attn_plan_build(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays], ndense.data_ptr())
