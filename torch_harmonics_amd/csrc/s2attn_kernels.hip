@@ -2250,6 +2250,10 @@ int check_shape(const s2attn_shape *sh)
         return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
     if (sh->ck > 128 || sh->cv > 128)
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 128 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
+    // the kernels form offsets inside one latitude of one batch entry in 32 bits
+    const long long wmax = sh->nlon_in > sh->nlon_out ? sh->nlon_in : sh->nlon_out, cmax = sh->ck > sh->cv ? sh->ck : sh->cv;
+    if (wmax * sh->num_heads * cmax * 4 >= (1LL << 31))
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "one latitude row of a tensor (%lld points x %d heads x %lld channels) exceeds 2 GiB", wmax, sh->num_heads, cmax);
     return S2ATTN_OK;
 }
 
