@@ -136,14 +136,23 @@ struct RowCost {
     }
 };
 
-// order: dense latitudes first (most work first), then the others (most work first); returns the dense count
+// order: latitudes with long runs first, then the others; inside each class most work first -- but by cost CLASS
+// (steps of 1/8 in log2), keeping the natural order inside a class.  A plain sort by cost interleaves the two
+// hemispheres (mirror latitudes cost the same); with classes, consecutive entries are neighboring latitudes, whose
+// tiles share most of their K/V rows in L2.  Returns the number of long-run latitudes.
+int cost_class(int64_t c)
+{
+    int cls = 0;
+    while ((c >> cls) > 15) cls++; // c = m * 2^cls, 8 <= m < 16
+    return c <= 0 ? -1 : cls * 8 + (int)((c >> cls) - 8);
+}
 int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order)
 {
     const int n = (int)cost.size();
     std::vector<int32_t> dense, vec;
     for (int i = 0; i < n; i++) (cost[i].dense < cost[i].vector ? dense : vec).push_back(i);
-    std::stable_sort(dense.begin(), dense.end(), [&](int32_t a, int32_t b) { return cost[a].dense > cost[b].dense; });
-    std::stable_sort(vec.begin(), vec.end(), [&](int32_t a, int32_t b) { return cost[a].vector > cost[b].vector; });
+    std::stable_sort(dense.begin(), dense.end(), [&](int32_t a, int32_t b) { return cost_class(cost[a].dense) > cost_class(cost[b].dense); });
+    std::stable_sort(vec.begin(), vec.end(), [&](int32_t a, int32_t b) { return cost_class(cost[a].vector) > cost_class(cost[b].vector); });
     std::copy(dense.begin(), dense.end(), order);
     std::copy(vec.begin(), vec.end(), order + dense.size());
     return (int32_t)dense.size();
