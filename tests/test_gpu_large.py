@@ -125,3 +125,62 @@ def test_cfg2_full_size_forward_and_sampled_backward():
     assert_close("cfg2 dk", dk, dk64, **TOL)
     assert_close("cfg2 dv", dv, dv64, **TOL)
     assert_close("cfg2 dq", dq, dq64, **TOL)
+
+
+def _bf16_close(name, got, want):
+    """2e-2 of the tensor's RMS (bf16 storage, fp32 accumulation)."""
+    rms = want.double().pow(2).mean().sqrt().item()
+    assert_close(name, got, want, rtol=2e-2, atol=2e-2 * rms)
+
+
+def test_cfg5_bf16_sampled_rows_and_properties():
+    """Legendre-Gauss 361x720 self-attention, head_dim 64, bf16 storage, cutoff 8 spacings (197..5562 neighbors per query).
+    Sampled latitudes of 2 of the 16 heads at batch 1 against the float64 spec on the bf16-rounded inputs (0.5 * N(0,1)),
+    then size-independent properties with all 16 heads and the full batch of 4."""
+    from torch_harmonics_amd import ops
+
+    c, (Hi, Wi, Ho, Wo, nh, d), col, roff, w, k, v, q, dy = _setup("cfg5", heads=2, batch=1)
+    k, v, q, dy = [(0.5 * t).to(torch.bfloat16).float() for t in (k, v, q, dy)]
+    kd, vd, qd, gd = [t.to(device=DEV, dtype=torch.bfloat16) for t in (k, v, q, dy)]
+    wd, cd, rd = [t.to(DEV) for t in (w, col, roff)]
+    args = (wd, cd, rd, nh, Wi, Ho, Wo)
+    y, lse = ops.forward_lse(kd, vd, qd, *args)
+    dk, dv, dq = ops.backward_saved(kd, vd, qd, gd, y, lse, *args)
+    dk2, dv2, dq2 = ops.backward(kd, vd, qd, gd, *args)  # recomputes y and lse into the workspace
+    torch.cuda.synchronize()
+    assert torch.equal(dq, dq2) and torch.equal(dk, dk2) and torch.equal(dv, dv2)
+    for r in (0, 2, 180, 360):
+        y64 = oracle.forward_f64(k, v, q, w, col, roff, nh, ho_range=(r, r + 1))
+        _bf16_close(f"cfg5 y row {r}", y[:, r].cpu(), y64[:, r])
+    # equator: output rows 165..195 -> input latitudes 173..187 see all their queries (band half-height 8)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, w, col, roff, nh, ho_range=(165, 196))
+    _bf16_close("cfg5 dq equator", dq[:, 165:196].cpu(), dq64[:, 165:196])
+    _bf16_close("cfg5 dk equator", dk[:, 173:188].cpu(), dk64[:, 173:188])
+    _bf16_close("cfg5 dv equator", dv[:, 173:188].cpu(), dv64[:, 173:188])
+    # north pole: output rows 0..11 -> input latitudes 0..3 complete
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, w, col, roff, nh, ho_range=(0, 12))
+    _bf16_close("cfg5 dq pole", dq[:, 0:12].cpu(), dq64[:, 0:12])
+    _bf16_close("cfg5 dk pole", dk[:, 0:4].cpu(), dk64[:, 0:4])
+    _bf16_close("cfg5 dv pole", dv[:, 0:4].cpu(), dv64[:, 0:4])
+    del kd, vd, qd, gd, y, lse, dk, dv, dq, dk2, dv2, dq2
+
+    # full size: 4 x 361 x 720 x 1024 bf16 (2.1 GB per tensor), generated on the device
+    nh, B = c["nh"], c["B"]
+    gen = torch.Generator(device=DEV).manual_seed(333)
+    kd, vd, gd = [(0.5 * torch.randn(B, Hi, Wi, nh * d, device=DEV, generator=gen)).to(torch.bfloat16) for _ in range(3)]
+    qd = (0.5 * torch.randn(B, Ho, Wo, nh * d, device=DEV, generator=gen) / math.sqrt(d)).to(torch.bfloat16)
+    args = (wd, cd, rd, nh, Wi, Ho, Wo)
+    y, lse = ops.forward_lse(kd, vd, qd, *args)
+    assert torch.isfinite(y).all() and torch.isfinite(lse).all()
+    const = vd[:, :1, :1, :].expand_as(vd).contiguous()
+    yc, lsec = ops.forward_lse(kd, const, qd, *args)
+    _bf16_close("constant v", yc, const[:, :1, :1, :].expand_as(yc).float())
+    dk, dv, dq = ops.backward_saved(kd, const, qd, gd, yc, lsec, *args)
+    # with constant v the exact dq and dk vanish; what is left is the bf16 rounding of y inside I = <dy, y>
+    assert float(dq.float().abs().max()) < 0.05 and float(dk.float().abs().max()) < 0.05
+    gsum = gd.double().sum(dim=(1, 2))
+    assert_close("sum dv == sum dy", dv.double().sum(dim=(1, 2)), gsum, rtol=2e-2, atol=2e-2 * gsum.abs().mean().item() + 2.0)
+    y_roll = ops.forward(torch.roll(kd, 5, 2), torch.roll(vd, 5, 2), torch.roll(qd, 5, 2), *args)
+    _bf16_close("roll equivariance", y_roll, torch.roll(y, 5, 2).float())  # other tile alignment: equal up to bf16 rounding
+    dk, dv, dq = ops.backward_saved(kd, vd, qd, gd, y, lse, *args)
+    assert torch.isfinite(dk).all() and torch.isfinite(dv).all() and torch.isfinite(dq).all()
