@@ -1,21 +1,29 @@
 // Spherical neighborhood attention on gfx950: forward, dq and dk/dv kernels, layout
 // permutes, and the C entry points declared in include/s2attn.h.
 //
-// Work decomposition (all three attention kernels)
-//   One wavefront (= one workgroup of 64 threads) owns 64 consecutive longitudes of
-//   one latitude for one (batch, head); lane i owns longitude w0 + i and keeps its
-//   per-point vectors (q and the y accumulator, or k, v and the dk, dv accumulators)
-//   in registers.  The neighborhood of a whole latitude is a short list of runs
-//   (lat, ws, len): for the 64 lanes together a run touches one contiguous, circular
-//   band of the other grid's longitudes, which the wavefront copies into LDS with
-//   coalesced loads and then slides over: lane i reads row pscale*i + t.  No
-//   cross-lane reduction and no atomics anywhere; dk/dv are produced by a transposed
-//   gather (runs regrouped by input latitude) instead of a scatter.
-//   Workgroups are issued longest latitude first; the linear block index has
-//   (batch, head) fastest so the 8 XCDs each see one head's band of K/V.
+// Work decomposition (all attention kernels)
+//   One wavefront (= one workgroup of 64 threads) owns a tile of consecutive longitudes of
+//   one latitude for one (batch, head) and keeps its per-point vectors (q and the y
+//   accumulator, or k, v and the dk, dv accumulators) in registers.  The neighborhood of
+//   a whole latitude is a short list of runs (lat, ws, len): for the tile a run touches
+//   one contiguous, circular band of the other grid's longitudes, which the wavefront
+//   copies into LDS with coalesced 16-byte loads and then slides over (point i reads band
+//   rows i + t).  No atomics anywhere: dk/dv are produced by a transposed gather (runs
+//   regrouped by input latitude) instead of a scatter.  Longitude ratios between the two
+//   grids are removed by the plan (virtual latitudes, see key_point() / query_point()).
 //
-// Numerics: storage dtype in/out (fp32, bf16, fp16), everything else fp32.  Scores
-// are kept in the log2 domain (q is multiplied by log2(e) once) so the softmax uses
+// Kernel families, chosen on the host from the shape (launch_t):
+//   *_h16_kernel<T, D>     16-bit storage, head dim 32/64/128: 16-longitude tiles, 16-bit matrix cores   (s2attn_h16.hpp)
+//   *_mfma_kernel<T>       head dim 32: 32-longitude tiles, fp32 matrix cores for runs >= LMIN, vector path below
+//   *_fast_kernel<T, P>    head dim P in {4, 8, 16, 32}: 64-longitude tiles, lane = grid point, register-prefetched band
+//   *_wide_kernel<T, LPQ>  head dims 33..128: 2 or 4 lanes per grid point
+//   *_kernel<T, P, VEC>    everything else (ck != cv, odd head dims, unaligned pointers, narrow grids)
+//   Workgroups are issued longest latitude first; the linear block index has (batch, head)
+//   fastest (16-bit family: one (batch, head) per XCD at a time), so the 8 XCDs each see one
+//   head's band of K/V.
+//
+// Numerics: storage dtype in/out (fp32, bf16, fp16), softmax and accumulation fp32.  Scores
+// are kept in the log2 domain (q, or the score, is multiplied by log2(e)) so the softmax uses
 // the hardware exp2.
 
 #include <hip/hip_runtime.h>
@@ -224,7 +232,7 @@ struct Args {
     const float *quad_w;
     const int *goff, *gorder, *soff, *sorder;
     const Run *gruns, *sruns;
-    int B, nh, Hi, Wi, Ho, Wo, dk_, dv_, pscale;
+    int B, nh, Hi, Wi, Ho, Wo, dk_, dv_;
     int kps; // nlon_in / nlon_out when the input grid is the finer one, else 1; see key_point()
     int qps; // nlon_out / nlon_in when the output grid is the finer one, else 1; see query_point()
     int tile_rows; // LDS rows per staged band
@@ -234,7 +242,7 @@ struct Args {
 // Key-side addressing.  With nlon_in = kps * nlon_out, query column wo sees input columns ws + t + kps * wo: on the
 // sub-lattice {par, par + kps, ...} of a real input latitude that is a unit-stride problem.  The plan therefore lists
 // neighborhoods over Hi = nlat_in * kps "virtual" latitudes (real latitude * kps + par) of Wi = nlon_out columns each,
-// every kernel works as if nlon_in == nlon_out (pscale == 1), and only the address of a virtual grid point differs:
+// every kernel works as if nlon_in == nlon_out, and only the address of a virtual grid point differs:
 // key_point() is the real point index of column 0 of a virtual latitude, consecutive columns lie kps points apart.
 // Gather runs carry the real latitude in Run::pad (also the index of the quadrature weight).
 __device__ inline long key_point(const Args &a, int b, int vlat, int rlat)
@@ -272,7 +280,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void fwd
     const int b = bh / a.nh, h = bh % a.nh;
     const int wo0 = wt * TQ;
     const int nvalid = min(TQ, a.Wo - wo0);
-    const int ps = a.pscale;
+    constexpr int ps = 1; // the plan removed the longitude stride (virtual latitudes, see key_point())
     const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
 
     const T *kx = static_cast<const T *>(a.k);
@@ -375,7 +383,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dq_
     const int b = bh / a.nh, h = bh % a.nh;
     const int wo0 = wt * TQ;
     const int nvalid = min(TQ, a.Wo - wo0);
-    const int ps = a.pscale;
+    constexpr int ps = 1; // the plan removed the longitude stride (virtual latitudes, see key_point())
     const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
 
     const T *kx = static_cast<const T *>(a.k);
@@ -498,7 +506,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
     const int b = bh / a.nh, h = bh % a.nh;
     const int wi0 = ct * TQ;
     const int nvalid = min(TQ, a.Wi - wi0);
-    const int ps = a.pscale;
+    constexpr int ps = 1; // the plan removed the longitude stride (virtual latitudes, see key_point())
     const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
 
     const T *kx = static_cast<const T *>(a.k);
@@ -635,7 +643,7 @@ template <int LPQ> __device__ inline float slice_sum(float x)
     const int b = bh / a.nh, h = bh % a.nh;                                   \
     const int w0 = wt * TQW;                                                  \
     const int nvalid = min(TQW, (W_TILED)-w0);                                \
-    const int ps = a.pscale;                                                  \
+    constexpr int ps = 1; /* longitude stride removed by the plan */           \
     const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
 
 template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void fwd_wide_kernel(const Args a)
@@ -916,7 +924,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
 }
 
 // ---------------------------------------------------------------------------------
-// Software-pipelined band staging (fast path: vector loads, pscale == 1, nlon >= tile rows).
+// Software-pipelined band staging (fast path: vector loads, at least one band of columns per virtual latitude).
 // A band of up to TQ-1+TL grid points is fetched into registers with one 16-byte (8-byte for
 // 16-bit storage) load per lane and iteration, NIT iterations, while the previous band is being
 // consumed from LDS; it is written to LDS afterwards.  Lane constants: row r0 = lane / (P/4) of
@@ -1226,7 +1234,7 @@ template <typename T, int P> __global__ __launch_bounds__(TQ) void dq_fast_kerne
     unstage_rows<T, P, true>(dq, Ks, ldk * a.qps, a.dk_, w0, nvalid, lane);
 }
 
-// backward dk/dv, fast path (pscale == 1: the queries that see input longitude wi through run (ho, ws, len)
+// backward dk/dv, fast path (the queries that see input longitude wi through run (ho, ws, len)
 // are wo = wi - ws - t, t in [0, len))
 template <typename T, int P> __global__ __launch_bounds__(TQ) void dkdv_fast_kernel(const Args a)
 {
@@ -1434,7 +1442,7 @@ __device__ inline int run_stride(int len) { return run_is_dense(len) ? MT : VC; 
     const int w0 = wt * MT;                                                   \
     const int nvalid = min(MT, (W_TILED)-w0);
 
-// forward, head dim 32, pscale 1.  Lane (j, half) keeps channels 8g + 4 half + e (g, e < 4) of query j: that is the
+// forward, head dim 32.  Lane (j, half) keeps channels 8g + 4 half + e (g, e < 4) of query j: that is the
 // accumulator layout of the matrix-core product, and the vector path for short runs uses the same one (each half
 // computes half of a dot product, one cross-half exchange completes it).
 template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(const Args a)
@@ -2275,7 +2283,7 @@ template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a
     size_t lds = 0;
     // fast path: 16-byte loads, equal longitude counts, and a grid at least as wide as one staged band
     constexpr int FAST_ROWS = Band<T, P>::NIT * Band<T, P>::RPI;
-    const bool fast = VEC && a.pscale == 1 && a.Wi >= FAST_ROWS && a.dk_ == P && a.dv_ == P;
+    const bool fast = VEC && a.Wi >= FAST_ROWS && a.dk_ == P && a.dv_ == P;
     if (fast) a.tile_rows = FAST_ROWS;
     if (which == FWD) {
         kern = fast ? fwd_fast_kernel<T, P> : fwd_kernel<T, P, VEC>;
@@ -2291,7 +2299,7 @@ template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
     }
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "longitude ratio %d needs %zu bytes of LDS per workgroup", a.pscale, lds);
+    if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the staged band needs %zu bytes of LDS per workgroup", lds);
     if (lds > 48 * 1024) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -2314,19 +2322,19 @@ template <typename T, int LPQ, bool VEC> int launch_wide(Which which, const Args
     size_t lds = 0;
     if (which == DKDV) {
         kern = dkdv_wide_kernel<T, LPQ, VEC>;
-        a.tile_rows = (TQW - 1) / a.pscale + 1 + TL;
+        a.tile_rows = TQW + TL;
         if (a.tile_rows < TQW) a.tile_rows = TQW;
         nblocks = (long)row_count * ((a.Wi + TQW - 1) / TQW) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
     } else {
         kern = which == FWD ? fwd_wide_kernel<T, LPQ, VEC> : dq_wide_kernel<T, LPQ, VEC>;
-        a.tile_rows = a.pscale * (TQW - 1) + TL;
+        a.tile_rows = TQW - 1 + TL;
         if (a.tile_rows < TQW) a.tile_rows = TQW;
         nblocks = (long)row_count * ((a.Wo + TQW - 1) / TQW) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
     }
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "longitude ratio %d needs %zu bytes of LDS per workgroup", a.pscale, lds);
+    if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the staged band needs %zu bytes of LDS per workgroup", lds);
     if (lds > 48 * 1024) {
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
@@ -2348,7 +2356,7 @@ template <typename T, bool VEC> int launch_p(Which which, const Args &a, int row
     return launch_one<T, 32, VEC>(which, a, row_first, row_count, stream);
 }
 
-// dense kernels: head dims 32, pscale 1, vector-aligned rows, nlon >= 32
+// dense kernels: head dims 32, vector-aligned rows, at least 64 columns per virtual latitude
 template <typename T> int launch_dense(Which which, const Args &a0, int row_count, hipStream_t stream)
 {
     if (row_count <= 0) return S2ATTN_OK;
@@ -2405,7 +2413,7 @@ template <typename T, int D> int launch_h16(Which which, const Args &a0, hipStre
 template <typename T> bool h16_ok(Which which, const Args &a)
 {
     if (std::is_same<T, float>::value) return false;
-    if (a.pscale != 1 || a.dk_ != a.dv_ || (a.dk_ != 32 && a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
+    if (a.dk_ != a.dv_ || (a.dk_ != 32 && a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
     if (which == DQ && !(a.ysaved && a.lse)) return false;
     const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
     for (const void *p : ptrs)
@@ -2416,7 +2424,7 @@ template <typename T> bool h16_ok(Which which, const Args &a)
 bool dense_ok(Which which, const Args &a, bool vec)
 {
     (void)which;
-    return vec && a.pscale == 1 && a.dk_ == 32 && a.dv_ == 32 && a.Wi >= 64;
+    return vec && a.dk_ == 32 && a.dv_ == 32 && a.Wi >= 64;
 }
 
 template <typename T> int launch_t(Which which, const Args &a, bool vec, int ndense, hipStream_t stream)
@@ -2465,7 +2473,6 @@ void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const f
     a.Wi = a.Wo = up ? sh->nlon_in : sh->nlon_out; // columns of a virtual latitude
     a.dk_ = sh->ck;
     a.dv_ = sh->cv;
-    a.pscale = 1;
 }
 
 } // namespace
@@ -2491,7 +2498,7 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     fill_args(a, plan, shape, quad_weights);
     a.k = k, a.v = v, a.q = q, a.y = y;
     a.lse = lse;
-    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    a.tile_rows = TQ - 1 + TL;
     const size_t al = 4 * (size_t)esize(shape->dtype);
     const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(y, al);
     return launch(FWD, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
@@ -2549,7 +2556,7 @@ extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, c
     if (!dq) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     a.dq = dq;
     vec = vec && aligned(dq, 4 * (size_t)esize(shape->dtype));
-    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    a.tile_rows = TQ - 1 + TL;
     if (h16_shape(shape) && aligned(workspace, 16)) {
         const int64_t n = stat_points(shape);
         char *ws = static_cast<char *>(workspace);
@@ -2578,7 +2585,7 @@ extern "C" int s2attn_backward_dq_saved(const void *k, const void *v, const void
     a.lse = const_cast<float *>(lse);
     const size_t al = 4 * (size_t)esize(shape->dtype);
     vec = vec && aligned(dq, al) && aligned(y, al);
-    a.tile_rows = a.pscale * (TQ - 1) + TL;
+    a.tile_rows = TQ - 1 + TL;
     return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
 }
 
@@ -2594,7 +2601,7 @@ extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q,
     a.dk = dk, a.dv = dv;
     const size_t al = 4 * (size_t)esize(shape->dtype);
     vec = vec && aligned(dk, al) && aligned(dv, al);
-    a.tile_rows = (TQ - 1) / a.pscale + 1 + TL;
+    a.tile_rows = TQ + TL;
     if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile also stages the lane-owned k/v and dk/dv rows
     return launch(DKDV, a, shape->dtype, vec, plan->scatter_ndense, static_cast<hipStream_t>(stream));
 }
