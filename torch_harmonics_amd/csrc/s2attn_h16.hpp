@@ -114,13 +114,11 @@ template <int PITCH> __device__ inline uint4 h16_read_row(const char *tile, int 
 
 __device__ inline float h16_quarter_max(float x)
 {
-    x = fmaxf(x, __shfl_xor(x, 16));
-    return fmaxf(x, __shfl_xor(x, 32));
+    return xor32_max(xor16_max(x));
 }
 __device__ inline float h16_quarter_sum(float x)
 {
-    x += __shfl_xor(x, 16);
-    return x + __shfl_xor(x, 32);
+    return xor32_sum(xor16_sum(x));
 }
 
 // Workgroup index -> ((batch, head), index inside it).  The hardware deals consecutive workgroups round-robin to the 8

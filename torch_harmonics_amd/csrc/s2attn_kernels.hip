@@ -160,6 +160,30 @@ __device__ inline float4 widen4(uint2 r, const f16_t *)
 __device__ inline float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 __device__ inline float fast_log2(float x) { return __builtin_amdgcn_logf(x); }
 
+// Exchange with the lane 32 (16) positions away without going through LDS.  v_permlane32_swap swaps the upper half of its
+// first operand with the lower half of its second: called with (x, x) it returns (x of the lower half, x of the upper
+// half), each replicated in both halves.  v_permlane16_swap does the same with the odd and even rows of 16 lanes.
+__device__ inline float xor32_sum(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ inline float xor32_max(float x)
+{
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ inline float xor16_sum(float x)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ inline float xor16_max(float x)
+{
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(x), __float_as_uint(x), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+
 // ---- LDS staging -------------------------------------------------------------------
 // Copies `nrows` grid points (longitudes c0, c0+1, ... wrapping at W) of one latitude and
 // one head into LDS as fp32 rows of P floats (zero padded past d), row stride P+4 floats so
@@ -1532,7 +1556,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
             float mx = sc[0];
 #pragma unroll
             for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            mx = xor32_max(mx);
             const float mn = fmaxf(m, mx);
             if (__any(mn > m)) {
                 const float corr = fast_exp2(m - mn);
@@ -1557,7 +1581,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
                     rs += p;
                 }
             }
-            rs += __shfl_xor(rs, 32);
+            rs = xor32_sum(rs);
             S += rs;
             // Y^T += V^T P^T
 #pragma unroll
@@ -1583,7 +1607,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
                         part = fmaf(qb[4 * g + 2], x.z, part);
                         part = fmaf(qb[4 * g + 3], x.w, part);
                     }
-                    s[t] = part + __shfl_xor(part, 32);
+                    s[t] = xor32_sum(part);
                     cm = fmaxf(cm, s[t]);
                 }
             }
@@ -1735,7 +1759,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
             float mx = sc[0];
 #pragma unroll
             for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
-            mx = fmaxf(mx, __shfl_xor(mx, 32));
+            mx = xor32_max(mx);
             const float mn = fmaxf(m, mx);
             if (__any(mn > m)) {
                 const float corr = fast_exp2(m - mn);
@@ -1759,8 +1783,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
                 rs += p;
                 rg += pg;
             }
-            rs += __shfl_xor(rs, 32);
-            rg += __shfl_xor(rg, 32);
+            rs = xor32_sum(rs);
+            rg = xor32_sum(rg);
             S += rs;
             Ag += rg;
 #pragma unroll
@@ -1792,8 +1816,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
                         pg_ = fmaf(gb[4 * g + 2], z.z, pg_);
                         pg_ = fmaf(gb[4 * g + 3], z.w, pg_);
                     }
-                    s[t] = ps_ + __shfl_xor(ps_, 32);
-                    gd[t] = pg_ + __shfl_xor(pg_, 32);
+                    s[t] = xor32_sum(ps_);
+                    gd[t] = xor32_sum(pg_);
                     cm = fmaxf(cm, s[t]);
                 }
             }
@@ -1890,7 +1914,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
             I = fmaf(z.z, yv.z, I);
             I = fmaf(z.w, yv.w, I);
         }
-        I += __shfl_xor(I, 32);
+        I = xor32_sum(I);
     }
     const float lse = a.lse[sidx];
     if (mine && half == 0) a.stats[sidx] = make_float2(lse, I);
@@ -1990,8 +2014,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
                         pg_ = fmaf(gb[4 * g + 2], z.z, pg_);
                         pg_ = fmaf(gb[4 * g + 3], z.w, pg_);
                     }
-                    const float sv = ps_ + __shfl_xor(ps_, 32);
-                    const float gv = pg_ + __shfl_xor(pg_, 32);
+                    const float sv = xor32_sum(ps_);
+                    const float gv = xor32_sum(pg_);
                     const float coef = fast_exp2(sv - lse) * w * (gv - I);
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
@@ -2176,8 +2200,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
                         pg_ = fmaf(vb[4 * g + 2], xg[g].z, pg_);
                         pg_ = fmaf(vb[4 * g + 3], xg[g].w, pg_);
                     }
-                    const float s = ps_ + __shfl_xor(ps_, 32);
-                    const float gd = pg_ + __shfl_xor(pg_, 32);
+                    const float s = xor32_sum(ps_);
+                    const float gd = xor32_sum(pg_);
                     const float p = fast_exp2(s - Ls[j + i]) * w;
                     const float coef = p * (gd - Is[j + i]);
 #pragma unroll
