@@ -260,3 +260,23 @@ def test_upsampling_direction(case, dtype):
             else:
                 rms = w.pow(2).mean().sqrt().item()
                 assert_close(f"{tname} ({name})", got, w, rtol=2e-2, atol=2e-2 * rms)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_results_are_bitwise_reproducible(dtype):
+    """No atomics anywhere (dk and dv are a transposed gather, not the reference's atomic scatter, attention_cuda_bwd.cu:242-307):
+    two runs on the same inputs give identical bits, in every kernel family."""
+    from torch_harmonics_amd import ops
+
+    dev = torch.device("cuda", 0)
+    for nh, d, ins, outs in ((2, 32, (24, 96), (24, 96)), (1, 16, (12, 160), (12, 160)), (1, 64, (16, 48), (16, 48)), (2, 32, (24, 96), (12, 48)), (1, 5, (10, 20), (10, 20))):
+        col_idx, row_off, quad = _psi(ins, outs, "equiangular", "equiangular", 0.5)
+        k, v, q, dy = [t.to(device=dev, dtype=dtype) for t in randn_inputs(2, ins[0], ins[1], outs[0], outs[1], nh, d, d)]
+        geo = (quad.to(dev), col_idx.to(dev), row_off.to(dev), nh, ins[1], outs[0], outs[1])
+        runs = []
+        for _ in range(2):
+            y, lse = ops.forward_lse(k, v, q, *geo)
+            runs.append((y, lse) + tuple(ops.backward_saved(k, v, q, dy, y, lse, *geo)) + tuple(ops.backward(k, v, q, dy, *geo)))
+        torch.cuda.synchronize()
+        for a, b in zip(*runs):
+            assert torch.equal(a, b)
