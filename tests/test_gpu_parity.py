@@ -75,6 +75,9 @@ SMALL_CASES = [
     (1, 1, 128, 128, (10, 20), (10, 20), "equiangular", "equiangular", 0.7),
     (1, 2, 96, 72, (12, 48), (12, 16), "equiangular", "equiangular", 0.5),
     (1, 1, 33, 65, (8, 16), (8, 16), "equiangular", "equiangular", 0.8),
+    (1, 1, 256, 256, (8, 16), (8, 16), "equiangular", "equiangular", 0.8),
+    (1, 1, 160, 300, (9, 12), (5, 4), "equiangular", "equiangular", 0.9),
+    (1, 1, 512, 96, (6, 12), (6, 12), "legendre-gauss", "legendre-gauss", 0.9),
     # head dim 32 on grids wide enough for the matrix-core kernels (nlon >= 64), incl. full-circle rows and long runs
     (1, 2, 32, 32, (24, 96), (24, 96), "equiangular", "equiangular", 0.5),
     (2, 1, 32, 32, (16, 128), (16, 128), "legendre-gauss", "legendre-gauss", 0.9),

@@ -16,7 +16,7 @@
 //   *_h16_kernel<T, D>     16-bit storage, head dim 32/64/128: 16-longitude tiles, 16-bit matrix cores   (s2attn_h16.hpp)
 //   *_mfma_kernel<T>       head dim 32: 32-longitude tiles, fp32 matrix cores for runs >= LMIN, vector path below
 //   *_fast_kernel<T, P>    head dim P in {4, 8, 16, 32}: 64-longitude tiles, lane = grid point, register-prefetched band
-//   *_wide_kernel<T, LPQ>  head dims 33..128: 2 or 4 lanes per grid point
+//   *_wide_kernel<T, LPQ>  head dims 33..512: 2 to 16 lanes per grid point
 //   *_kernel<T, P, VEC>    everything else (ck != cv, odd head dims, unaligned pointers, narrow grids)
 //   Workgroups are issued longest latitude first; the linear block index has (batch, head)
 //   fastest (16-bit family: one (batch, head) per XCD at a time), so the 8 XCDs each see one
@@ -639,7 +639,7 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
 
 
 // ---------------------------------------------------------------------------------
-// Wide heads (32 < head dim <= 128): same single-wavefront tiling as the generic kernels, but LPQ = 2 or 4
+// Wide heads (32 < head dim <= 512): same single-wavefront tiling as the generic kernels, but LPQ = 2, 4, 8 or 16
 // adjacent lanes share one grid point and each keeps a 32-channel slice of its vectors, so the register
 // footprint stays that of a 32-channel head; a dot product is completed by LPQ-lane butterfly adds.
 // A wavefront therefore covers 64 / LPQ longitudes.
@@ -2280,8 +2280,8 @@ int check_shape(const s2attn_shape *sh)
         return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d), or the other way round", sh->nlon_in, sh->nlon_out);
     if (sh->dtype != S2ATTN_F32 && sh->dtype != S2ATTN_BF16 && sh->dtype != S2ATTN_F16)
         return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
-    if (sh->ck > 128 || sh->cv > 128)
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 128 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
+    if (sh->ck > 512 || sh->cv > 512)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 512 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
     // the kernels form offsets inside one latitude of one batch entry in 32 bits
     const long long wmax = sh->nlon_in > sh->nlon_out ? sh->nlon_in : sh->nlon_out, cmax = sh->ck > sh->cv ? sh->ck : sh->cv;
     if (wmax * sh->num_heads * cmax * 4 >= (1LL << 31))
@@ -2372,6 +2372,8 @@ template <typename T, int LPQ, bool VEC> int launch_wide(Which which, const Args
 template <typename T, bool VEC> int launch_p(Which which, const Args &a, int row_first, int row_count, hipStream_t stream)
 {
     const int d = a.dk_ > a.dv_ ? a.dk_ : a.dv_;
+    if (d > 256) return launch_wide<T, 16, VEC>(which, a, row_first, row_count, stream);
+    if (d > 128) return launch_wide<T, 8, VEC>(which, a, row_first, row_count, stream);
     if (d > 64) return launch_wide<T, 4, VEC>(which, a, row_first, row_count, stream);
     if (d > 32) return launch_wide<T, 2, VEC>(which, a, row_first, row_count, stream);
     if (d <= 4) return launch_one<T, 4, VEC>(which, a, row_first, row_count, stream);
