@@ -47,7 +47,7 @@ def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     bad = _lib.ShapeStruct(1, 2, 4, 9, 4, 6, 8, 8, _lib.S2ATTN_F32)  # 9 % 6 != 0
     assert lib.s2attn_backward_workspace_bytes(ctypes.byref(bad)) == -1
     assert b"multiple" in lib.s2attn_last_error()
-    wide = _lib.ShapeStruct(1, 1, 4, 8, 4, 8, 160, 160, _lib.S2ATTN_F32)
+    wide = _lib.ShapeStruct(1, 1, 4, 8, 4, 8, 520, 520, _lib.S2ATTN_F32)
     assert lib.s2attn_backward_workspace_bytes(ctypes.byref(wide)) == -2  # unsupported head width
     dt = _lib.ShapeStruct(1, 1, 4, 8, 4, 8, 8, 8, 7)
     assert lib.s2attn_backward_workspace_bytes(ctypes.byref(dt)) == -1
