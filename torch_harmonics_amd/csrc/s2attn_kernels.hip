@@ -644,6 +644,8 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
 // footprint stays that of a 32-channel head; a dot product is completed by LPQ-lane butterfly adds.
 // A wavefront therefore covers 64 / LPQ longitudes.
 // ---------------------------------------------------------------------------------
+constexpr int TSW = 32; // neighbors staged per band refill in the gather kernels of this family
+
 template <int LPQ> __device__ inline float slice_sum(float x)
 {
 #pragma unroll
@@ -697,16 +699,19 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
         const float w = a.quad_w[run.pad];
         const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
         const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
-        for (int t0 = 0; t0 < run.len; t0 += TL) {
-            const int L = min(TL, run.len - t0);
-            const int c0 = (run.ws + t0 + ps * w0) % a.Wi;
-            const int nrows = ps * (nvalid - 1) + L;
+        // one refill of the band serves up to TSW neighbors, consumed TL at a time: long runs pay the staging latency 4x less often
+        for (int T0 = 0; T0 < run.len; T0 += TSW) {
+            const int LT = min(TSW, run.len - T0);
+            const int c0 = (run.ws + T0 + w0) % a.Wi;
+            const int nrows = nvalid - 1 + LT;
             __syncthreads();
             stage_rows<T, PT, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
             stage_rows<T, PT, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
             __syncthreads();
-            const float *krow = Ks + (ps * qi) * LS + sl * 32;
-            const float *vrow = Vs + (ps * qi) * LS + sl * 32;
+          for (int t0 = 0; t0 < LT; t0 += TL) {
+            const int L = min(TL, LT - t0);
+            const float *krow = Ks + (qi + t0) * LS + sl * 32;
+            const float *vrow = Vs + (qi + t0) * LS + sl * 32;
             float s[TL];
             float cm = NEG_BIG;
 #pragma unroll
@@ -739,6 +744,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
                     }
                 }
             }
+          }
         }
     }
     if (a.lse && qi < nvalid && sl == 0) a.lse[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = m + fast_log2(S);
@@ -782,16 +788,19 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
         const float w = a.quad_w[run.pad];
         const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
         const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
-        for (int t0 = 0; t0 < run.len; t0 += TL) {
-            const int L = min(TL, run.len - t0);
-            const int c0 = (run.ws + t0 + ps * w0) % a.Wi;
-            const int nrows = ps * (nvalid - 1) + L;
+        // one refill of the band serves up to TSW neighbors, consumed TL at a time: long runs pay the staging latency 4x less often
+        for (int T0 = 0; T0 < run.len; T0 += TSW) {
+            const int LT = min(TSW, run.len - T0);
+            const int c0 = (run.ws + T0 + w0) % a.Wi;
+            const int nrows = nvalid - 1 + LT;
             __syncthreads();
             stage_rows<T, PT, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
             stage_rows<T, PT, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
             __syncthreads();
-            const float *krow = Ks + (ps * qi) * LS + sl * 32;
-            const float *vrow = Vs + (ps * qi) * LS + sl * 32;
+          for (int t0 = 0; t0 < LT; t0 += TL) {
+            const int L = min(TL, LT - t0);
+            const float *krow = Ks + (qi + t0) * LS + sl * 32;
+            const float *vrow = Vs + (qi + t0) * LS + sl * 32;
             float s[TL], g[TL];
             float cm = NEG_BIG;
 #pragma unroll
@@ -836,6 +845,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
                     }
                 }
             }
+          }
         }
     }
     const float inv = 1.0f / S;
@@ -2352,7 +2362,7 @@ template <typename T, int LPQ, bool VEC> int launch_wide(Which which, const Args
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
     } else {
         kern = which == FWD ? fwd_wide_kernel<T, LPQ, VEC> : dq_wide_kernel<T, LPQ, VEC>;
-        a.tile_rows = TQW - 1 + TL;
+        a.tile_rows = TQW - 1 + TSW;
         if (a.tile_rows < TQW) a.tile_rows = TQW;
         nblocks = (long)row_count * ((a.Wo + TQW - 1) / TQW) * BH;
         lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
