@@ -264,3 +264,25 @@ def test_forward_and_backward_replay_from_a_hip_graph():
         torch.cuda.synchronize()
         for name, g_, w_ in zip(("y", "dk", "dv", "dq"), got, want):
             assert torch.equal(g_, w_), f"replay {it}: {name} differs from the eager result"
+
+
+def test_module_traces_under_torch_compile():
+    """The operators carry fake (meta) kernels and autograd formulas registered through torch.library, so the module traces as one
+    graph (fullgraph) through AOT autograd; forward and gradients must equal the eager ones (tests/test_attention_layout.py:170-200
+    does the same for the layout ops)."""
+    m = _small_module()
+    xq = torch.randn(2, 8, 6, 12, device=DEV)
+    xkv = torch.randn(2, 8, 12, 24, device=DEV)
+    gout = torch.randn(2, 8, 6, 12, device=DEV)
+
+    def run(fn):
+        a, b = xq.clone().requires_grad_(True), xkv.clone().requires_grad_(True)
+        m.zero_grad(set_to_none=True)
+        out = fn(a, b, b)
+        out.backward(gout)
+        return [out.detach(), a.grad, b.grad] + [p.grad.clone() for p in m.parameters()]
+
+    eager = run(m)
+    compiled = run(torch.compile(m, backend="aot_eager", fullgraph=True))
+    for i, (e, c) in enumerate(zip(eager, compiled)):
+        assert_close(f"tensor {i}", c, e, rtol=1e-6, atol=1e-6)

@@ -4,26 +4,24 @@ import torch
 
 
 def _check_ndim(tensor: torch.Tensor, ndim: int, name: str) -> None:
-    """RuntimeError unless tensor has `ndim` dimensions; the message closes over plain ints only so dynamo can trace it."""
-    actual = tensor.dim()
-    torch._check(actual == ndim, lambda: f"Expected {ndim}-dimensional {name} tensor, got {actual} dimensions")
+    """RuntimeError unless tensor has `ndim` dimensions (a plain branch: dynamo folds it to a constant while tracing)."""
+    if tensor.dim() != ndim:
+        raise RuntimeError(f"Expected {ndim}-dimensional {name} tensor, got {tensor.dim()} dimensions")
 
 
 def _check_extent(tensor: torch.Tensor, dim: int, expected: int, name: str) -> None:
-    """RuntimeError unless tensor.shape[dim] == expected (the actual extent may be symbolic and stays out of the message)."""
+    """RuntimeError unless tensor.shape[dim] == expected (under tracing the comparison becomes a shape guard)."""
     expected = int(expected)
-    torch._check(tensor.shape[dim] == expected, lambda: f"Expected {name} shape[{dim}] == {expected}")
-
-
-def _dtype_mismatch_message() -> str:
-    return "all attention inputs must share a single dtype"
+    if tensor.shape[dim] != expected:
+        raise RuntimeError(f"Expected {name} shape[{dim}] == {expected}, got {tensor.shape[dim]}")
 
 
 def _check_dtypes_match(tensors) -> None:
     """RuntimeError unless all tensors share one dtype: the kernels read every activation as q's element type."""
     first = tensors[0].dtype
     for t in tensors[1:]:
-        torch._check(t.dtype == first, _dtype_mismatch_message)
+        if t.dtype != first:
+            raise RuntimeError("all attention inputs must share a single dtype")
 
 
 def _setup_context_attention_backward(ctx, inputs, output):
