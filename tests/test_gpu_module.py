@@ -173,7 +173,8 @@ def test_wrong_shapes_raise_runtime_error():
         m(torch.randn(2, 8, 6, 12, device=DEV), torch.randn(2, 8, 11, 24, device=DEV), torch.randn(2, 8, 12, 24, device=DEV))
 
 
-LAYOUT_SHAPES = [(2, 3, 5, 7), (1, 1, 4, 4), (2, 4, 1, 1), (1, 256, 33, 70), (3, 65, 64, 65), (2, 8, 1, 9), (1, 1, 1, 1), (0, 4, 3, 2)]
+# the last two: more than 65535 tiles along H*W, and more than 65535 batch entries (a launch's y and z extents stop there)
+LAYOUT_SHAPES = [(2, 3, 5, 7), (1, 1, 4, 4), (2, 4, 1, 1), (1, 256, 33, 70), (3, 65, 64, 65), (2, 8, 1, 9), (1, 1, 1, 1), (0, 4, 3, 2), (1, 2, 2100, 2048), (70000, 2, 3, 1)]
 
 
 @pytest.mark.parametrize("shape", LAYOUT_SHAPES)

@@ -2253,11 +2253,14 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
 // ---------------------------------------------------------------------------------
 // layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
 // ---------------------------------------------------------------------------------
-template <typename E> __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ src, E *__restrict__ dst, long R, long S)
+// The grid is one-dimensional (a grid's y and z extents stop at 65535, and H*W/64 passes that on fine grids): workgroup
+// id = (batch * gy + row tile) * gx + column tile.
+template <typename E> __global__ __launch_bounds__(256) void transpose_kernel(const E *__restrict__ src, E *__restrict__ dst, long R, long S, unsigned gx, unsigned gy)
 {
     __shared__ E tile[64][65];
-    const long bofs = (long)blockIdx.z * R * S;
-    const long s0 = (long)blockIdx.x * 64, r0 = (long)blockIdx.y * 64;
+    const unsigned bx = blockIdx.x % gx, rest = blockIdx.x / gx;
+    const long bofs = (long)(rest / gy) * R * S;
+    const long s0 = (long)bx * 64, r0 = (long)(rest % gy) * 64;
     const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
     for (int i = ty; i < 64; i += 4) {
         const long r = r0 + i, s = s0 + tx;
@@ -2667,9 +2670,10 @@ template <typename E> int launch_transpose(const void *src, void *dst, long nb, 
 {
     if (nb == 0 || R == 0 || S == 0) return S2ATTN_OK;
     const long gx = (S + 63) / 64, gy = (R + 63) / 64;
-    if (gx > 0x7fffffffL || gy > 65535 || nb > 65535) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "permute grid (%ld, %ld, %ld) exceeds launch limits", gx, gy, nb);
-    hipLaunchKernelGGL(s2::transpose_kernel<E>, dim3((unsigned)gx, (unsigned)gy, (unsigned)nb), dim3(256), 0, stream, static_cast<const E *>(src),
-                       static_cast<E *>(dst), R, S);
+    if (gx > 0x7fffffffL || gy > 0x7fffffffL || nb > 0x7fffffffL || gx * gy > 0x7fffffffL || gx * gy * nb > 0x7fffffffL)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "permute needs %ld x %ld x %ld workgroups, more than one grid holds", gx, gy, nb);
+    hipLaunchKernelGGL(s2::transpose_kernel<E>, dim3((unsigned)(gx * gy * nb)), dim3(256), 0, stream, static_cast<const E *>(src),
+                       static_cast<E *>(dst), R, S, (unsigned)gx, (unsigned)gy);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
