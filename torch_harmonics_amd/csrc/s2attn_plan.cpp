@@ -108,6 +108,7 @@ int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int n
             }
         }
     }
+    if (total > 0x7fffffffLL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the neighborhood has %lld runs, more than the plan's 32-bit offsets index", (long long)total);
     *count = total;
     return S2ATTN_OK;
 }

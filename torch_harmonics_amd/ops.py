@@ -32,9 +32,11 @@ def _stream_ptr(device: torch.device) -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
-def _require_gpu(t: torch.Tensor, name: str) -> None:
+def _require_gpu(t: torch.Tensor, name: str, device: torch.device = None) -> None:
     if t.device.type != "cuda":
         raise RuntimeError(f"{name} is on {t.device}; the s2attn operators only run on a ROCm GPU (no CPU implementation is shipped)")
+    if device is not None and t.device != device:
+        raise RuntimeError(f"{name} is on {t.device} but the other operands are on {device}")
 
 
 def _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
@@ -85,7 +87,7 @@ def _shape_struct(kx, vx, qy, num_heads) -> _lib.ShapeStruct:
 def _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, with_lse):
     _validate(kx, vx, qy, None, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
     for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
-        _require_gpu(t, name)
+        _require_gpu(t, name, kx.device)
     if qy.dtype == torch.float64:  # stored as fp64, computed in fp32 like the reference (attention_cuda_utils.cuh:185-190)
         y, lse = _forward_impl(kx.float(), vx.float(), qy.float(), quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, with_lse)
         return y.double(), lse
@@ -159,11 +161,11 @@ def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, 
 def _backward_impl(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
     _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
     for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("dy", dy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
-        _require_gpu(t, name)
+        _require_gpu(t, name, kx.device)
     saved = y is not None
     if saved:
-        _require_gpu(y, "y")
-        _require_gpu(lse, "lse")
+        _require_gpu(y, "y", kx.device)
+        _require_gpu(lse, "lse", kx.device)
         if y.shape != dy.shape or y.dtype != dy.dtype or not y.is_contiguous():
             raise RuntimeError("y must be the contiguous forward output (shape and dtype of dy)")
         if lse.shape != (kx.shape[0], num_heads, nlat_out, nlon_out) or lse.dtype != torch.float32 or not lse.is_contiguous():
