@@ -190,13 +190,13 @@ __device__ inline float xor16_max(float x)
 // that 128-bit reads by consecutive lanes fall in distinct banks.
 //   src : first element of (batch, latitude, longitude 0, head)
 //   ld  : elements between two longitudes (num_heads * d)
-template <typename T, int P, bool VEC>
+template <typename T, int P, bool VEC, int NT = TQ>
 __device__ inline void stage_rows(float *dst, const T *src, long ld, int d, int c0, int W, int nrows, int lane)
 {
     constexpr int LS = P + 4;
     if (VEC) {
         constexpr int V4 = P / 4;
-        for (int idx = lane; idx < nrows * V4; idx += TQ) {
+        for (int idx = lane; idx < nrows * V4; idx += NT) {
             const int r = idx / V4, c = 4 * (idx % V4);
             int col = c0 + r;
             while (col >= W) col -= W;
@@ -205,7 +205,7 @@ __device__ inline void stage_rows(float *dst, const T *src, long ld, int d, int 
             *reinterpret_cast<float4 *>(dst + r * LS + c) = val;
         }
     } else {
-        for (int idx = lane; idx < nrows * P; idx += TQ) {
+        for (int idx = lane; idx < nrows * P; idx += NT) {
             const int r = idx / P, c = idx % P;
             int col = c0 + r;
             while (col >= W) col -= W;
@@ -215,18 +215,18 @@ __device__ inline void stage_rows(float *dst, const T *src, long ld, int d, int 
 }
 
 // Writes `nrows` LDS rows back to consecutive longitudes c0.. (no wrap) of one latitude/head.
-template <typename T, int P, bool VEC>
+template <typename T, int P, bool VEC, int NT = TQ>
 __device__ inline void unstage_rows(T *dst, const float *src, long ld, int d, int c0, int nrows, int lane)
 {
     constexpr int LS = P + 4;
     if (VEC) {
         constexpr int V4 = P / 4;
-        for (int idx = lane; idx < nrows * V4; idx += TQ) {
+        for (int idx = lane; idx < nrows * V4; idx += NT) {
             const int r = idx / V4, c = 4 * (idx % V4);
             if (c < d) store4(dst + (long)(c0 + r) * ld + c, *reinterpret_cast<const float4 *>(src + r * LS + c));
         }
     } else {
-        for (int idx = lane; idx < nrows * P; idx += TQ) {
+        for (int idx = lane; idx < nrows * P; idx += NT) {
             const int r = idx / P, c = idx % P;
             if (c < d) from_f32(dst[(long)(c0 + r) * ld + c], src[r * LS + c]);
         }
@@ -639,12 +639,23 @@ template <typename T, int P, bool VEC> __global__ __launch_bounds__(TQ) void dkd
 
 
 // ---------------------------------------------------------------------------------
-// Wide heads (32 < head dim <= 512): same single-wavefront tiling as the generic kernels, but LPQ = 2, 4, 8 or 16
-// adjacent lanes share one grid point and each keeps a 32-channel slice of its vectors, so the register
-// footprint stays that of a 32-channel head; a dot product is completed by LPQ-lane butterfly adds.
-// A wavefront therefore covers 64 / LPQ longitudes.
+// Wide heads (32 < head dim <= 512): LPQ = 2, 4, 8 or 16 adjacent lanes share one grid point and each keeps a
+// 32-channel slice of its vectors, so the register footprint stays that of a 32-channel head; a dot product is
+// completed by LPQ-lane butterfly adds.  A wavefront therefore covers 64 / LPQ longitudes.
+// A workgroup is WNW wavefronts over the SAME longitudes: they stage every band together and split its neighbors
+// (wavefront w takes the w-th quarter of each staged chunk), each with its own running softmax state; the states
+// are merged through LDS at the end, in wavefront order, so results do not depend on timing.  The band in LDS --
+// 34 KB at 64 channels -- then serves four wavefronts instead of one, and a pole row, thousands of neighbors per
+// grid point, is worked on by four wavefronts at once.
 // ---------------------------------------------------------------------------------
-constexpr int TSW = 32; // neighbors staged per band refill in the gather kernels of this family
+constexpr int WNW = 4;        // wavefronts per workgroup
+constexpr int WNT = TQ * WNW; // threads per workgroup
+// Neighbors staged per band refill: each wavefront takes WSUB groups of TL of them.  Two groups where the band stays
+// small (64-channel heads: 95 rows, 52 KB for both tiles), one for wider heads.
+template <int LPQ> struct WideCfg {
+    static constexpr int WSUB = LPQ <= 2 ? 2 : 1;
+    static constexpr int TSW = WNW * WSUB * TL;
+};
 
 template <int LPQ> __device__ inline float slice_sum(float x)
 {
@@ -657,7 +668,9 @@ template <int LPQ> __device__ inline float slice_sum(float x)
     constexpr int TQW = TQ / LPQ;                                             \
     constexpr int PT = 32 * LPQ;                                              \
     constexpr int LS = PT + 4;                                                \
-    const int lane = threadIdx.x;                                             \
+    constexpr int TSW = WideCfg<LPQ>::TSW;                                    \
+    const int tid = threadIdx.x;                                              \
+    const int lane = tid % TQ, wv = tid / TQ;                                 \
     const int qi = lane / LPQ, sl = lane % LPQ;                               \
     const int BH = a.B * a.nh;                                                \
     const int ntile = ((W_TILED) + TQW - 1) / TQW;                            \
@@ -669,10 +682,9 @@ template <int LPQ> __device__ inline float slice_sum(float x)
     const int b = bh / a.nh, h = bh % a.nh;                                   \
     const int w0 = wt * TQW;                                                  \
     const int nvalid = min(TQW, (W_TILED)-w0);                                \
-    constexpr int ps = 1; /* longitude stride removed by the plan */           \
     const long ldk = (long)a.nh * a.dk_, ldv = (long)a.nh * a.dv_;
 
-template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void fwd_wide_kernel(const Args a)
+template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(WNT) void fwd_wide_kernel(const Args a)
 {
     extern __shared__ float4 smem4[];
     float *Ks = reinterpret_cast<float *>(smem4);
@@ -684,7 +696,7 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
     const T *qy = static_cast<const T *>(a.q);
     T *y = static_cast<T *>(a.y);
 
-    stage_rows<T, PT, VEC>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, PT, VEC, WNT>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, tid);
     __syncthreads();
     float qr[32], acc[32];
 #pragma unroll
@@ -699,17 +711,19 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
         const float w = a.quad_w[run.pad];
         const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
         const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
-        // one refill of the band serves up to TSW neighbors, consumed TL at a time: long runs pay the staging latency 4x less often
         for (int T0 = 0; T0 < run.len; T0 += TSW) {
             const int LT = min(TSW, run.len - T0);
             const int c0 = (run.ws + T0 + w0) % a.Wi;
             const int nrows = nvalid - 1 + LT;
             __syncthreads();
-            stage_rows<T, PT, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
-            stage_rows<T, PT, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC, WNT>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, tid);
+            stage_rows<T, PT, VEC, WNT>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, tid);
             __syncthreads();
-          for (int t0 = 0; t0 < LT; t0 += TL) {
-            const int L = min(TL, LT - t0);
+            // this wavefront's share of the chunk: neighbors wv * share .. tend - 1, TL at a time
+            const int share = (LT + WNW - 1) / WNW;
+            const int tend = min(LT, (wv + 1) * share);
+          for (int t0 = wv * share; t0 < tend; t0 += TL) {
+            const int L = min(TL, tend - t0);
             const float *krow = Ks + (qi + t0) * LS + sl * 32;
             const float *vrow = Vs + (qi + t0) * LS + sl * 32;
             float s[TL];
@@ -747,17 +761,39 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void f
           }
         }
     }
-    if (a.lse && qi < nvalid && sl == 0) a.lse[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = m + fast_log2(S);
-    const float inv = 1.0f / S;
-    __syncthreads();
+    // wavefront 0 takes in the other wavefronts' states one after the other (34 floats per lane, stored [value][lane])
+    for (int ow = 1; ow < WNW; ow++) {
+        __syncthreads();
+        if (wv == ow) {
 #pragma unroll
-    for (int c = 0; c < 32; c += 4)
-        *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
+            for (int c = 0; c < 32; c++) Ks[c * TQ + lane] = acc[c];
+            Ks[32 * TQ + lane] = m;
+            Ks[33 * TQ + lane] = S;
+        }
+        __syncthreads();
+        if (wv == 0) {
+            const float mo = Ks[32 * TQ + lane];
+            const float mn = fmaxf(m, mo);
+            const float c0 = fast_exp2(m - mn), c1 = fast_exp2(mo - mn);
+            m = mn;
+            S = S * c0 + Ks[33 * TQ + lane] * c1;
+#pragma unroll
+            for (int c = 0; c < 32; c++) acc[c] = acc[c] * c0 + Ks[c * TQ + lane] * c1;
+        }
+    }
     __syncthreads();
-    unstage_rows<T, PT, VEC>(y + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, Ks, ldv * a.qps, a.dv_, w0, nvalid, lane);
+    if (wv == 0) {
+        if (a.lse && qi < nvalid && sl == 0) a.lse[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = m + fast_log2(S);
+        const float inv = 1.0f / S;
+#pragma unroll
+        for (int c = 0; c < 32; c += 4)
+            *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c) = make_float4(acc[c] * inv, acc[c + 1] * inv, acc[c + 2] * inv, acc[c + 3] * inv);
+    }
+    __syncthreads();
+    unstage_rows<T, PT, VEC, WNT>(y + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, Ks, ldv * a.qps, a.dv_, w0, nvalid, tid);
 }
 
-template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void dq_wide_kernel(const Args a)
+template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(WNT) void dq_wide_kernel(const Args a)
 {
     extern __shared__ float4 smem4[];
     float *Ks = reinterpret_cast<float *>(smem4);
@@ -770,8 +806,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
     const T *gy = static_cast<const T *>(a.dy);
     T *dq = static_cast<T *>(a.dq);
 
-    stage_rows<T, PT, VEC>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, lane);
-    stage_rows<T, PT, VEC>(Vs, gy + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, ldv * a.qps, a.dv_, w0, a.Wo, nvalid, lane);
+    stage_rows<T, PT, VEC, WNT>(Ks, qy + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, ldk * a.qps, a.dk_, w0, a.Wo, nvalid, tid);
+    stage_rows<T, PT, VEC, WNT>(Vs, gy + query_point(a, b, ho, ho / a.qps) * ldv + (long)h * a.dv_, ldv * a.qps, a.dv_, w0, a.Wo, nvalid, tid);
     __syncthreads();
     float qr[32], gr[32], Ak[32], Akg[32];
 #pragma unroll
@@ -788,17 +824,18 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
         const float w = a.quad_w[run.pad];
         const T *kl = kx + key_point(a, b, run.lat, run.pad) * ldk + (long)h * a.dk_;
         const T *vl = vx + key_point(a, b, run.lat, run.pad) * ldv + (long)h * a.dv_;
-        // one refill of the band serves up to TSW neighbors, consumed TL at a time: long runs pay the staging latency 4x less often
         for (int T0 = 0; T0 < run.len; T0 += TSW) {
             const int LT = min(TSW, run.len - T0);
             const int c0 = (run.ws + T0 + w0) % a.Wi;
             const int nrows = nvalid - 1 + LT;
             __syncthreads();
-            stage_rows<T, PT, VEC>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, lane);
-            stage_rows<T, PT, VEC>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, lane);
+            stage_rows<T, PT, VEC, WNT>(Ks, kl, ldk * a.kps, a.dk_, c0, a.Wi, nrows, tid);
+            stage_rows<T, PT, VEC, WNT>(Vs, vl, ldv * a.kps, a.dv_, c0, a.Wi, nrows, tid);
             __syncthreads();
-          for (int t0 = 0; t0 < LT; t0 += TL) {
-            const int L = min(TL, LT - t0);
+            const int share = (LT + WNW - 1) / WNW;
+            const int tend = min(LT, (wv + 1) * share);
+          for (int t0 = wv * share; t0 < tend; t0 += TL) {
+            const int L = min(TL, tend - t0);
             const float *krow = Ks + (qi + t0) * LS + sl * 32;
             const float *vrow = Vs + (qi + t0) * LS + sl * 32;
             float s[TL], g[TL];
@@ -848,20 +885,51 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
           }
         }
     }
-    const float inv = 1.0f / S;
-    const float I = Ag * inv;
-    if (qi < nvalid && sl == 0) a.stats[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = make_float2(m + fast_log2(S), I);
-    __syncthreads();
+    // wavefront 0 takes in the other wavefronts' states one after the other (67 floats per lane, stored [value][lane];
+    // the K and V tiles are contiguous and together hold them)
+    for (int ow = 1; ow < WNW; ow++) {
+        __syncthreads();
+        if (wv == ow) {
 #pragma unroll
-    for (int c = 0; c < 32; c += 4)
-        *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c)
-            = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
-                          (Akg[c + 3] - I * Ak[c + 3]) * inv);
+            for (int c = 0; c < 32; c++) {
+                Ks[c * TQ + lane] = Ak[c];
+                Ks[(32 + c) * TQ + lane] = Akg[c];
+            }
+            Ks[64 * TQ + lane] = m;
+            Ks[65 * TQ + lane] = S;
+            Ks[66 * TQ + lane] = Ag;
+        }
+        __syncthreads();
+        if (wv == 0) {
+            const float mo = Ks[64 * TQ + lane];
+            const float mn = fmaxf(m, mo);
+            const float c0 = fast_exp2(m - mn), c1 = fast_exp2(mo - mn);
+            m = mn;
+            S = S * c0 + Ks[65 * TQ + lane] * c1;
+            Ag = Ag * c0 + Ks[66 * TQ + lane] * c1;
+#pragma unroll
+            for (int c = 0; c < 32; c++) {
+                Ak[c] = Ak[c] * c0 + Ks[c * TQ + lane] * c1;
+                Akg[c] = Akg[c] * c0 + Ks[(32 + c) * TQ + lane] * c1;
+            }
+        }
+    }
     __syncthreads();
-    unstage_rows<T, PT, VEC>(dq + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, Ks, ldk * a.qps, a.dk_, w0, nvalid, lane);
+    if (wv == 0) {
+        const float inv = 1.0f / S;
+        const float I = Ag * inv;
+        if (qi < nvalid && sl == 0) a.stats[((long)bh * a.Ho + ho) * a.Wo + w0 + qi] = make_float2(m + fast_log2(S), I);
+#pragma unroll
+        for (int c = 0; c < 32; c += 4)
+            *reinterpret_cast<float4 *>(Ks + qi * LS + sl * 32 + c)
+                = make_float4((Akg[c] - I * Ak[c]) * inv, (Akg[c + 1] - I * Ak[c + 1]) * inv, (Akg[c + 2] - I * Ak[c + 2]) * inv,
+                              (Akg[c + 3] - I * Ak[c + 3]) * inv);
+    }
+    __syncthreads();
+    unstage_rows<T, PT, VEC, WNT>(dq + query_point(a, b, ho, ho / a.qps) * ldk + (long)h * a.dk_, Ks, ldk * a.qps, a.dk_, w0, nvalid, tid);
 }
 
-template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void dkdv_wide_kernel(const Args a)
+template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(WNT) void dkdv_wide_kernel(const Args a)
 {
     extern __shared__ float4 smem4[];
     float *Qs = reinterpret_cast<float *>(smem4);
@@ -876,8 +944,8 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
     T *dk = static_cast<T *>(a.dk);
     T *dv = static_cast<T *>(a.dv);
 
-    stage_rows<T, PT, VEC>(Qs, kx + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, ldk * a.kps, a.dk_, w0, a.Wi, nvalid, lane);
-    stage_rows<T, PT, VEC>(Gs, vx + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, ldv * a.kps, a.dv_, w0, a.Wi, nvalid, lane);
+    stage_rows<T, PT, VEC, WNT>(Qs, kx + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, ldk * a.kps, a.dk_, w0, a.Wi, nvalid, tid);
+    stage_rows<T, PT, VEC, WNT>(Gs, vx + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, ldv * a.kps, a.dv_, w0, a.Wi, nvalid, tid);
     __syncthreads();
     float kr[32], vr[32], dkr[32], dvr[32];
 #pragma unroll
@@ -889,45 +957,45 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
     }
     const float w = a.quad_w[hi / a.kps];
 
+    // Input column w0 + qi is neighbor t of output column (w0 + qi - ws - t) mod W.  A chunk covers t = u0 .. u0 + UL - 1:
+    // the output columns c0 .. c0 + nvalid - 2 + UL are staged, and neighbor t = u0 + jj of lane qi sits in staged row
+    // qi + UL - 1 - jj.
     for (int ri = a.soff[hi]; ri < a.soff[hi + 1]; ri++) {
         const Run run = a.sruns[ri];
         const int ho = run.lat;
         int d0 = w0 - run.ws;
         if (d0 < 0) d0 += a.Wi;
-        const int al = (d0 + qi) / ps - d0 / ps;
-        const int r0 = (d0 + qi) % ps;
-        const int a0 = d0 / ps;
-        const int span = (d0 + nvalid - 1) / ps - a0;
-        const int U = (run.len + ps - 1) / ps;
         const T *ql = qy + query_point(a, b, ho, run.pad) * ldk + (long)h * a.dk_;
         const T *gl = gy + query_point(a, b, ho, run.pad) * ldv + (long)h * a.dv_;
         const float2 *sl2 = a.stats + ((long)bh * a.Ho + ho) * a.Wo;
-        for (int u0 = 0; u0 < U; u0 += TL) {
-            const int UL = min(TL, U - u0);
-            int c0 = (a0 - u0 - UL + 1) % a.Wo;
+        for (int u0 = 0; u0 < run.len; u0 += TSW) {
+            const int UL = min(TSW, run.len - u0);
+            int c0 = (d0 - u0 - UL + 1) % a.Wo;
             if (c0 < 0) c0 += a.Wo;
-            const int nrows = span + UL;
+            const int nrows = nvalid - 1 + UL;
             __syncthreads();
-            stage_rows<T, PT, VEC>(Qs, ql, ldk * a.qps, a.dk_, c0, a.Wo, nrows, lane);
-            stage_rows<T, PT, VEC>(Gs, gl, ldv * a.qps, a.dv_, c0, a.Wo, nrows, lane);
-            for (int r = lane; r < nrows; r += TQ) {
+            stage_rows<T, PT, VEC, WNT>(Qs, ql, ldk * a.qps, a.dk_, c0, a.Wo, nrows, tid);
+            stage_rows<T, PT, VEC, WNT>(Gs, gl, ldv * a.qps, a.dv_, c0, a.Wo, nrows, tid);
+            for (int r = tid; r < nrows; r += WNT) {
                 int col = c0 + r;
                 while (col >= a.Wo) col -= a.Wo;
                 Ss[r] = sl2[col];
             }
             __syncthreads();
+            const int share = (UL + WNW - 1) / WNW;
+            const int jend = min(UL, (wv + 1) * share);
+          for (int j0 = wv * share; j0 < jend; j0 += TL) {
+            const int L = min(TL, jend - j0);
 #pragma unroll
             for (int jj = 0; jj < TL; jj++) {
-                if (jj < UL) {
-                    const int row = al + (UL - 1 - jj);
-                    const int t = r0 + ps * (u0 + jj);
+                if (jj < L) {
+                    const int row = qi + (UL - 1 - j0 - jj);
                     const float *qrow = Qs + row * LS + sl * 32;
                     const float *grow = Gs + row * LS + sl * 32;
                     const float s = slice_sum<LPQ>(dot_row<32>(kr, qrow));
                     const float g = slice_sum<LPQ>(dot_row<32>(vr, grow));
                     const float2 st = Ss[row];
-                    float p = fast_exp2(s - st.x) * w;
-                    if (t >= run.len) p = 0.f;
+                    const float p = fast_exp2(s - st.x) * w;
                     const float coef = p * (g - st.y);
 #pragma unroll
                     for (int c = 0; c < 32; c += 4) {
@@ -944,17 +1012,39 @@ template <typename T, int LPQ, bool VEC> __global__ __launch_bounds__(TQ) void d
                     }
                 }
             }
+          }
+        }
+    }
+    // wavefront 0 adds up the other wavefronts' sums one after the other (64 floats per lane, stored [value][lane])
+    for (int ow = 1; ow < WNW; ow++) {
+        __syncthreads();
+        if (wv == ow) {
+#pragma unroll
+            for (int c = 0; c < 32; c++) {
+                Qs[c * TQ + lane] = dkr[c];
+                Qs[(32 + c) * TQ + lane] = dvr[c];
+            }
+        }
+        __syncthreads();
+        if (wv == 0) {
+#pragma unroll
+            for (int c = 0; c < 32; c++) {
+                dkr[c] += Qs[c * TQ + lane];
+                dvr[c] += Qs[(32 + c) * TQ + lane];
+            }
         }
     }
     __syncthreads();
+    if (wv == 0) {
 #pragma unroll
-    for (int c = 0; c < 32; c += 4) {
-        *reinterpret_cast<float4 *>(Qs + qi * LS + sl * 32 + c) = make_float4(dkr[c], dkr[c + 1], dkr[c + 2], dkr[c + 3]);
-        *reinterpret_cast<float4 *>(Gs + qi * LS + sl * 32 + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
+        for (int c = 0; c < 32; c += 4) {
+            *reinterpret_cast<float4 *>(Qs + qi * LS + sl * 32 + c) = make_float4(dkr[c], dkr[c + 1], dkr[c + 2], dkr[c + 3]);
+            *reinterpret_cast<float4 *>(Gs + qi * LS + sl * 32 + c) = make_float4(dvr[c], dvr[c + 1], dvr[c + 2], dvr[c + 3]);
+        }
     }
     __syncthreads();
-    unstage_rows<T, PT, VEC>(dk + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, Qs, ldk * a.kps, a.dk_, w0, nvalid, lane);
-    unstage_rows<T, PT, VEC>(dv + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, Gs, ldv * a.kps, a.dv_, w0, nvalid, lane);
+    unstage_rows<T, PT, VEC, WNT>(dk + key_point(a, b, hi, hi / a.kps) * ldk + (long)h * a.dk_, Qs, ldk * a.kps, a.dk_, w0, nvalid, tid);
+    unstage_rows<T, PT, VEC, WNT>(dv + key_point(a, b, hi, hi / a.kps) * ldv + (long)h * a.dv_, Gs, ldv * a.kps, a.dv_, w0, nvalid, tid);
 }
 
 // ---------------------------------------------------------------------------------
@@ -2352,23 +2442,22 @@ template <typename T, int LPQ, bool VEC> int launch_wide(Which which, const Args
     if (row_count <= 0) return S2ATTN_OK;
     Args a = a0;
     a.row_first = row_first;
-    constexpr int TQW = TQ / LPQ, LS = 32 * LPQ + 4;
+    constexpr int TQW = TQ / LPQ, LS = 32 * LPQ + 4, TSW = WideCfg<LPQ>::TSW;
     const int BH = a.B * a.nh;
     void (*kern)(const Args) = nullptr;
     long nblocks = 0;
-    size_t lds = 0;
+    a.tile_rows = TQW - 1 + TSW; // a band: the tile's grid points slid over one chunk of neighbors
+    size_t lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
+    // the tiles double as the exchange buffer when the wavefronts merge their states: 34 / 67 / 64 floats per lane
+    static_assert((size_t)2 * (TQW - 1 + TSW) * LS >= (size_t)67 * TQ, "band tiles too small for the state merge");
+    static_assert((size_t)(TQW - 1 + TSW) * LS >= (size_t)34 * TQ, "band tile too small for the forward state merge");
     if (which == DKDV) {
         kern = dkdv_wide_kernel<T, LPQ, VEC>;
-        a.tile_rows = TQW + TL;
-        if (a.tile_rows < TQW) a.tile_rows = TQW;
         nblocks = (long)row_count * ((a.Wi + TQW - 1) / TQW) * BH;
-        lds = (size_t)2 * a.tile_rows * LS * sizeof(float) + (size_t)a.tile_rows * sizeof(float2);
+        lds += (size_t)a.tile_rows * sizeof(float2);
     } else {
         kern = which == FWD ? fwd_wide_kernel<T, LPQ, VEC> : dq_wide_kernel<T, LPQ, VEC>;
-        a.tile_rows = TQW - 1 + TSW;
-        if (a.tile_rows < TQW) a.tile_rows = TQW;
         nblocks = (long)row_count * ((a.Wo + TQW - 1) / TQW) * BH;
-        lds = (size_t)2 * a.tile_rows * LS * sizeof(float);
     }
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
     if (lds > 160 * 1024) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the staged band needs %zu bytes of LDS per workgroup", lds);
@@ -2376,7 +2465,7 @@ template <typename T, int LPQ, bool VEC> int launch_wide(Which which, const Args
         const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(TQ), lds, stream, a);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(WNT), lds, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
