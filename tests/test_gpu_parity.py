@@ -78,6 +78,13 @@ SMALL_CASES = [
     (1, 1, 256, 256, (8, 16), (8, 16), "equiangular", "equiangular", 0.8),
     (1, 1, 160, 300, (9, 12), (5, 4), "equiangular", "equiangular", 0.9),
     (1, 1, 512, 96, (6, 12), (6, 12), "legendre-gauss", "legendre-gauss", 0.9),
+    # head dim 64 in fp32 on grids of at least 32 longitudes: the fp32 16-longitude matrix-core kernels; stride-2 input grid,
+    # runs longer than one 32-position step, a ragged last tile
+    (1, 2, 64, 64, (12, 96), (6, 48), "equiangular", "equiangular", 0.5),
+    (1, 1, 64, 64, (10, 80), (10, 80), "equiangular", "equiangular", 1.2),
+    (2, 2, 64, 64, (9, 44), (9, 44), "legendre-gauss", "legendre-gauss", 0.6),
+    (1, 2, 128, 128, (8, 40), (8, 40), "equiangular", "equiangular", 0.9),
+    (1, 1, 128, 128, (10, 72), (5, 36), "equiangular", "legendre-gauss", 0.7),
     # head dim 32 on grids wide enough for the matrix-core kernels (nlon >= 64), incl. full-circle rows and long runs
     (1, 2, 32, 32, (24, 96), (24, 96), "equiangular", "equiangular", 0.5),
     (2, 1, 32, 32, (16, 128), (16, 128), "legendre-gauss", "legendre-gauss", 0.9),
@@ -170,6 +177,7 @@ SAVED_CASES = [
     (1, 2, 64, 64, (16, 48), (16, 48), "legendre-gauss", "legendre-gauss", 0.4),
     (2, 1, 64, 64, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
     (1, 1, 64, 64, (8, 40), (8, 40), "equiangular", "equiangular", 7.0),
+    (1, 1, 128, 128, (8, 36), (8, 36), "equiangular", "equiangular", 0.8),
     (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
     (1, 1, 128, 128, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
 ]

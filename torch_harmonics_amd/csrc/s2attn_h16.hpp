@@ -61,16 +61,14 @@ template <> struct H16<f16_t> {
     }
 };
 
-// 32 consecutive longitudes (c0.., wrapping once at W) of one latitude/head as a [32][D] 16-bit LDS tile; rows are
-// PITCH bytes apart.  fetch() keeps the tile in registers (one 16-byte load per lane per iteration) so that the
-// loads of the next step fly while the current one is consumed; commit() writes it to LDS.
-template <int D> struct HTile {
-    static constexpr int CPR = D / 8;        // 16-byte pieces per row
+// 32 consecutive longitudes (c0.., wrapping once at W) of one latitude/head as a [32][row] LDS tile: rows of CPR_
+// 16-byte pieces, PITCH_ bytes apart.  fetch() keeps the tile in registers (one 16-byte load per lane per iteration) so
+// that the loads of the next step fly while the current one is consumed; commit() writes it to LDS.
+template <int CPR_, int PITCH_> struct BandTile {
+    static constexpr int CPR = CPR_;         // 16-byte pieces per row
     static constexpr int RPI = 64 / CPR;     // rows per iteration
     static constexpr int NIT = HK / RPI;     // iterations
-    static constexpr int PITCH = 2 * D + 32; // bytes.  Measured with SQ_LDS_BANK_CONFLICT: row pitches of 32 or 96 bytes modulo 128
-                                             // are free of bank conflicts for all three access patterns (16-byte row pieces by lanes
-                                             // (c, qd), transposing 8-byte reads, 16-byte writes); 2 D + 16 costs both reads 2x
+    static constexpr int PITCH = PITCH_;     // bytes
     u4v raw[NIT];
     // Byte offsets of this lane's pieces inside one latitude of one (batch, head) slice; the same for every tensor of
     // a step (k and v, or q and dy).  lane_off = (lane / CPR) * ldb + 16 * (lane % CPR).
@@ -94,6 +92,11 @@ template <int D> struct HTile {
         for (int it = 0; it < NIT; it++) *reinterpret_cast<u4v *>(dst + (r0 + it * RPI) * PITCH + cb) = raw[it];
     }
 };
+
+// 16-bit tile of D channels.  Row pitch measured with SQ_LDS_BANK_CONFLICT: pitches of 32 or 96 bytes modulo 128 are free
+// of bank conflicts for all three access patterns (16-byte row pieces by lanes (c, qd), transposing 8-byte reads, 16-byte
+// writes); 2 D + 16 costs both reads 2x.
+template <int D> struct HTile : BandTile<D / 8, 2 * D + 32> {};
 
 // A operand "channels 16 cb + c, positions (kb, v) of this lane's quarter" from a [position][channel] tile
 template <int PITCH> __device__ inline uint4 h16_read_transposed(const char *tile, int cb, int c, int qd)

@@ -2339,6 +2339,7 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
 }
 
 #include "s2attn_h16.hpp"
+#include "s2attn_m32.hpp"
 
 // ---------------------------------------------------------------------------------
 // layout permutes: batched 2-D transpose [R, S] -> [S, R] through a 64x65 LDS tile
@@ -2549,6 +2550,41 @@ template <typename T> bool h16_ok(Which which, const Args &a)
     return true;
 }
 
+// fp32 matrix-core kernels for 64- and 128-channel heads: same launch geometry and the same conditions as the 16-bit family.
+template <int D> int launch_m32(Which which, const Args &a0, hipStream_t stream)
+{
+    Args a = a0;
+    a.row_first = 0;
+    void (*kern)(const Args) = nullptr;
+    long nblocks = 0;
+    if (which == FWD) {
+        kern = fwd_m32_kernel<D>;
+        nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+    } else if (which == DQ) {
+        kern = dq_m32_kernel<D>;
+        nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+    } else {
+        kern = dkdv_m32_kernel<D>;
+        nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
+    }
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+
+template <typename T> bool m32_ok(Which which, const Args &a)
+{
+    if (!std::is_same<T, float>::value) return false;
+    if (a.dk_ != a.dv_ || (a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
+    if (which == DQ && !(a.ysaved && a.lse)) return false;
+    const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
+    for (const void *p : ptrs)
+        if (p && !aligned(p, 16)) return false;
+    return true;
+}
+
 bool dense_ok(Which which, const Args &a, bool vec)
 {
     (void)which;
@@ -2564,6 +2600,7 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         if (a.dk_ == 64) return launch_h16<T, 64>(which, a, stream);
         return launch_h16<T, 128>(which, a, stream);
     }
+    if (m32_ok<T>(which, a)) return a.dk_ == 64 ? launch_m32<64>(which, a, stream) : launch_m32<128>(which, a, stream);
     if (dense_ok(which, a, vec)) {
         // the dense kernels handle short runs themselves (vector path inside), so they take every latitude
         (void)ndense;
@@ -2633,12 +2670,14 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
 }
 
 namespace {
-// Shapes of the 16-bit matrix-core kernels.  Their dq pass consumes the forward's output and normaliser; a backward
+// Shapes of the 16-bit and the fp32 (64, 128 channels) matrix-core kernels.  Their dq pass consumes the forward's output and normaliser; a backward
 // that is not handed them (s2attn_backward, s2attn_backward_dq) first recomputes both into the tail of the workspace.
 bool h16_shape(const s2attn_shape *sh)
 {
     const int w = sh->nlon_out < sh->nlon_in ? sh->nlon_out : sh->nlon_in; // columns of a virtual latitude
-    return sh->dtype != S2ATTN_F32 && sh->ck == sh->cv && (sh->ck == 32 || sh->ck == 64 || sh->ck == 128) && w >= HK;
+    if (sh->ck != sh->cv || w < HK) return false;
+    if (sh->dtype == S2ATTN_F32) return sh->ck == 64 || sh->ck == 128; // the fp32 matrix-core family works the same way
+    return sh->ck == 32 || sh->ck == 64 || sh->ck == 128;
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
 int64_t round16(int64_t n) { return (n + 15) / 16 * 16; }
@@ -2650,7 +2689,7 @@ extern "C" int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape)
     if (rc != S2ATTN_OK) return rc;
     const int64_t n = stat_points(shape);
     int64_t bytes = round16(n * (int64_t)sizeof(float2));
-    if (h16_shape(shape)) bytes += round16(n * 4) + n * shape->cv * 2; // lse, y
+    if (h16_shape(shape)) bytes += round16(n * 4) + n * shape->cv * esize(shape->dtype); // lse, y
     return bytes;
 }
 

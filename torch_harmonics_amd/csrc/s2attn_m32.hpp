@@ -1,0 +1,417 @@
+// Matrix-core kernels for fp32 storage and head dims 64 / 128: forward, dq and dk/dv with v_mfma_f32_16x16x4_f32.
+// Included by s2attn_kernels.hip inside namespace s2 after s2attn_h16.hpp, whose tiling they share: one wavefront owns
+// HQ = 16 consecutive longitudes of one latitude for one (batch, head) and walks every run of that latitude in steps of
+// HK = 32 band positions; lane l = (c = l % 16, qd = l / 16); scores are produced transposed, S^T[position][column].
+//
+// Shape domain: ck == cv == D, nlon_in == nlon_out >= 32 on the virtual grid, 16-byte aligned rows.
+//
+// Facts about the instruction:  A operand: the lane supplies A[i = c][k = qd];  B operand: B[k = qd][j = c];
+// D: register v of the lane holds D[i = 4 qd + v][j = c].  The k index of a product is only a summation index, so each
+// product numbers it the way that makes its operands cheap:
+//   scores (K Q^T, V dY^T, ...): k slot qd of instruction s <-> channel qd * D/4 + s.  A lane's B operands are then a
+//     contiguous quarter of its column's vector, loaded once with 16-byte loads and kept in registers, and its A operands
+//     a contiguous quarter of a staged row (16-byte LDS reads, four instructions each);
+//   second products (V^T P^T, K^T dS^T, ...): k slot qd of instruction (kb, v) <-> position 16 kb + 4 qd + v.  B is
+//     register v of score block kb as it stands, A one float of the staged tile (lanes c read consecutive channels).
+
+// fp32 tile of D channels.  With a row pitch of 16 bytes modulo 128 the four-byte reads of the second products (two
+// rows 4 apart per 32 lanes, 16 consecutive floats each) fall in distinct banks.
+template <int D> struct FTile : BandTile<D / 4, 4 * D + 16> {};
+
+__device__ inline f4v m32_mfma(float a, float b, f4v c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
+
+// One 16 x 16 block of transposed scores: rows = staged rows 16 kb + c, summed over the D channels in four independent
+// accumulation chains (smaller partial sums round less, and consecutive instructions do not depend on each other).
+template <int D, int PITCH> __device__ inline f4v m32_scores(const char *tile, int kb, int c, int qd, const float (&op)[D / 4])
+{
+    f4v s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0, s2 = s0, s3 = s0;
+    const char *row = tile + (16 * kb + c) * PITCH + qd * D; // this lane's quarter: D/4 floats = D bytes
+#pragma unroll
+    for (int i = 0; i < D / 16; i++) {
+        const float4 x = *reinterpret_cast<const float4 *>(row + 16 * i);
+        s0 = m32_mfma(x.x, op[4 * i + 0], s0);
+        s1 = m32_mfma(x.y, op[4 * i + 1], s1);
+        s2 = m32_mfma(x.z, op[4 * i + 2], s2);
+        s3 = m32_mfma(x.w, op[4 * i + 3], s3);
+    }
+    return (s0 + s1) + (s2 + s3);
+}
+
+// acc[cb] (channels 16 cb + 4 qd + v of column c) += sum over the 32 staged rows of tile[row][channel] * coef[row][c]
+template <int D, int PITCH> __device__ inline void m32_accumulate(f4v (&acc)[D / 16], const char *tile, int c, int qd, const f4v (&coef)[2])
+{
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+        for (int v = 0; v < 4; v++) {
+            const char *row = tile + (16 * kb + 4 * qd + v) * PITCH + 4 * c;
+#pragma unroll
+            for (int cb = 0; cb < D / 16; cb++) acc[cb] = m32_mfma(*reinterpret_cast<const float *>(row + 64 * cb), coef[kb][v], acc[cb]);
+        }
+    }
+}
+
+// this lane's quarter (channels qd * D/4 ..) of one grid point's vector
+template <int D> __device__ inline void m32_load_quarter(float (&op)[D / 4], const char *vec, int qd, float scale)
+{
+#pragma unroll
+    for (int i = 0; i < D / 16; i++) {
+        const float4 x = *reinterpret_cast<const float4 *>(vec + qd * D + 16 * i);
+        op[4 * i + 0] = x.x * scale;
+        op[4 * i + 1] = x.y * scale;
+        op[4 * i + 2] = x.z * scale;
+        op[4 * i + 3] = x.w * scale;
+    }
+}
+
+// ---- forward ---------------------------------------------------------------------------------------------------
+template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args a)
+{
+    typedef FTile<D> Tile;
+    constexpr int PITCH = Tile::PITCH, NCB = D / 16;
+    __shared__ __attribute__((aligned(16))) char Ks[HK * PITCH];
+    __shared__ __attribute__((aligned(16))) char Vs[HK * PITCH];
+
+    S2_H16_IDS(a.Wo, a.Ho)
+    const int ho = a.gorder[a.row_first + rowsel];
+    const unsigned ldb = a.nh * D * 4; // bytes between two grid points
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
+    const bool mine = c < nvalid;
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
+
+    float qop[D / 4];
+    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (D * 4), qd, 1.0f);
+    f4v acc[NCB]; // Y^T: register v of block cb is channel 16 cb + 4 qd + v of column c
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) acc[cb] = f4v{0.f, 0.f, 0.f, 0.f};
+    float m = NEG_BIG, S = 0.f;
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int pos = 0;
+    Run run = {0, 0, 0, 0};
+    Tile kt, vt;
+    const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
+    auto fetch = [&](const Run &rn, int p) {
+        const int c0 = (rn.ws + w0 + p) % a.Wi;
+        unsigned off[Tile::NIT];
+        Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
+        const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
+        kt.fetch(kx + lat_off, off);
+        vt.fetch(vx + lat_off, off);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+        kt.commit(Ks, lane);
+        vt.commit(Vs, lane);
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const float lw = fast_log2(a.quad_w[run.pad]);
+        const int len = run.len;
+        int nri = ri, npos = pos + HK;
+        Run nrun = run;
+        if (npos >= len + HQ - 1) {
+            nri++;
+            npos = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, npos);
+
+        f4v sc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) sc[kb] = m32_scores<D, PITCH>(Ks, kb, c, qd, qop);
+        // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
+        const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
+        float mx = -INFINITY;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned t = (unsigned)(tb + 16 * kb + v);
+                sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
+                mx = fmaxf(mx, sc[kb][v]);
+            }
+        }
+        mx = h16_quarter_max(mx);
+        const float mn = fmaxf(m, fmaf(mx, LOG2E, lw)); // m starts finite, so mn is finite
+        if (__any(mn > m)) {
+            const float corr = fast_exp2(m - mn);
+            S *= corr;
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
+        }
+        m = mn;
+        const float sh = lw - mn;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // masked: exp2(-inf) = 0
+                sc[kb][v] = p;
+                S += p; // this lane's share; the four lanes of a column are added up at the end
+            }
+        }
+        m32_accumulate<D, PITCH>(acc, Vs, c, qd, sc);
+
+        __syncthreads();
+        if (more) {
+            kt.commit(Ks, lane);
+            vt.commit(Vs, lane);
+        }
+        __syncthreads();
+        ri = nri;
+        pos = npos;
+        run = nrun;
+    }
+
+    S = h16_quarter_sum(S);
+    if (mine) {
+        if (a.lse && qd == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + c] = m + fast_log2(S);
+        const float inv = 1.0f / S;
+        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (D * 4) + 16 * qd;
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++)
+            *reinterpret_cast<float4 *>(y + 64 * cb) = make_float4(acc[cb][0] * inv, acc[cb][1] * inv, acc[cb][2] * inv, acc[cb][3] * inv);
+    }
+}
+
+// ---- backward, dq pass (needs the forward's y and lse) -------------------------------------------------------------
+// Three products per step:  S^T = K Q^T,  G^T = V dY^T,  dQ^T += K^T dS^T  with dS = P o (G - I),  I = <dy, y>.
+template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args a)
+{
+    typedef FTile<D> Tile;
+    constexpr int PITCH = Tile::PITCH, NCB = D / 16;
+    __shared__ __attribute__((aligned(16))) char Ks[HK * PITCH];
+    __shared__ __attribute__((aligned(16))) char Vs[HK * PITCH];
+
+    S2_H16_IDS(a.Wo, a.Ho)
+    const int ho = a.gorder[a.row_first + rowsel];
+    const unsigned ldb = a.nh * D * 4;
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
+    const bool mine = c < nvalid;
+    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
+    const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
+
+    float qop[D / 4], gop[D / 4];
+    float I = 0.f;
+    {
+        const size_t off = pt * ldb + (size_t)h * (D * 4);
+        m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + off, qd, 1.0f);
+        m32_load_quarter<D>(gop, static_cast<const char *>(a.dy) + off, qd, 1.0f);
+        float yq[D / 4];
+        m32_load_quarter<D>(yq, static_cast<const char *>(a.ysaved) + off, qd, 1.0f);
+#pragma unroll
+        for (int i = 0; i < D / 4; i++) I = fmaf(gop[i], yq[i], I);
+    }
+    I = h16_quarter_sum(I);
+    const float lse = a.lse[sidx];
+    if (mine && qd == 0) a.stats[sidx] = make_float2(lse, I);
+
+    f4v acc[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) acc[cb] = f4v{0.f, 0.f, 0.f, 0.f};
+
+    int ri = a.goff[ho];
+    const int rend = a.goff[ho + 1];
+    int pos = 0;
+    Run run = {0, 0, 0, 0};
+    Tile kt, vt;
+    const unsigned ldbk = ldb * a.kps;
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
+    auto fetch = [&](const Run &rn, int p) {
+        const int c0 = (rn.ws + w0 + p) % a.Wi;
+        unsigned off[Tile::NIT];
+        Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
+        const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
+        kt.fetch(kx + lat_off, off);
+        vt.fetch(vx + lat_off, off);
+    };
+    if (ri < rend) {
+        run = a.gruns[ri];
+        fetch(run, 0);
+        kt.commit(Ks, lane);
+        vt.commit(Vs, lane);
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const float lwl = fast_log2(a.quad_w[run.pad]) - lse;
+        const int len = run.len;
+        int nri = ri, npos = pos + HK;
+        Run nrun = run;
+        if (npos >= len + HQ - 1) {
+            nri++;
+            npos = 0;
+            if (nri < rend) nrun = a.gruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, npos);
+
+        f4v sc[2], gc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+            sc[kb] = m32_scores<D, PITCH>(Ks, kb, c, qd, qop);
+            gc[kb] = m32_scores<D, PITCH>(Vs, kb, c, qd, gop);
+        }
+        const int tb = pos + 4 * qd - c;
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned t = (unsigned)(tb + 16 * kb + v);
+                const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
+                gc[kb][v] = p * (gc[kb][v] - I);
+            }
+        }
+        m32_accumulate<D, PITCH>(acc, Ks, c, qd, gc);
+
+        __syncthreads();
+        if (more) {
+            kt.commit(Ks, lane);
+            vt.commit(Vs, lane);
+        }
+        __syncthreads();
+        ri = nri;
+        pos = npos;
+        run = nrun;
+    }
+
+    if (mine) {
+        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (D * 4) + 16 * qd;
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) *reinterpret_cast<float4 *>(dq + 64 * cb) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+    }
+}
+
+// ---- backward, dk/dv pass: transposed gather ---------------------------------------------------------------------
+// The wavefront owns 16 INPUT longitudes (column c = key) and walks the runs grouped by input latitude; staged rows
+// are queries.  Staged row r of a run (first row = longitude w0 - ws - len + 1) sees key c iff 0 <= r - c < len.
+// Four products per step:  S = Q K^T,  G = dY V^T  (rows = queries, columns = keys),  dV^T += dY^T P,  dK^T += Q^T dS.
+template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Args a)
+{
+    typedef FTile<D> Tile;
+    constexpr int PITCH = Tile::PITCH, NCB = D / 16;
+    __shared__ __attribute__((aligned(16))) char Qs[HK * PITCH];
+    __shared__ __attribute__((aligned(16))) char Gs[HK * PITCH];
+    __shared__ __attribute__((aligned(16))) float Ls[HK];
+    __shared__ __attribute__((aligned(16))) float Is[HK];
+
+    S2_H16_IDS(a.Wi, a.Hi)
+    const int hi = a.sorder[a.row_first + rowsel];
+    const unsigned ldb = a.nh * D * 4;
+    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 4);
+    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 4);
+    const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
+    const bool mine = c < nvalid;
+    const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? c : 0)) * a.kps;
+
+    float kop[D / 4], vop[D / 4]; // this lane's quarter of key c
+    {
+        const size_t off = pt * ldb + (size_t)h * (D * 4);
+        m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + off, qd, 1.0f);
+        m32_load_quarter<D>(vop, static_cast<const char *>(a.v) + off, qd, 1.0f);
+    }
+    f4v dkt[NCB], dvt[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) {
+        dkt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
+        dvt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
+    }
+    const float lw = fast_log2(a.quad_w[hi / a.kps]);
+
+    int ri = a.soff[hi];
+    const int rend = a.soff[hi + 1];
+    int pos = 0;
+    Run run = {0, 0, 0, 0};
+    Tile qt, gt;
+    float2 st = make_float2(0.f, 0.f);
+    const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
+    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbq + 16u * (lane % Tile::CPR);
+    auto fetch = [&](const Run &rn, int p) {
+        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
+        c0 += (c0 < 0) ? a.Wo : 0;
+        unsigned off[Tile::NIT];
+        Tile::offsets(off, lane_off, lane, c0, a.Wo, ldbq);
+        const size_t lat_off = (size_t)query_row(a, rn.lat, rn.pad) * ldb;
+        qt.fetch(qy + lat_off, off);
+        gt.fetch(gy + lat_off, off);
+        int col = c0 + lane; // lanes 0..31 fetch the statistics of the staged rows
+        col -= (col >= a.Wo) ? a.Wo : 0;
+        if (lane < HK) st = stats[(size_t)rn.lat * a.Wo + col];
+    };
+    auto commit = [&]() {
+        qt.commit(Qs, lane);
+        gt.commit(Gs, lane);
+        if (lane < HK) {
+            Ls[lane] = st.x;
+            Is[lane] = st.y;
+        }
+    };
+    if (ri < rend) {
+        run = a.sruns[ri];
+        fetch(run, 0);
+        commit();
+    }
+    __syncthreads();
+
+    while (ri < rend) {
+        const int len = run.len;
+        int nri = ri, npos = pos + HK;
+        Run nrun = run;
+        if (npos >= len + HQ - 1) {
+            nri++;
+            npos = 0;
+            if (nri < rend) nrun = a.sruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, npos);
+
+        f4v sc[2], gc[2];
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            sc[qb] = m32_scores<D, PITCH>(Qs, qb, c, qd, kop);
+            gc[qb] = m32_scores<D, PITCH>(Gs, qb, c, qd, vop);
+        }
+        const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 16 * qb + 4 * qd);
+            const float4 i4 = *reinterpret_cast<const float4 *>(Is + 16 * qb + 4 * qd);
+            const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+            const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const unsigned t = (unsigned)(tb + 16 * qb + v);
+                const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v])) : 0.f;
+                sc[qb][v] = p;
+                gc[qb][v] = p * (gc[qb][v] - iv[v]);
+            }
+        }
+        m32_accumulate<D, PITCH>(dvt, Gs, c, qd, sc);
+        m32_accumulate<D, PITCH>(dkt, Qs, c, qd, gc);
+
+        __syncthreads();
+        if (more) commit();
+        __syncthreads();
+        ri = nri;
+        pos = npos;
+        run = nrun;
+    }
+
+    if (mine) {
+        const size_t off = pt * ldb + (size_t)h * (D * 4) + 16 * qd;
+        char *dk = static_cast<char *>(a.dk) + off, *dv = static_cast<char *>(a.dv) + off;
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) {
+            *reinterpret_cast<float4 *>(dk + 64 * cb) = make_float4(dkt[cb][0], dkt[cb][1], dkt[cb][2], dkt[cb][3]);
+            *reinterpret_cast<float4 *>(dv + 64 * cb) = make_float4(dvt[cb][0], dvt[cb][1], dvt[cb][2], dvt[cb][3]);
+        }
+    }
+}
