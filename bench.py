@@ -46,6 +46,9 @@ CONFIGS = {
     "cfg5": dict(
         in_shape=(361, 720), out_shape=(361, 720), grid_in="legendre-gauss", grid_out="legendre-gauss", B=4, C=1024, nh=16, theta_cutoff=8 * math.pi / 360, dtype="bf16"
     ),
+    # not one of the five named configurations: fp32 with 64-channel heads (the head width of the reference's published
+    # benchmark shapes, benchmarks/attention.py:71-112) at a size where throughput, not launch overhead, sets the time
+    "d64": dict(in_shape=(361, 720), out_shape=(361, 720), grid_in="equiangular", grid_out="equiangular", B=2, C=512, nh=8, theta_cutoff=0.03),
 }
 
 
@@ -298,7 +301,12 @@ def main():
     d = k.shape[3] // nh
     # per launch: compulsory traffic (every tensor the kernel must read or write, once), algorithmic flops
     # (2*d per contraction per pair: forward q.k, p.v; dq pass q.k, dy.v, dq; dk/dv pass q.k, dy.v, dk, dv), time
-    kname = ("fwd_h16_kernel", "dq_h16_kernel", "dkdv_h16_kernel") if bf16 else ("fwd_mfma_kernel", "dq_saved_mfma_kernel", "dkdv_mfma_kernel")
+    if bf16:
+        kname = ("fwd_h16_kernel", "dq_h16_kernel", "dkdv_h16_kernel")
+    elif d in (64, 128):
+        kname = ("fwd_m32_kernel", "dq_m32_kernel", "dkdv_m32_kernel")
+    else:
+        kname = ("fwd_mfma_kernel", "dq_saved_mfma_kernel", "dkdv_mfma_kernel")
     alg = {
         f"s2::{kname[0]} (forward)": (esz * (nq + nk + nv + ny) + 4 * nstat, 4 * d * pairs, t_fwd),
         f"s2::{kname[1]} (backward, dq)": (esz * (nq + nk + nv + ny + ny + nq) + 12 * nstat, 6 * d * pairs, t_dq),

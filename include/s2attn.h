@@ -129,8 +129,10 @@ int s2attn_forward_lse(const void *k, const void *v, const void *q, const float 
  * Backward.  Replaces attention_kernels::backward (attention_interface.cpp:117-119;
  * CUDA implementation s2_attention_bwd_dkvq_cuda, attention_cuda_bwd.cu:856-956).
  * Writes dk, dv, dq (every element; no pre-zeroing needed, no atomics).
- * workspace: device fp32 scratch of s2attn_backward_workspace_bytes(shape) bytes
- * holding two softmax statistics per (batch, head, output point).
+ * workspace: device scratch of s2attn_backward_workspace_bytes(shape) bytes, 8-byte aligned (16 for the matrix-core
+ * shapes below): two fp32 softmax statistics per (batch, head, output point), plus, for the shapes whose dq pass works
+ * from the forward's output and normaliser (16-bit storage with head dim 32 / 64 / 128, fp32 with head dim 64 / 128,
+ * ck == cv, at least 32 columns per virtual latitude), room to recompute those two when the caller does not pass them.
  */
 int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape);
 
@@ -155,8 +157,9 @@ int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void
 /*
  * Backward from saved forward results: y (the forward output) and lse (from s2attn_forward_lse) make the softmax
  * final from the first neighbor on, which saves one of the four matrix products of the dq pass and all running-maximum
- * bookkeeping.  Same outputs as s2attn_backward to rounding; same workspace.  Shapes outside the matrix-core kernels'
- * domain (head dim != 32, nlon_in != nlon_out, nlon < 64) ignore y and lse and take the s2attn_backward path.
+ * bookkeeping.  Same outputs as s2attn_backward to rounding; same workspace.  Shapes that run on the vector kernels
+ * (head dims other than 32 / 64 / 128, ck != cv, narrow grids, unaligned tensors) ignore y and lse and take the
+ * s2attn_backward path.
  */
 int s2attn_backward_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
                           const float *quad_weights, void *dk, void *dv, void *dq, void *workspace, const s2attn_plan *plan,
