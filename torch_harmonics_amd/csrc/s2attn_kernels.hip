@@ -2550,7 +2550,7 @@ template <typename T> bool h16_ok(Which which, const Args &a)
     return true;
 }
 
-// fp32 matrix-core kernels for 64- and 128-channel heads: same launch geometry and the same conditions as the 16-bit family.
+// fp32 matrix-core kernels for 16-, 32-, 64- and 128-channel heads: same launch geometry and the same conditions as the 16-bit family.
 template <int D> int launch_m32(Which which, const Args &a0, hipStream_t stream)
 {
     Args a = a0;
@@ -2577,7 +2577,7 @@ template <int D> int launch_m32(Which which, const Args &a0, hipStream_t stream)
 template <typename T> bool m32_ok(Which which, const Args &a)
 {
     if (!std::is_same<T, float>::value) return false;
-    if (a.dk_ != a.dv_ || (a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
+    if (a.dk_ != a.dv_ || (a.dk_ != 16 && a.dk_ != 32 && a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
     if (which == DQ && !(a.ysaved && a.lse)) return false;
     const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
     for (const void *p : ptrs)
@@ -2600,14 +2600,16 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         if (a.dk_ == 64) return launch_h16<T, 64>(which, a, stream);
         return launch_h16<T, 128>(which, a, stream);
     }
-    if (m32_ok<T>(which, a)) return a.dk_ == 64 ? launch_m32<64>(which, a, stream) : launch_m32<128>(which, a, stream);
     if (dense_ok(which, a, vec)) {
-        // the dense kernels handle short runs themselves (vector path inside), so they take every latitude
+        // head dim 32 on at least 64 columns: the hybrid kernels handle short runs themselves (vector path inside), so
+        // they take every latitude; measured ahead of the 16-longitude family there (cfg3 13.5 against 16.4 ms)
         (void)ndense;
-        const int take = nrows;
-        const int rc = launch_dense<T>(which, a, take, stream);
-        if (rc != S2ATTN_OK) return rc;
-        first = take;
+        return launch_dense<T>(which, a, nrows, stream);
+    }
+    if (m32_ok<T>(which, a)) {
+        if (a.dk_ == 16) return launch_m32<16>(which, a, stream);
+        if (a.dk_ == 32) return launch_m32<32>(which, a, stream);
+        return a.dk_ == 64 ? launch_m32<64>(which, a, stream) : launch_m32<128>(which, a, stream);
     }
     return vec ? launch_p<T, true>(which, a, first, nrows - first, stream) : launch_p<T, false>(which, a, first, nrows - first, stream);
 }
@@ -2676,7 +2678,8 @@ bool h16_shape(const s2attn_shape *sh)
 {
     const int w = sh->nlon_out < sh->nlon_in ? sh->nlon_out : sh->nlon_in; // columns of a virtual latitude
     if (sh->ck != sh->cv || w < HK) return false;
-    if (sh->dtype == S2ATTN_F32) return sh->ck == 64 || sh->ck == 128; // the fp32 matrix-core family works the same way
+    if (sh->dtype == S2ATTN_F32) // the fp32 16-longitude family works the same way (head dim 32: only below the hybrid kernels' 64 columns)
+        return sh->ck == 16 || (sh->ck == 32 && w < 64) || sh->ck == 64 || sh->ck == 128;
     return sh->ck == 32 || sh->ck == 64 || sh->ck == 128;
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
