@@ -303,7 +303,7 @@ def main():
     # (2*d per contraction per pair: forward q.k, p.v; dq pass q.k, dy.v, dq; dk/dv pass q.k, dy.v, dk, dv), time
     if bf16:
         kname = ("fwd_h16_kernel", "dq_h16_kernel", "dkdv_h16_kernel")
-    elif d in (64, 128):
+    elif d in (16, 64, 128) or (d == 32 and min(Wi, Wo) < 64):
         kname = ("fwd_m32_kernel", "dq_m32_kernel", "dkdv_m32_kernel")
     else:
         kname = ("fwd_mfma_kernel", "dq_saved_mfma_kernel", "dkdv_mfma_kernel")
