@@ -84,6 +84,12 @@ SMALL_CASES = [
     (1, 1, 64, 64, (10, 80), (10, 80), "equiangular", "equiangular", 1.2),
     (2, 2, 64, 64, (9, 44), (9, 44), "legendre-gauss", "legendre-gauss", 0.6),
     (1, 2, 128, 128, (8, 40), (8, 40), "equiangular", "equiangular", 0.9),
+    # the same family with heads narrower than its 16 / 32 / 64 / 128-channel tiles (any multiple of 4 from 16 up)
+    (1, 1, 48, 48, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
+    (1, 2, 96, 96, (8, 36), (8, 36), "legendre-gauss", "legendre-gauss", 0.8),
+    (1, 3, 20, 20, (12, 48), (12, 48), "equiangular", "equiangular", 0.5),
+    (2, 1, 100, 100, (6, 32), (6, 32), "equiangular", "equiangular", 0.9),
+    (1, 2, 48, 48, (12, 96), (6, 48), "equiangular", "equiangular", 0.5),
     (1, 1, 128, 128, (10, 72), (5, 36), "equiangular", "legendre-gauss", 0.7),
     # head dim 32 on grids wide enough for the matrix-core kernels (nlon >= 64), incl. full-circle rows and long runs
     (1, 2, 32, 32, (24, 96), (24, 96), "equiangular", "equiangular", 0.5),
@@ -178,6 +184,7 @@ SAVED_CASES = [
     (2, 1, 64, 64, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
     (1, 1, 64, 64, (8, 40), (8, 40), "equiangular", "equiangular", 7.0),
     (1, 1, 128, 128, (8, 36), (8, 36), "equiangular", "equiangular", 0.8),
+    (1, 2, 40, 40, (8, 36), (8, 36), "equiangular", "equiangular", 0.8),
     (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
     (1, 1, 128, 128, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
 ]

@@ -85,6 +85,16 @@ template <int CPR_, int PITCH_> struct BandTile {
 #pragma unroll
         for (int it = 0; it < NIT; it++) raw[it] = *reinterpret_cast<const u4v *>(src + off[it]);
     }
+    // the same for a lane that may own a piece beyond the end of the row (a head narrower than the tile): it stages zeros
+    __device__ inline void fetch_if(const char *src, const unsigned (&off)[NIT], bool valid)
+    {
+#pragma unroll
+        for (int it = 0; it < NIT; it++) raw[it] = u4v{0u, 0u, 0u, 0u};
+        if (valid) {
+#pragma unroll
+            for (int it = 0; it < NIT; it++) raw[it] = *reinterpret_cast<const u4v *>(src + off[it]);
+        }
+    }
     __device__ inline void commit(char *dst, int lane) const
     {
         const int r0 = lane / CPR, cb = 16 * (lane % CPR);

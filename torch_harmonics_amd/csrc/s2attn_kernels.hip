@@ -2550,7 +2550,7 @@ template <typename T> bool h16_ok(Which which, const Args &a)
     return true;
 }
 
-// fp32 matrix-core kernels for 16-, 32-, 64- and 128-channel heads: same launch geometry and the same conditions as the 16-bit family.
+// fp32 16-longitude matrix-core kernels, tiles of 16, 32, 64 or 128 channels: same launch geometry and the same conditions as the 16-bit family.
 template <int D> int launch_m32(Which which, const Args &a0, hipStream_t stream)
 {
     Args a = a0;
@@ -2574,10 +2574,13 @@ template <int D> int launch_m32(Which which, const Args &a0, hipStream_t stream)
     return S2ATTN_OK;
 }
 
+// Head widths: any multiple of 4 from 16 to 128, staged in a tile of 16, 32, 64 or 128 channels (zeros past the head).
+bool m32_width(int ck, int cv) { return ck == cv && ck % 4 == 0 && ck >= 16 && ck <= 128; }
+
 template <typename T> bool m32_ok(Which which, const Args &a)
 {
     if (!std::is_same<T, float>::value) return false;
-    if (a.dk_ != a.dv_ || (a.dk_ != 16 && a.dk_ != 32 && a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
+    if (!m32_width(a.dk_, a.dv_) || a.Wi < HK) return false;
     if (which == DQ && !(a.ysaved && a.lse)) return false;
     const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
     for (const void *p : ptrs)
@@ -2607,9 +2610,9 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         return launch_dense<T>(which, a, nrows, stream);
     }
     if (m32_ok<T>(which, a)) {
-        if (a.dk_ == 16) return launch_m32<16>(which, a, stream);
-        if (a.dk_ == 32) return launch_m32<32>(which, a, stream);
-        return a.dk_ == 64 ? launch_m32<64>(which, a, stream) : launch_m32<128>(which, a, stream);
+        if (a.dk_ <= 16) return launch_m32<16>(which, a, stream);
+        if (a.dk_ <= 32) return launch_m32<32>(which, a, stream);
+        return a.dk_ <= 64 ? launch_m32<64>(which, a, stream) : launch_m32<128>(which, a, stream);
     }
     return vec ? launch_p<T, true>(which, a, first, nrows - first, stream) : launch_p<T, false>(which, a, first, nrows - first, stream);
 }
@@ -2672,14 +2675,14 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
 }
 
 namespace {
-// Shapes of the 16-bit and the fp32 (64, 128 channels) matrix-core kernels.  Their dq pass consumes the forward's output and normaliser; a backward
+// Shapes of the 16-bit and the fp32 16-longitude matrix-core kernels.  Their dq pass consumes the forward's output and normaliser; a backward
 // that is not handed them (s2attn_backward, s2attn_backward_dq) first recomputes both into the tail of the workspace.
 bool h16_shape(const s2attn_shape *sh)
 {
     const int w = sh->nlon_out < sh->nlon_in ? sh->nlon_out : sh->nlon_in; // columns of a virtual latitude
     if (sh->ck != sh->cv || w < HK) return false;
     if (sh->dtype == S2ATTN_F32) // the fp32 16-longitude family works the same way (head dim 32: only below the hybrid kernels' 64 columns)
-        return sh->ck == 16 || (sh->ck == 32 && w < 64) || sh->ck == 64 || sh->ck == 128;
+        return m32_width(sh->ck, sh->cv) && !(sh->ck == 32 && w >= 64);
     return sh->ck == 32 || sh->ck == 64 || sh->ck == 128;
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }

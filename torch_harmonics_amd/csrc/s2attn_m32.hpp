@@ -3,7 +3,8 @@
 // HQ = 16 consecutive longitudes of one latitude for one (batch, head) and walks every run of that latitude in steps of
 // HK = 32 band positions; lane l = (c = l % 16, qd = l / 16); scores are produced transposed, S^T[position][column].
 //
-// Shape domain: ck == cv == D, nlon_in == nlon_out >= 32 on the virtual grid, 16-byte aligned rows.
+// Shape domain: ck == cv = dr, a multiple of 4 with dr <= D (the tile is D channels wide; channels from dr on are staged
+// as zeros and never stored), at least 32 columns per virtual latitude, 16-byte aligned rows.
 //
 // Facts about the instruction:  A operand: the lane supplies A[i = c][k = qd];  B operand: B[k = qd][j = c];
 // D: register v of the lane holds D[i = 4 qd + v][j = c].  The k index of a product is only a summation index, so each
@@ -51,16 +52,17 @@ template <int D, int PITCH> __device__ inline void m32_accumulate(f4v (&acc)[D /
     }
 }
 
-// this lane's quarter (channels qd * D/4 ..) of one grid point's vector
-template <int D> __device__ inline void m32_load_quarter(float (&op)[D / 4], const char *vec, int qd, float scale)
+// this lane's quarter (channels qd * D/4 ..) of one grid point's vector of dr channels; zeros from channel dr on
+template <int D> __device__ inline void m32_load_quarter(float (&op)[D / 4], const char *vec, int qd, int dr)
 {
 #pragma unroll
     for (int i = 0; i < D / 16; i++) {
-        const float4 x = *reinterpret_cast<const float4 *>(vec + qd * D + 16 * i);
-        op[4 * i + 0] = x.x * scale;
-        op[4 * i + 1] = x.y * scale;
-        op[4 * i + 2] = x.z * scale;
-        op[4 * i + 3] = x.w * scale;
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (qd * (D / 4) + 4 * i < dr) x = *reinterpret_cast<const float4 *>(vec + qd * D + 16 * i);
+        op[4 * i + 0] = x.x;
+        op[4 * i + 1] = x.y;
+        op[4 * i + 2] = x.z;
+        op[4 * i + 3] = x.w;
     }
 }
 
@@ -74,14 +76,15 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
 
     S2_H16_IDS(a.Wo, a.Ho)
     const int ho = a.gorder[a.row_first + rowsel];
-    const unsigned ldb = a.nh * D * 4; // bytes between two grid points
-    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
-    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
+    const int dr = a.dk_;              // real head width
+    const unsigned ldb = a.nh * dr * 4; // bytes between two grid points
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
     const bool mine = c < nvalid;
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
 
     float qop[D / 4];
-    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (D * 4), qd, 1.0f);
+    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (dr * 4), qd, dr);
     f4v acc[NCB]; // Y^T: register v of block cb is channel 16 cb + 4 qd + v of column c
 #pragma unroll
     for (int cb = 0; cb < NCB; cb++) acc[cb] = f4v{0.f, 0.f, 0.f, 0.f};
@@ -94,13 +97,14 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
     Tile kt, vt;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
     const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         unsigned off[Tile::NIT];
         Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        kt.fetch(kx + lat_off, off);
-        vt.fetch(vx + lat_off, off);
+        kt.fetch_if(kx + lat_off, off, piece_ok);
+        vt.fetch_if(vx + lat_off, off, piece_ok);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -174,10 +178,11 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
     if (mine) {
         if (a.lse && qd == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + c] = m + fast_log2(S);
         const float inv = 1.0f / S;
-        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (D * 4) + 16 * qd;
+        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++)
-            *reinterpret_cast<float4 *>(y + 64 * cb) = make_float4(acc[cb][0] * inv, acc[cb][1] * inv, acc[cb][2] * inv, acc[cb][3] * inv);
+            if (16 * cb + 4 * qd < dr)
+                *reinterpret_cast<float4 *>(y + 64 * cb) = make_float4(acc[cb][0] * inv, acc[cb][1] * inv, acc[cb][2] * inv, acc[cb][3] * inv);
     }
 }
 
@@ -192,9 +197,10 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
 
     S2_H16_IDS(a.Wo, a.Ho)
     const int ho = a.gorder[a.row_first + rowsel];
-    const unsigned ldb = a.nh * D * 4;
-    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
-    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 4);
+    const int dr = a.dk_;
+    const unsigned ldb = a.nh * dr * 4;
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
     const bool mine = c < nvalid;
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
     const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
@@ -202,11 +208,11 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
     float qop[D / 4], gop[D / 4];
     float I = 0.f;
     {
-        const size_t off = pt * ldb + (size_t)h * (D * 4);
-        m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + off, qd, 1.0f);
-        m32_load_quarter<D>(gop, static_cast<const char *>(a.dy) + off, qd, 1.0f);
+        const size_t off = pt * ldb + (size_t)h * (dr * 4);
+        m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + off, qd, dr);
+        m32_load_quarter<D>(gop, static_cast<const char *>(a.dy) + off, qd, dr);
         float yq[D / 4];
-        m32_load_quarter<D>(yq, static_cast<const char *>(a.ysaved) + off, qd, 1.0f);
+        m32_load_quarter<D>(yq, static_cast<const char *>(a.ysaved) + off, qd, dr);
 #pragma unroll
         for (int i = 0; i < D / 4; i++) I = fmaf(gop[i], yq[i], I);
     }
@@ -225,13 +231,14 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
     Tile kt, vt;
     const unsigned ldbk = ldb * a.kps;
     const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         unsigned off[Tile::NIT];
         Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        kt.fetch(kx + lat_off, off);
-        vt.fetch(vx + lat_off, off);
+        kt.fetch_if(kx + lat_off, off, piece_ok);
+        vt.fetch_if(vx + lat_off, off, piece_ok);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -284,9 +291,10 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
     }
 
     if (mine) {
-        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (D * 4) + 16 * qd;
+        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) *reinterpret_cast<float4 *>(dq + 64 * cb) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+        for (int cb = 0; cb < NCB; cb++)
+            if (16 * cb + 4 * qd < dr) *reinterpret_cast<float4 *>(dq + 64 * cb) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
     }
 }
 
@@ -305,18 +313,19 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
 
     S2_H16_IDS(a.Wi, a.Hi)
     const int hi = a.sorder[a.row_first + rowsel];
-    const unsigned ldb = a.nh * D * 4;
-    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 4);
-    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 4);
+    const int dr = a.dk_;
+    const unsigned ldb = a.nh * dr * 4;
+    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (dr * 4);
+    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (dr * 4);
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = c < nvalid;
     const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? c : 0)) * a.kps;
 
     float kop[D / 4], vop[D / 4]; // this lane's quarter of key c
     {
-        const size_t off = pt * ldb + (size_t)h * (D * 4);
-        m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + off, qd, 1.0f);
-        m32_load_quarter<D>(vop, static_cast<const char *>(a.v) + off, qd, 1.0f);
+        const size_t off = pt * ldb + (size_t)h * (dr * 4);
+        m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + off, qd, dr);
+        m32_load_quarter<D>(vop, static_cast<const char *>(a.v) + off, qd, dr);
     }
     f4v dkt[NCB], dvt[NCB];
 #pragma unroll
@@ -334,14 +343,15 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
     float2 st = make_float2(0.f, 0.f);
     const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
     const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbq + 16u * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
         unsigned off[Tile::NIT];
         Tile::offsets(off, lane_off, lane, c0, a.Wo, ldbq);
         const size_t lat_off = (size_t)query_row(a, rn.lat, rn.pad) * ldb;
-        qt.fetch(qy + lat_off, off);
-        gt.fetch(gy + lat_off, off);
+        qt.fetch_if(qy + lat_off, off, piece_ok);
+        gt.fetch_if(gy + lat_off, off, piece_ok);
         int col = c0 + lane; // lanes 0..31 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
         if (lane < HK) st = stats[(size_t)rn.lat * a.Wo + col];
@@ -406,12 +416,14 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
     }
 
     if (mine) {
-        const size_t off = pt * ldb + (size_t)h * (D * 4) + 16 * qd;
+        const size_t off = pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
         char *dk = static_cast<char *>(a.dk) + off, *dv = static_cast<char *>(a.dv) + off;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++) {
-            *reinterpret_cast<float4 *>(dk + 64 * cb) = make_float4(dkt[cb][0], dkt[cb][1], dkt[cb][2], dkt[cb][3]);
-            *reinterpret_cast<float4 *>(dv + 64 * cb) = make_float4(dvt[cb][0], dvt[cb][1], dvt[cb][2], dvt[cb][3]);
+            if (16 * cb + 4 * qd < dr) {
+                *reinterpret_cast<float4 *>(dk + 64 * cb) = make_float4(dkt[cb][0], dkt[cb][1], dkt[cb][2], dkt[cb][3]);
+                *reinterpret_cast<float4 *>(dv + 64 * cb) = make_float4(dvt[cb][0], dvt[cb][1], dvt[cb][2], dvt[cb][3]);
+            }
         }
     }
 }
