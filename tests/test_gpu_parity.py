@@ -184,7 +184,11 @@ SAVED_CASES = [
     (2, 1, 64, 64, (12, 70), (12, 70), "equiangular", "equiangular", 0.35),
     (1, 1, 64, 64, (8, 40), (8, 40), "equiangular", "equiangular", 7.0),
     (1, 1, 128, 128, (8, 36), (8, 36), "equiangular", "equiangular", 0.8),
+    # heads narrower than the matrix-core tiles (zero-padded in LDS): multiples of 8 for 16-bit storage, of 4 for fp32
     (1, 2, 40, 40, (8, 36), (8, 36), "equiangular", "equiangular", 0.8),
+    (1, 1, 96, 96, (8, 40), (8, 40), "legendre-gauss", "legendre-gauss", 0.7),
+    (2, 1, 24, 24, (8, 48), (8, 48), "equiangular", "equiangular", 0.6),
+    (1, 2, 16, 16, (12, 64), (6, 32), "equiangular", "equiangular", 0.6),
     (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
     (1, 1, 128, 128, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
 ]

@@ -1,7 +1,8 @@
 // Matrix-core kernels for 16-bit storage (bf16, fp16): forward, dq and dk/dv with v_mfma_f32_16x16x32_{bf16,f16}.
 // Included by s2attn_kernels.hip inside namespace s2 (uses its Args, Run and storage types).
 //
-// Shape domain: ck == cv == D (a multiple of 32), nlon_in == nlon_out >= 32, 16-byte aligned rows.
+// Shape domain: ck == cv = dr, a multiple of 8 with dr <= D (the tile is D channels wide, D a multiple of 32; channels
+// from dr on are staged as zeros and never stored), at least 32 columns per virtual latitude, 16-byte aligned rows.
 //
 // One wavefront owns HQ = 16 consecutive longitudes of one latitude for one (batch, head) and walks every run of that
 // latitude in steps of HK = 32 band positions (len + 15 positions per run; position u belongs to the neighborhood of
@@ -88,11 +89,12 @@ template <int CPR_, int PITCH_> struct BandTile {
     // the same for a lane that may own a piece beyond the end of the row (a head narrower than the tile): it stages zeros
     __device__ inline void fetch_if(const char *src, const unsigned (&off)[NIT], bool valid)
     {
-#pragma unroll
-        for (int it = 0; it < NIT; it++) raw[it] = u4v{0u, 0u, 0u, 0u};
         if (valid) {
 #pragma unroll
             for (int it = 0; it < NIT; it++) raw[it] = *reinterpret_cast<const u4v *>(src + off[it]);
+        } else {
+#pragma unroll
+            for (int it = 0; it < NIT; it++) raw[it] = u4v{0u, 0u, 0u, 0u};
         }
     }
     __device__ inline void commit(char *dst, int lane) const
@@ -123,6 +125,14 @@ template <int PITCH> __device__ inline uint4 h16_read_transposed(const char *til
 template <int PITCH> __device__ inline uint4 h16_read_row(const char *tile, int kb, int s, int c, int qd)
 {
     return *reinterpret_cast<const uint4 *>(tile + (16 * kb + c) * PITCH + 64 * s + 16 * qd);
+}
+
+// one 16-byte piece of a grid point's vector, zeros when the head ends before it
+__device__ inline uint4 h16_load_piece(const char *p, bool ok)
+{
+    uint4 r = make_uint4(0u, 0u, 0u, 0u);
+    if (ok) r = *reinterpret_cast<const uint4 *>(p);
+    return r;
 }
 
 __device__ inline float h16_quarter_max(float x)
@@ -166,7 +176,7 @@ __device__ inline void xcd_split(int id, int BH, int per_bh, int &bh, int &rest)
     const int nvalid = min(HQ, (W_TILED)-w0);
 
 // ---- forward ---------------------------------------------------------------------------------------------------
-template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kernel(const Args a)
+template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void fwd_h16_kernel(const Args a)
 {
     typedef HTile<D> Tile;
     typedef H16<T> M;
@@ -176,17 +186,18 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
 
     S2_H16_IDS(a.Wo, a.Ho)
     const int ho = a.gorder[a.row_first + rowsel];
-    const unsigned ldb = a.nh * D * 2; // bytes between two grid points
-    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
-    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
+    const int dr = PAD ? a.dk_ : D;     // real head width (PAD = false: a compile-time constant, every mask below folds away)
+    const unsigned ldb = a.nh * dr * 2; // bytes between two grid points
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 2);
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 2);
     const bool mine = c < nvalid;
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
 
     uint4 qop[NS]; // B operand of S^T = K Q^T: channels 32 s + 8 qd .. + 8 of column c
     {
-        const char *qrow = static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (D * 2) + 16 * qd;
+        const char *qrow = static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (dr * 2) + 16 * qd;
 #pragma unroll
-        for (int s = 0; s < NS; s++) qop[s] = *reinterpret_cast<const uint4 *>(qrow + 64 * s);
+        for (int s = 0; s < NS; s++) qop[s] = h16_load_piece(qrow + 64 * s, 32 * s + 8 * qd < dr);
     }
     f4v acc[NCB]; // Y^T: register v of block cb is channel 16 cb + 4 qd + v of column c
 #pragma unroll
@@ -200,13 +211,14 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
     Tile kt, vt;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
     const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
+    const bool piece_ok = 8 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         unsigned off[Tile::NIT];
         Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        kt.fetch(kx + lat_off, off);
-        vt.fetch(vx + lat_off, off);
+        kt.fetch_if(kx + lat_off, off, piece_ok);
+        vt.fetch_if(vx + lat_off, off, piece_ok);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -286,16 +298,17 @@ template <typename T, int D> __global__ __launch_bounds__(64) void fwd_h16_kerne
     if (mine) {
         if (a.lse && qd == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + c] = m + fast_log2(S);
         const float inv = 1.0f / S;
-        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (D * 2) + 8 * qd;
+        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (dr * 2) + 8 * qd;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++)
-            *reinterpret_cast<uint2 *>(y + 32 * cb) = make_uint2(M::pack2(acc[cb][0] * inv, acc[cb][1] * inv), M::pack2(acc[cb][2] * inv, acc[cb][3] * inv));
+            if (16 * cb + 4 * qd < dr)
+                *reinterpret_cast<uint2 *>(y + 32 * cb) = make_uint2(M::pack2(acc[cb][0] * inv, acc[cb][1] * inv), M::pack2(acc[cb][2] * inv, acc[cb][3] * inv));
     }
 }
 
 // ---- backward, dq pass (needs the forward's y and lse) -------------------------------------------------------------
 // Three products per step:  S^T = K Q^T,  G^T = V dY^T,  dQ^T += K^T dS^T  with dS = P o (G - I),  I = <dy, y>.
-template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel(const Args a)
+template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_h16_kernel(const Args a)
 {
     typedef HTile<D> Tile;
     typedef H16<T> M;
@@ -305,9 +318,10 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
 
     S2_H16_IDS(a.Wo, a.Ho)
     const int ho = a.gorder[a.row_first + rowsel];
-    const unsigned ldb = a.nh * D * 2;
-    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
-    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (D * 2);
+    const int dr = PAD ? a.dk_ : D;
+    const unsigned ldb = a.nh * dr * 2;
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 2);
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 2);
     const bool mine = c < nvalid;
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
     const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
@@ -315,12 +329,13 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
     uint4 qop[NS], gop[NS];
     float I = 0.f;
     {
-        const size_t off = pt * ldb + (size_t)h * (D * 2) + 16 * qd;
+        const size_t off = pt * ldb + (size_t)h * (dr * 2) + 16 * qd;
 #pragma unroll
         for (int s = 0; s < NS; s++) {
-            qop[s] = *reinterpret_cast<const uint4 *>(static_cast<const char *>(a.q) + off + 64 * s);
-            gop[s] = *reinterpret_cast<const uint4 *>(static_cast<const char *>(a.dy) + off + 64 * s);
-            const uint4 yv = *reinterpret_cast<const uint4 *>(static_cast<const char *>(a.ysaved) + off + 64 * s);
+            const bool ok = 32 * s + 8 * qd < dr;
+            qop[s] = h16_load_piece(static_cast<const char *>(a.q) + off + 64 * s, ok);
+            gop[s] = h16_load_piece(static_cast<const char *>(a.dy) + off + 64 * s, ok);
+            const uint4 yv = h16_load_piece(static_cast<const char *>(a.ysaved) + off + 64 * s, ok);
             const unsigned gu[4] = {gop[s].x, gop[s].y, gop[s].z, gop[s].w}, yu[4] = {yv.x, yv.y, yv.z, yv.w};
 #pragma unroll
             for (int i = 0; i < 4; i++) {
@@ -345,13 +360,14 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
     Tile kt, vt;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
     const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
+    const bool piece_ok = 8 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
         const int c0 = (rn.ws + w0 + p) % a.Wi;
         unsigned off[Tile::NIT];
         Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        kt.fetch(kx + lat_off, off);
-        vt.fetch(vx + lat_off, off);
+        kt.fetch_if(kx + lat_off, off, piece_ok);
+        vt.fetch_if(vx + lat_off, off, piece_ok);
     };
     if (ri < rend) {
         run = a.gruns[ri];
@@ -411,10 +427,11 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
     }
 
     if (mine) {
-        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (D * 2) + 8 * qd;
+        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (dr * 2) + 8 * qd;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++)
-            *reinterpret_cast<uint2 *>(dq + 32 * cb) = make_uint2(M::pack2(acc[cb][0], acc[cb][1]), M::pack2(acc[cb][2], acc[cb][3]));
+            if (16 * cb + 4 * qd < dr)
+                *reinterpret_cast<uint2 *>(dq + 32 * cb) = make_uint2(M::pack2(acc[cb][0], acc[cb][1]), M::pack2(acc[cb][2], acc[cb][3]));
     }
 }
 
@@ -422,7 +439,7 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dq_h16_kernel
 // The wavefront owns 16 INPUT longitudes (column c = key) and walks the runs grouped by input latitude; staged rows
 // are queries.  Staged row r of a run (first row = longitude w0 - ws - len + 1) sees key c iff 0 <= r - c < len.
 // Four products per step:  S = Q K^T,  G = dY V^T  (rows = queries, columns = keys),  dV^T += dY^T P,  dK^T += Q^T dS.
-template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kernel(const Args a)
+template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dkdv_h16_kernel(const Args a)
 {
     typedef HTile<D> Tile;
     typedef H16<T> M;
@@ -434,20 +451,22 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
 
     S2_H16_IDS(a.Wi, a.Hi)
     const int hi = a.sorder[a.row_first + rowsel];
-    const unsigned ldb = a.nh * D * 2;
-    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 2);
-    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (D * 2);
+    const int dr = PAD ? a.dk_ : D;
+    const unsigned ldb = a.nh * dr * 2;
+    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (dr * 2);
+    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (dr * 2);
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = c < nvalid;
     const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? c : 0)) * a.kps;
 
     uint4 kop[NS], vop[NS]; // B operands: channels 32 s + 8 qd .. + 8 of key c
     {
-        const size_t off = pt * ldb + (size_t)h * (D * 2) + 16 * qd;
+        const size_t off = pt * ldb + (size_t)h * (dr * 2) + 16 * qd;
 #pragma unroll
         for (int s = 0; s < NS; s++) {
-            kop[s] = *reinterpret_cast<const uint4 *>(static_cast<const char *>(a.k) + off + 64 * s);
-            vop[s] = *reinterpret_cast<const uint4 *>(static_cast<const char *>(a.v) + off + 64 * s);
+            const bool ok = 32 * s + 8 * qd < dr;
+            kop[s] = h16_load_piece(static_cast<const char *>(a.k) + off + 64 * s, ok);
+            vop[s] = h16_load_piece(static_cast<const char *>(a.v) + off + 64 * s, ok);
         }
     }
     f4v dkt[NCB], dvt[NCB];
@@ -466,14 +485,15 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
     float2 st = make_float2(0.f, 0.f);
     const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
     const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbq + 16u * (lane % Tile::CPR);
+    const bool piece_ok = 8 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
         unsigned off[Tile::NIT];
         Tile::offsets(off, lane_off, lane, c0, a.Wo, ldbq);
         const size_t lat_off = (size_t)query_row(a, rn.lat, rn.pad) * ldb;
-        qt.fetch(qy + lat_off, off);
-        gt.fetch(gy + lat_off, off);
+        qt.fetch_if(qy + lat_off, off, piece_ok);
+        gt.fetch_if(gy + lat_off, off, piece_ok);
         int col = c0 + lane; // lanes 0..31 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
         if (lane < HK) st = stats[(size_t)rn.lat * a.Wo + col];
@@ -548,12 +568,14 @@ template <typename T, int D> __global__ __launch_bounds__(64) void dkdv_h16_kern
     }
 
     if (mine) {
-        const size_t off = pt * ldb + (size_t)h * (D * 2) + 8 * qd;
+        const size_t off = pt * ldb + (size_t)h * (dr * 2) + 8 * qd;
         char *dk = static_cast<char *>(a.dk) + off, *dv = static_cast<char *>(a.dv) + off;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++) {
-            *reinterpret_cast<uint2 *>(dk + 32 * cb) = make_uint2(M::pack2(dkt[cb][0], dkt[cb][1]), M::pack2(dkt[cb][2], dkt[cb][3]));
-            *reinterpret_cast<uint2 *>(dv + 32 * cb) = make_uint2(M::pack2(dvt[cb][0], dvt[cb][1]), M::pack2(dvt[cb][2], dvt[cb][3]));
+            if (16 * cb + 4 * qd < dr) {
+                *reinterpret_cast<uint2 *>(dk + 32 * cb) = make_uint2(M::pack2(dkt[cb][0], dkt[cb][1]), M::pack2(dkt[cb][2], dkt[cb][3]));
+                *reinterpret_cast<uint2 *>(dv + 32 * cb) = make_uint2(M::pack2(dvt[cb][0], dvt[cb][1]), M::pack2(dvt[cb][2], dvt[cb][3]));
+            }
         }
     }
 }

@@ -2512,7 +2512,7 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
 
 // 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
 // dq pass exists only in the form that takes the forward's y and lse.
-template <typename T, int D> int launch_h16(Which which, const Args &a0, hipStream_t stream)
+template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream)
 {
     if constexpr (std::is_same<T, float>::value) {
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "16-bit kernels asked for fp32 storage");
@@ -2522,13 +2522,13 @@ template <typename T, int D> int launch_h16(Which which, const Args &a0, hipStre
         void (*kern)(const Args) = nullptr;
         long nblocks = 0;
         if (which == FWD) {
-            kern = fwd_h16_kernel<T, D>;
+            kern = fwd_h16_kernel<T, D, PAD>;
             nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
         } else if (which == DQ) {
-            kern = dq_h16_kernel<T, D>;
+            kern = dq_h16_kernel<T, D, PAD>;
             nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
         } else {
-            kern = dkdv_h16_kernel<T, D>;
+            kern = dkdv_h16_kernel<T, D, PAD>;
             nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
         }
         if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
@@ -2539,10 +2539,13 @@ template <typename T, int D> int launch_h16(Which which, const Args &a0, hipStre
     }
 }
 
+// Head widths: any multiple of 8 from 16 to 128, staged in a tile of 32, 64 or 128 channels (zeros past the head).
+bool h16_width(int ck, int cv) { return ck == cv && ck % 8 == 0 && ck >= 16 && ck <= 128; }
+
 template <typename T> bool h16_ok(Which which, const Args &a)
 {
     if (std::is_same<T, float>::value) return false;
-    if (a.dk_ != a.dv_ || (a.dk_ != 32 && a.dk_ != 64 && a.dk_ != 128) || a.Wi < HK) return false;
+    if (!h16_width(a.dk_, a.dv_) || a.Wi < HK) return false;
     if (which == DQ && !(a.ysaved && a.lse)) return false;
     const void *ptrs[] = {a.k, a.v, a.q, a.dy, a.y, a.dk, a.dv, a.dq, a.ysaved};
     for (const void *p : ptrs)
@@ -2599,9 +2602,12 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
     const int nrows = which == DKDV ? a.Hi : a.Ho;
     int first = 0;
     if (h16_ok<T>(which, a)) {
-        if (a.dk_ == 32) return launch_h16<T, 32>(which, a, stream);
-        if (a.dk_ == 64) return launch_h16<T, 64>(which, a, stream);
-        return launch_h16<T, 128>(which, a, stream);
+        if (a.dk_ == 32) return launch_h16<T, 32, false>(which, a, stream);
+        if (a.dk_ == 64) return launch_h16<T, 64, false>(which, a, stream);
+        if (a.dk_ == 128) return launch_h16<T, 128, false>(which, a, stream);
+        if (a.dk_ < 32) return launch_h16<T, 32, true>(which, a, stream);
+        if (a.dk_ < 64) return launch_h16<T, 64, true>(which, a, stream);
+        return launch_h16<T, 128, true>(which, a, stream);
     }
     if (dense_ok(which, a, vec)) {
         // head dim 32 on at least 64 columns: the hybrid kernels handle short runs themselves (vector path inside), so
@@ -2683,7 +2689,7 @@ bool h16_shape(const s2attn_shape *sh)
     if (sh->ck != sh->cv || w < HK) return false;
     if (sh->dtype == S2ATTN_F32) // the fp32 16-longitude family works the same way (head dim 32: only below the hybrid kernels' 64 columns)
         return m32_width(sh->ck, sh->cv) && !(sh->ck == 32 && w >= 64);
-    return sh->ck == 32 || sh->ck == 64 || sh->ck == 128;
+    return h16_width(sh->ck, sh->cv);
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
 int64_t round16(int64_t n) { return (n + 15) / 16 * 16; }
