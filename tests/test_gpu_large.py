@@ -20,7 +20,7 @@ def _setup(name, heads=None, batch=None, seed=333):
     from torch_harmonics_amd.neighborhood import precompute_neighborhood_s2
     from torch_harmonics_amd.quadrature import precompute_latitudes
 
-    c = CONFIGS[name]
+    c = name if isinstance(name, dict) else CONFIGS[name]
     (Hi, Wi), (Ho, Wo) = c["in_shape"], c["out_shape"]
     nh = heads or c["nh"]
     B = batch or c["B"]
@@ -115,6 +115,26 @@ def test_cfg4_downsampling_sampled_rows():
     assert_close("cfg4 dq pole", dq[:, 0:6].cpu(), dq64[:, 0:6], **TOL)
     assert_close("cfg4 dk pole", dk[:, 0:4].cpu(), dk64[:, 0:4], **TOL)
     assert_close("cfg4 dv pole", dv[:, 0:4].cpu(), dv64[:, 0:4], **TOL)
+
+
+# the reference's published benchmark shape (benchmarks/attention.py:71-112: B = 1, C = 64, one head) at 360 x 720, fp32
+PUB64 = dict(in_shape=(360, 720), out_shape=(360, 720), grid_in="equiangular", grid_out="equiangular", B=1, C=64, nh=1, theta_cutoff=0.03)
+
+
+@pytest.mark.parametrize("saved", [False, True], ids=["recompute", "saved"])
+def test_published_shape_head64_fp32_sampled_rows(saved):
+    """One head of 64 channels in fp32 (the fp32 16-longitude matrix-core kernels): pole rows (2,000+ neighbors per
+    point), equator, and the gradients of the input latitudes whose contributing rows are all checked."""
+    c, (Hi, Wi, Ho, Wo, nh, d), col, roff, w, k, v, q, dy = _setup(PUB64)
+    y, dk, dv, dq = _hip(k, v, q, dy, w, col, roff, nh, (Hi, Wi, Ho, Wo), saved=saved)
+    # cutoff 0.03 rad = 3.4 latitude spacings: output rows 170..190 complete the input latitudes 174..186
+    dk64, dv64 = _check_rows("pub64", [0, 1, 3, 180, 358, 359], (170, 191), k, v, q, dy, w, col, roff, nh, y, dk, dv, dq, 4)
+    assert_close("pub64 dk equator", dk[:, 174:187].cpu(), dk64[:, 174:187], **TOL)
+    assert_close("pub64 dv equator", dv[:, 174:187].cpu(), dv64[:, 174:187], **TOL)
+    dk64, dv64, dq64 = oracle.backward_f64(k, v, q, dy, w, col, roff, nh, ho_range=(0, 9))
+    assert_close("pub64 dq pole", dq[:, 0:9].cpu(), dq64[:, 0:9], **TOL)
+    assert_close("pub64 dk pole", dk[:, 0:5].cpu(), dk64[:, 0:5], **TOL)
+    assert_close("pub64 dv pole", dv[:, 0:5].cpu(), dv64[:, 0:5], **TOL)
 
 
 def test_cfg2_full_size_forward_and_sampled_backward():
