@@ -135,6 +135,18 @@ __device__ inline uint4 h16_load_piece(const char *p, bool ok)
     return r;
 }
 
+// Values that a kernel loads from global memory before its main loop and keeps in registers for the whole walk are
+// passed through settle() right before the loop.  The empty asm uses the register, so the wait for the load is placed
+// there; without it the compiler (which cannot see that the loop only runs on a path that has already waited) puts a
+// vmcnt(0) at the first use INSIDE the loop, and that also waits for the tile prefetch issued just before it, every step.
+__device__ inline void settle(float &x) { asm("" : "+v"(x)); }
+__device__ inline void settle(uint4 &x) { asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w)); }
+template <typename V, int N> __device__ inline void settle(V (&x)[N])
+{
+#pragma unroll
+    for (int i = 0; i < N; i++) settle(x[i]);
+}
+
 __device__ inline float h16_quarter_max(float x)
 {
     return xor32_max(xor16_max(x));
@@ -227,6 +239,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void fwd
         vt.commit(Vs, lane);
     }
     __syncthreads();
+    settle(qop);
 
     while (ri < rend) {
         const float lw = fast_log2(a.quad_w[run.pad]);
@@ -347,7 +360,6 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
     }
     I = h16_quarter_sum(I);
     const float lse = a.lse[sidx];
-    if (mine && qd == 0) a.stats[sidx] = make_float2(lse, I);
 
     f4v acc[NCB];
 #pragma unroll
@@ -376,9 +388,13 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
         vt.commit(Vs, lane);
     }
     __syncthreads();
+    settle(qop);
+    settle(gop);
+    float lse_ = lse;
+    settle(lse_);
 
     while (ri < rend) {
-        const float lwl = fast_log2(a.quad_w[run.pad]) - lse;
+        const float lwl = fast_log2(a.quad_w[run.pad]) - lse_;
         const int len = run.len;
         int nri = ri, npos = pos + HK;
         Run nrun = run;
@@ -426,6 +442,9 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
         run = nrun;
     }
 
+    // (stored after the walk: a global store ahead of the loop would turn the loop's scalar loads of runs and weights,
+    // which the compiler only uses while nothing in the kernel can have written memory, into vector loads with waits)
+    if (mine && qd == 0) a.stats[sidx] = make_float2(lse, I);
     if (mine) {
         char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (dr * 2) + 8 * qd;
 #pragma unroll
@@ -512,6 +531,8 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dkd
         commit();
     }
     __syncthreads();
+    settle(kop);
+    settle(vop);
 
     while (ri < rend) {
         const int len = run.len;

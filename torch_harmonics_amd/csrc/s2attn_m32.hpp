@@ -21,34 +21,62 @@ template <int D> struct FTile : BandTile<D / 4, 4 * D + 16> {};
 
 __device__ inline f4v m32_mfma(float a, float b, f4v c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
 
-// One 16 x 16 block of transposed scores: rows = staged rows 16 kb + c, summed over the D channels in four independent
-// accumulation chains (smaller partial sums round less, and consecutive instructions do not depend on each other).
-template <int D, int PITCH> __device__ inline f4v m32_scores(const char *tile, int kb, int c, int qd, const float (&op)[D / 4])
+// Both 16 x 16 blocks of transposed scores of a step: rows = staged rows 16 kb + c, summed over the D channels in four
+// independent accumulation chains per block (smaller partial sums round less, and consecutive instructions do not depend
+// on each other).  The LDS reads run LA pieces ahead of the instructions that consume them; the scheduling barriers keep
+// the compiler from folding each read back next to its use, which would expose the LDS latency once per four instructions.
+template <int D, int PITCH> __device__ inline void m32_scores(f4v (&sc)[2], const char *tile, int c, int qd, const float (&op)[D / 4])
 {
-    f4v s0 = {0.f, 0.f, 0.f, 0.f}, s1 = s0, s2 = s0, s3 = s0;
-    const char *row = tile + (16 * kb + c) * PITCH + qd * D; // this lane's quarter: D/4 floats = D bytes
+    constexpr int NP = D / 16, NF = 2 * NP, LA = NF < 4 ? NF : 4;
+    const char *row = tile + c * PITCH + qd * D; // this lane's quarter of staged row c: D/4 floats = D bytes
+    float4 x[NF];
+    f4v s[2][4];
 #pragma unroll
-    for (int i = 0; i < D / 16; i++) {
-        const float4 x = *reinterpret_cast<const float4 *>(row + 16 * i);
-        s0 = m32_mfma(x.x, op[4 * i + 0], s0);
-        s1 = m32_mfma(x.y, op[4 * i + 1], s1);
-        s2 = m32_mfma(x.z, op[4 * i + 2], s2);
-        s3 = m32_mfma(x.w, op[4 * i + 3], s3);
+    for (int kb = 0; kb < 2; kb++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) s[kb][j] = f4v{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int i = 0; i < LA; i++) x[i] = *reinterpret_cast<const float4 *>(row + (i / NP) * 16 * PITCH + 16 * (i % NP));
+#pragma unroll
+    for (int i = 0; i < NF; i++) {
+        if (i + LA < NF) x[i + LA] = *reinterpret_cast<const float4 *>(row + ((i + LA) / NP) * 16 * PITCH + 16 * ((i + LA) % NP));
+        __builtin_amdgcn_sched_barrier(0);
+        const int kb = i / NP, p = i % NP;
+        s[kb][0] = m32_mfma(x[i].x, op[4 * p + 0], s[kb][0]);
+        s[kb][1] = m32_mfma(x[i].y, op[4 * p + 1], s[kb][1]);
+        s[kb][2] = m32_mfma(x[i].z, op[4 * p + 2], s[kb][2]);
+        s[kb][3] = m32_mfma(x[i].w, op[4 * p + 3], s[kb][3]);
+        __builtin_amdgcn_sched_barrier(0);
     }
-    return (s0 + s1) + (s2 + s3);
+#pragma unroll
+    for (int kb = 0; kb < 2; kb++) sc[kb] = (s[kb][0] + s[kb][1]) + (s[kb][2] + s[kb][3]);
 }
 
-// acc[cb] (channels 16 cb + 4 qd + v of column c) += sum over the 32 staged rows of tile[row][channel] * coef[row][c]
+// acc[cb] (channels 16 cb + 4 qd + v of column c) += sum over the 32 staged rows of tile[row][channel] * coef[row][c].
+// The eight rows of this lane (kb, v) are taken two at a time; the operands of the next two pairs are in flight while
+// one pair is consumed.
 template <int D, int PITCH> __device__ inline void m32_accumulate(f4v (&acc)[D / 16], const char *tile, int c, int qd, const f4v (&coef)[2])
 {
+    constexpr int NCB = D / 16;
+    float av[4][2][NCB];
+    const char *base = tile + (4 * qd) * PITCH + 4 * c;
+    auto load = [&](int g) { // rows (kb = g / 2, v = 2 (g % 2) + r), r < 2
 #pragma unroll
-    for (int kb = 0; kb < 2; kb++) {
+        for (int r = 0; r < 2; r++)
 #pragma unroll
-        for (int v = 0; v < 4; v++) {
-            const char *row = tile + (16 * kb + 4 * qd + v) * PITCH + 4 * c;
+            for (int cb = 0; cb < NCB; cb++) av[g][r][cb] = *reinterpret_cast<const float *>(base + (16 * (g / 2) + 2 * (g % 2) + r) * PITCH + 64 * cb);
+    };
+    load(0);
+    load(1);
 #pragma unroll
-            for (int cb = 0; cb < D / 16; cb++) acc[cb] = m32_mfma(*reinterpret_cast<const float *>(row + 64 * cb), coef[kb][v], acc[cb]);
-        }
+    for (int g = 0; g < 4; g++) {
+        if (g + 2 < 4) load(g + 2);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int r = 0; r < 2; r++)
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[cb] = m32_mfma(av[g][r][cb], coef[g / 2][2 * (g % 2) + r], acc[cb]);
+        __builtin_amdgcn_sched_barrier(0);
     }
 }
 
@@ -113,6 +141,7 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
         vt.commit(Vs, lane);
     }
     __syncthreads();
+    settle(qop);
 
     while (ri < rend) {
         const float lw = fast_log2(a.quad_w[run.pad]);
@@ -128,8 +157,7 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
         if (more) fetch(nrun, npos);
 
         f4v sc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) sc[kb] = m32_scores<D, PITCH>(Ks, kb, c, qd, qop);
+        m32_scores<D, PITCH>(sc, Ks, c, qd, qop);
         // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
         const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
         float mx = -INFINITY;
@@ -218,7 +246,6 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
     }
     I = h16_quarter_sum(I);
     const float lse = a.lse[sidx];
-    if (mine && qd == 0) a.stats[sidx] = make_float2(lse, I);
 
     f4v acc[NCB];
 #pragma unroll
@@ -247,9 +274,13 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
         vt.commit(Vs, lane);
     }
     __syncthreads();
+    settle(qop);
+    settle(gop);
+    float lse_ = lse;
+    settle(lse_);
 
     while (ri < rend) {
-        const float lwl = fast_log2(a.quad_w[run.pad]) - lse;
+        const float lwl = fast_log2(a.quad_w[run.pad]) - lse_;
         const int len = run.len;
         int nri = ri, npos = pos + HK;
         Run nrun = run;
@@ -262,11 +293,8 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
         if (more) fetch(nrun, npos);
 
         f4v sc[2], gc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            sc[kb] = m32_scores<D, PITCH>(Ks, kb, c, qd, qop);
-            gc[kb] = m32_scores<D, PITCH>(Vs, kb, c, qd, gop);
-        }
+        m32_scores<D, PITCH>(sc, Ks, c, qd, qop);
+        m32_scores<D, PITCH>(gc, Vs, c, qd, gop);
         const int tb = pos + 4 * qd - c;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
@@ -290,6 +318,9 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
         run = nrun;
     }
 
+    // (stored after the walk: a global store ahead of the loop would turn the loop's scalar loads of runs and weights,
+    // which the compiler only uses while nothing in the kernel can have written memory, into vector loads with waits)
+    if (mine && qd == 0) a.stats[sidx] = make_float2(lse, I);
     if (mine) {
         char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
 #pragma unroll
@@ -370,6 +401,8 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
         commit();
     }
     __syncthreads();
+    settle(kop);
+    settle(vop);
 
     while (ri < rend) {
         const int len = run.len;
@@ -384,11 +417,8 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
         if (more) fetch(nrun, npos);
 
         f4v sc[2], gc[2];
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++) {
-            sc[qb] = m32_scores<D, PITCH>(Qs, qb, c, qd, kop);
-            gc[qb] = m32_scores<D, PITCH>(Gs, qb, c, qd, vop);
-        }
+        m32_scores<D, PITCH>(sc, Qs, c, qd, kop);
+        m32_scores<D, PITCH>(gc, Gs, c, qd, vop);
         const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
