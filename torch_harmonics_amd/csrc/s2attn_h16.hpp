@@ -135,18 +135,6 @@ __device__ inline uint4 h16_load_piece(const char *p, bool ok)
     return r;
 }
 
-// Values that a kernel loads from global memory before its main loop and keeps in registers for the whole walk are
-// passed through settle() right before the loop.  The empty asm uses the register, so the wait for the load is placed
-// there; without it the compiler (which cannot see that the loop only runs on a path that has already waited) puts a
-// vmcnt(0) at the first use INSIDE the loop, and that also waits for the tile prefetch issued just before it, every step.
-__device__ inline void settle(float &x) { asm("" : "+v"(x)); }
-__device__ inline void settle(uint4 &x) { asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w)); }
-template <typename V, int N> __device__ inline void settle(V (&x)[N])
-{
-#pragma unroll
-    for (int i = 0; i < N; i++) settle(x[i]);
-}
-
 __device__ inline float h16_quarter_max(float x)
 {
     return xor32_max(xor16_max(x));

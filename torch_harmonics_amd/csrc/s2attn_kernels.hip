@@ -184,6 +184,18 @@ __device__ inline float xor16_max(float x)
     return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
 }
 
+// Values that a kernel loads from global memory before its main loop and keeps in registers for the whole walk are
+// passed through settle() right before the loop.  The empty asm uses the register, so the wait for the load is placed
+// there; without it the compiler (which cannot see that the loop only runs on a path that has already waited) puts a
+// vmcnt(0) at the first use INSIDE the loop, and that also waits for the tile prefetch issued just before it, every step.
+__device__ inline void settle(float &x) { asm("" : "+v"(x)); }
+__device__ inline void settle(uint4 &x) { asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w)); }
+template <typename V, int N> __device__ inline void settle(V (&x)[N])
+{
+#pragma unroll
+    for (int i = 0; i < N; i++) settle(x[i]);
+}
+
 // ---- LDS staging -------------------------------------------------------------------
 // Copies `nrows` grid points (longitudes c0, c0+1, ... wrapping at W) of one latitude and
 // one head into LDS as fp32 rows of P floats (zero padded past d), row stride P+4 floats so
@@ -1811,6 +1823,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const
         vt.commit(Vs, lane, !run_is_dense(run.len));
     }
     __syncthreads();
+    settle(qb);
+    settle(gb);
 
     while (ri < rend) {
         const float w = a.quad_w[run.pad];
@@ -2016,8 +2030,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
         }
         I = xor32_sum(I);
     }
-    const float lse = a.lse[sidx];
-    if (mine && half == 0) a.stats[sidx] = make_float2(lse, I);
+    float lse = a.lse[sidx];
     f16v dqt;
 #pragma unroll
     for (int v = 0; v < 16; v++) dqt[v] = 0.f;
@@ -2040,6 +2053,9 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
         vt.commit(Vs, lane, !run_is_dense(run.len));
     }
     __syncthreads();
+    settle(qb);
+    settle(gb);
+    settle(lse);
 
     while (ri < rend) {
         const float w = a.quad_w[run.pad];
@@ -2139,6 +2155,9 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
         run = nrun;
     }
 
+    // (stored after the walk: a global store ahead of the loop would turn the loop's scalar loads of runs and weights,
+    // which the compiler only uses while nothing in the kernel can have written memory, into vector loads with waits)
+    if (mine && half == 0) a.stats[sidx] = make_float2(lse, I);
     if (mine) {
         T *dq = static_cast<T *>(a.dq) + pt * ldk + (size_t)h * 32 + 4 * half;
 #pragma unroll
@@ -2218,6 +2237,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
         commit(!run_is_dense(run.len));
     }
     __syncthreads();
+    settle(kb);
+    settle(vb);
 
     while (ri < rend) {
         const int len = run.len;
