@@ -189,6 +189,9 @@ SAVED_CASES = [
     (1, 1, 96, 96, (8, 40), (8, 40), "legendre-gauss", "legendre-gauss", 0.7),
     (2, 1, 24, 24, (8, 48), (8, 48), "equiangular", "equiangular", 0.6),
     (1, 2, 16, 16, (12, 64), (6, 32), "equiangular", "equiangular", 0.6),
+    # up to 256 channels per head on the 16-bit matrix-core kernels (fp32: wide vector kernels)
+    (1, 1, 256, 256, (8, 40), (8, 40), "equiangular", "equiangular", 0.8),
+    (1, 2, 192, 192, (6, 36), (6, 36), "legendre-gauss", "legendre-gauss", 0.9),
     (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
     (1, 1, 128, 128, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
 ]

@@ -2560,8 +2560,8 @@ template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a
     }
 }
 
-// Head widths: any multiple of 8 from 16 to 128, staged in a tile of 32, 64 or 128 channels (zeros past the head).
-bool h16_width(int ck, int cv) { return ck == cv && ck % 8 == 0 && ck >= 16 && ck <= 128; }
+// Head widths: any multiple of 8 from 16 to 256, staged in a tile of 32, 64, 128 or 256 channels (zeros past the head).
+bool h16_width(int ck, int cv) { return ck == cv && ck % 8 == 0 && ck >= 16 && ck <= 256; }
 
 template <typename T> bool h16_ok(Which which, const Args &a)
 {
@@ -2628,7 +2628,8 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         if (a.dk_ == 128) return launch_h16<T, 128, false>(which, a, stream);
         if (a.dk_ < 32) return launch_h16<T, 32, true>(which, a, stream);
         if (a.dk_ < 64) return launch_h16<T, 64, true>(which, a, stream);
-        return launch_h16<T, 128, true>(which, a, stream);
+        if (a.dk_ < 128) return launch_h16<T, 128, true>(which, a, stream);
+        return launch_h16<T, 256, true>(which, a, stream);
     }
     if (dense_ok(which, a, vec)) {
         // head dim 32 on at least 64 columns: the hybrid kernels handle short runs themselves (vector path inside), so
