@@ -181,6 +181,56 @@ int s2attn_permute_to_nhwc(const void *src, void *dst, int64_t B, int64_t C, int
 int s2attn_permute_to_nchw(const void *src, void *dst, int64_t B, int64_t H, int64_t W, int64_t C, int elem_size,
                            void *stream);
 
+/*
+ * Ring-step variants of the gather direction (nlon_in a multiple of nlon_out): the pieces a longitude-sharded layer is
+ * built from.  K/V arrive one longitude chunk at a time (in such a layer the chunks travel around a ring of devices);
+ * q, dy and the per-point softmax state stay with the caller.  Each call handles ONE chunk on ONE device and talks to
+ * nobody.  Replace attention_kernels::forward_ring_step, backward_ring_step_pass1, backward_ring_step_pass2
+ * (attention_interface.cpp:138-156; CUDA: attention_cuda_fwd_ring.cu:66-175, attention_cuda_bwd_ring.cu:78-205 and
+ * 1312-1440; caller: torch_harmonics/distributed/distributed_attention.py:141-176, 303-431).
+ *
+ * Tensors (heads folded into the batch, NHWC, contiguous):
+ *   k, v         [batch, nlat_halo, nlon_kx, ck / cv]   the chunk: input latitudes lat_halo_start .. + nlat_halo,
+ *                                                      input longitudes lon_lo_kx .. + nlon_kx
+ *   q, dy        [batch, nlat_out, nlon_out, ck / cv]   local output points
+ *   y_acc        [batch, nlat_out, nlon_out, cv] fp32;  alpha_sum, qdotk_max, integral(_norm) [batch, nlat_out, nlon_out] fp32
+ *   alpha_k, alpha_kvw [batch, nlat_out, nlon_out, ck] fp32;   dk, dv: fp32, shaped like k, v (ADDED to, atomically)
+ *   quad_weights [global nlat_in] fp32, indexed by global input latitude
+ *   col_idx, row_off: the local CSR in device memory, int64: row_off has nlat_out + 1 entries, col_idx = hi_global *
+ *     nlon_in + wi with wi already shifted by pscale * (first local output longitude); row_idx (int32, nlat_out entries,
+ *     may be null) is the order in which output latitudes are launched.
+ * State starts as y_acc = alpha_sum = integral = alpha_k = alpha_kvw = 0, qdotk_max = -inf; after all chunks
+ *   y = y_acc / alpha_sum,   dq = (alpha_sum * alpha_kvw - integral * alpha_k) / alpha_sum^2,   integral_norm = integral / alpha_sum.
+ * The statistics are in the natural-exponential domain, as the reference's.
+ */
+typedef struct s2attn_ring_shape {
+    int32_t batch;          /* batch * heads */
+    int32_t nlat_halo;      /* input latitudes held in the chunk */
+    int32_t nlon_kx;        /* input longitudes held in the chunk */
+    int32_t nlat_out;       /* local output latitudes */
+    int32_t nlon_out;       /* local output longitudes */
+    int32_t ck, cv;         /* channels of k/q and of v/y (<= 512) */
+    int32_t nlon_in;        /* global input longitudes */
+    int32_t pscale;         /* global nlon_in / global nlon_out */
+    int32_t lon_lo_kx;      /* first global input longitude of the chunk */
+    int32_t lat_halo_start; /* first global input latitude of the chunk */
+    int32_t dtype;          /* S2ATTN_F32 / BF16 / F16: storage of k, v, q, dy */
+} s2attn_ring_shape;
+
+int s2attn_ring_forward_step(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                             const float *quad_weights, const int64_t *col_idx, const int64_t *row_off, const int32_t *row_idx,
+                             const s2attn_ring_shape *shape, void *stream);
+
+int s2attn_ring_backward_pass1(const void *k, const void *v, const void *q, const void *dy, float *alpha_sum, float *qdotk_max,
+                               float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                               const int64_t *col_idx, const int64_t *row_off, const int32_t *row_idx,
+                               const s2attn_ring_shape *shape, void *stream);
+
+int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                               const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                               const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
+                               const int32_t *row_idx, const s2attn_ring_shape *shape, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1,0 +1,129 @@
+"""
+Ring-step operators on the GPU (through the C ABI) against the CPU restatement oracle/cpu_ring.py after EVERY step, and,
+after the last chunk, against the dense float64 softmax attention and its autograd gradients on the rank's output window.
+The reference exercises these operators single-rank through opcheck only (tests/test_attention.py:894-1062).
+"""
+
+import pytest
+import torch
+
+from oracle import cpu_attention as oracle
+from oracle import cpu_ring as ring
+from tests.ring_util import RING_CASES, chunk_of, fresh_state, local_problem
+from tests.util import assert_close
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+TOL = dict(rtol=1e-5, atol=1e-5)
+
+
+def _geo_dev(p):
+    return p["quad"].to(DEV), p["col_l"].to(DEV), p["roff_l"].to(DEV), p["row_idx"].to(DEV)
+
+
+@pytest.mark.parametrize("case", RING_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_ring_steps_against_oracle_and_dense_attention(case, dtype):
+    from torch_harmonics_amd import ops
+
+    print(f"case {case} {dtype}", flush=True)
+    ck, cv = (70, 33) if case is RING_CASES[1] else (5, 3)  # one case with more than 64 channels (two per lane)
+    p = local_problem(case, ck=ck, cv=cv)
+    for name in ("k", "v", "q", "dy", "q_l", "dy_l"):  # the values the storage dtype can hold, shared by all three evaluations
+        p[name] = p[name].to(dtype).float()
+    B, Wi = p["k"].shape[0], p["ins"][1]
+    tol = TOL if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    stol = dict(rtol=1e-5, atol=1e-5)  # state against the oracle fed the same stored values: storage dtype plays no role
+    quad, col_l, roff_l, row_idx = _geo_dev(p)
+    split = ops.split_csr_rows(p["row_idx"], p["roff_l"], p["nlat_loc"])
+    tail = lambda c: (Wi, p["pscale"], p["chunks"][c][0], p["halo"][0], p["nlat_loc"], p["nlon_loc"], *split)  # noqa: E731
+    ogeo = lambda c: (p["quad"], p["col_l"], p["roff_l"], Wi, p["pscale"], p["chunks"][c][0], p["halo"][0])  # noqa: E731
+    qd, gd = p["q_l"].to(DEV, dtype), p["dy_l"].to(DEV, dtype)
+    q64, g64 = p["q_l"].double(), p["dy_l"].double()
+    nchunk = len(p["chunks"])
+    steps = [(1 + i) % nchunk for i in range(nchunk)]
+
+    st = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    ref = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float64)
+    for c in steps:
+        kc, vc = chunk_of(p, p["k"], c), chunk_of(p, p["v"], c)
+        ops.forward_ring_step(kc.to(DEV, dtype), vc.to(DEV, dtype), qd, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col_l, roff_l, row_idx, *tail(c))
+        ring.forward_step(kc.double(), vc.double(), q64, ref["y_acc"], ref["alpha_sum"], ref["qdotk_max"], *ogeo(c))
+        torch.cuda.synchronize()
+        seen = torch.isfinite(ref["qdotk_max"])
+        assert torch.equal(torch.isfinite(st["qdotk_max"]).cpu(), seen)
+        assert_close(f"qdotk_max after chunk {c}", st["qdotk_max"].cpu()[seen], ref["qdotk_max"][seen], **stol)
+        assert_close(f"alpha_sum after chunk {c}", st["alpha_sum"].cpu(), ref["alpha_sum"], **stol)
+        assert_close(f"y_acc after chunk {c}", st["y_acc"].cpu(), ref["y_acc"], **stol)
+
+    k, v, q = [t.double().requires_grad_(True) for t in (p["k"], p["v"], p["q"])]
+    y = oracle.dense_attention_f64(k, v, q, p["quad"], p["col"], p["roff"], 1)
+    la, na, lo, no = p["lat_lo"], p["nlat_loc"], p["lon_lo"], p["nlon_loc"]
+    win = y[:, la : la + na, lo : lo + no]
+    (win * g64).sum().backward()
+    assert_close("y", (st["y_acc"] / st["alpha_sum"][..., None]).cpu(), win.detach(), **tol)
+
+    bw = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    rbw = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float64)
+    for c in steps:
+        kc, vc = chunk_of(p, p["k"], c), chunk_of(p, p["v"], c)
+        ops.backward_ring_step_pass1(
+            kc.to(DEV, dtype), vc.to(DEV, dtype), qd, gd, bw["alpha_sum"], bw["qdotk_max"], bw["integral"], bw["alpha_k"], bw["alpha_kvw"],
+            quad, col_l, roff_l, row_idx, *tail(c),
+        )  # fmt: skip
+        ring.backward_pass1(kc.double(), vc.double(), q64, g64, rbw["alpha_sum"], rbw["qdotk_max"], rbw["integral"], rbw["alpha_k"], rbw["alpha_kvw"], *ogeo(c))
+        torch.cuda.synchronize()
+        assert_close(f"integral after chunk {c}", bw["integral"].cpu(), rbw["integral"], **stol)
+        assert_close(f"alpha_k after chunk {c}", bw["alpha_k"].cpu(), rbw["alpha_k"], **stol)
+        assert_close(f"alpha_kvw after chunk {c}", bw["alpha_kvw"].cpu(), rbw["alpha_kvw"], **stol)
+    assert_close("pass 1 alpha_sum == forward alpha_sum", bw["alpha_sum"], st["alpha_sum"], rtol=1e-6, atol=0)
+    S = st["alpha_sum"][..., None]
+    dq = (S * bw["alpha_kvw"] - bw["integral"][..., None] * bw["alpha_k"]) / S**2
+    assert_close("dq", dq.cpu(), q.grad[:, la : la + na, lo : lo + no], **tol)
+
+    integral_norm = (bw["integral"] / st["alpha_sum"]).contiguous()
+    dk, dv = torch.zeros_like(p["k"]), torch.zeros_like(p["v"])
+    h0, h1 = p["halo"]
+    for c in steps:
+        kc, vc = chunk_of(p, p["k"], c), chunk_of(p, p["v"], c)
+        dkc, dvc = torch.zeros(kc.shape, device=DEV), torch.zeros(vc.shape, device=DEV)
+        ops.backward_ring_step_pass2(
+            kc.to(DEV, dtype), vc.to(DEV, dtype), qd, gd, st["alpha_sum"], st["qdotk_max"], integral_norm, dkc, dvc, quad, col_l, roff_l, row_idx, *tail(c)
+        )
+        clo, chi = p["chunks"][c]
+        dk[:, h0:h1, clo:chi] += dkc.cpu()
+        dv[:, h0:h1, clo:chi] += dvc.cpu()
+    assert_close("dk", dk, k.grad, **tol)
+    assert_close("dv", dv, v.grad, **tol)
+
+
+def test_ring_ops_pass_opcheck_and_leave_state_alone_without_neighbors():
+    from torch_harmonics_amd import ops
+
+    p = local_problem(RING_CASES[2])
+    B, ck, cv, Wi = p["k"].shape[0], p["k"].shape[3], p["v"].shape[3], p["ins"][1]
+    quad, col_l, roff_l, row_idx = _geo_dev(p)
+    split = ops.split_csr_rows(p["row_idx"], p["roff_l"], p["nlat_loc"])
+    qd, gd = p["q_l"].to(DEV), p["dy_l"].to(DEV)
+    kc, vc = chunk_of(p, p["k"], 1).to(DEV), chunk_of(p, p["v"], 1).to(DEV)
+    tail = (Wi, p["pscale"], p["chunks"][1][0], p["halo"][0], p["nlat_loc"], p["nlon_loc"], *split)
+    st = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    torch.library.opcheck(ops.forward_ring_step, (kc, vc, qd, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col_l, roff_l, row_idx, *tail))
+    torch.library.opcheck(
+        ops.backward_ring_step_pass1, (kc, vc, qd, gd, st["alpha_sum"], st["qdotk_max"], st["integral"], st["alpha_k"], st["alpha_kvw"], quad, col_l, roff_l, row_idx, *tail)
+    )
+    st2 = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    ops.forward_ring_step(kc, vc, qd, st2["y_acc"], st2["alpha_sum"], st2["qdotk_max"], quad, col_l, roff_l, row_idx, *tail)
+    norm = (st2["integral"] * 0).contiguous()
+    torch.library.opcheck(
+        ops.backward_ring_step_pass2,
+        (kc, vc, qd, gd, st2["alpha_sum"].clamp_min(1e-30), st2["qdotk_max"].clamp_min(-1e30), norm, torch.zeros_like(kc), torch.zeros_like(vc), quad, col_l, roff_l, row_idx, *tail),
+    )
+    # a halo that holds none of the neighbor latitudes: the state must come back bit for bit
+    st3 = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    far = (Wi, p["pscale"], 0, 1000, p["nlat_loc"], p["nlon_loc"], *split)
+    ops.forward_ring_step(kc, vc, qd, st3["y_acc"], st3["alpha_sum"], st3["qdotk_max"], quad, col_l, roff_l, row_idx, *far)
+    torch.cuda.synchronize()
+    assert float(st3["alpha_sum"].abs().max()) == 0.0 and bool(torch.isinf(st3["qdotk_max"]).all()) and float(st3["y_acc"].abs().max()) == 0.0
+    with pytest.raises(RuntimeError):  # chunk outside the input grid
+        ops.forward_ring_step(kc, vc, qd, st3["y_acc"], st3["alpha_sum"], st3["qdotk_max"], quad, col_l, roff_l, row_idx, Wi, p["pscale"], Wi - 1, 0, p["nlat_loc"], p["nlon_loc"], *split)

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -50,6 +50,23 @@ class ShapeStruct(ctypes.Structure):
     ]
 
 
+class RingShapeStruct(ctypes.Structure):
+    _fields_ = [
+        ("batch", ctypes.c_int32),
+        ("nlat_halo", ctypes.c_int32),
+        ("nlon_kx", ctypes.c_int32),
+        ("nlat_out", ctypes.c_int32),
+        ("nlon_out", ctypes.c_int32),
+        ("ck", ctypes.c_int32),
+        ("cv", ctypes.c_int32),
+        ("nlon_in", ctypes.c_int32),
+        ("pscale", ctypes.c_int32),
+        ("lon_lo_kx", ctypes.c_int32),
+        ("lat_halo_start", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+    ]
+
+
 # every symbol include/s2attn.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "s2attn_last_error": (ctypes.c_char_p, []),
@@ -66,6 +83,9 @@ SYMBOLS = {
     "s2attn_backward_dkdv": (_int, [_vp] * 8 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_permute_to_nhwc": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "s2attn_permute_to_nchw": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
+    "s2attn_ring_forward_step": (_int, [_vp] * 10 + [ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
 }
 
 _lib = None

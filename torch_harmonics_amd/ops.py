@@ -405,3 +405,193 @@ def _make_autocast_impl_saved(device_type: str):
 for _device_type in ("cuda", "cpu"):
     _make_autocast_impl(_device_type)
     _make_autocast_impl_saved(_device_type)
+
+
+# ---------------------------------------------------------------------------------------------------------------------
+# Ring-step operators of the gather direction (attention_interface.cpp:137-156, fake kernels attention_optimized.py:82-160):
+# one longitude chunk of K/V per call, the softmax state lives in caller-owned fp32 buffers that the operators update in
+# place.  Same argument lists as the reference's; the three trailing row-split hints are accepted and not needed.
+# ---------------------------------------------------------------------------------------------------------------------
+def split_csr_rows(row_idx: torch.Tensor, row_off: torch.Tensor, nlat_out: int):
+    """(n_long_rows, max_row_len, mid_row_len) of a CSR whose rows are listed in row_idx by decreasing length: the long rows
+    are the leading ones of at least max(1024, 0.1 * longest) entries; max_row_len is the longest row if there is a long
+    one, else 0; mid_row_len the length of the first short row, else 0 (attention_cuda_utils.cu:286-384).  Host scalar
+    computation on either device's tensors; never traced."""
+    idx = row_idx.detach().to("cpu", torch.int64)
+    off = row_off.detach().to("cpu", torch.int64)
+    if nlat_out == 0:
+        return 0, 0, 0
+    lens = (off[1:] - off[:-1])[idx[:nlat_out]]
+    max_rlen = int(lens[0])
+    min_long = max(1024, int(float(torch.tensor(max_rlen, dtype=torch.float32) * torch.tensor(0.1, dtype=torch.float32))))
+    short = (lens < min_long).nonzero()
+    n_long = int(short[0]) if short.numel() else int(nlat_out)
+    return n_long, (max_rlen if n_long else 0), (int(lens[n_long]) if n_long < nlat_out else 0)
+
+
+def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out) -> _lib.RingShapeStruct:
+    B, nlat_halo, nlon_kx, ck = kx.shape
+    return _lib.RingShapeStruct(B, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, vx.shape[3], nlon_in, pscale, lon_lo_kx, lat_halo_start, _DTYPE_CODE[qy.dtype])
+
+
+def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out):
+    """state: (name, tensor, trailing channel count or None) fp32 buffers shaped like the local output grid."""
+    for name, t in (("kx", kx), ("vx", vx), ("qy", qy)) + ((("dy", dy),) if dy is not None else ()):
+        if t.dim() != 4 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous 4-dimensional (batch*heads, nlat, nlon, channels) tensor")
+        _require_gpu(t, name, kx.device)
+        if t.dtype != qy.dtype or t.dtype not in _DTYPE_CODE:
+            raise RuntimeError(f"{name} has dtype {t.dtype}; k, v, q and dy must share one of fp32, bf16, fp16")
+    if kx.shape[:3] != vx.shape[:3] or kx.shape[0] != qy.shape[0] or kx.shape[3] != qy.shape[3]:
+        raise RuntimeError("kx and vx must share (batch, nlat_halo, nlon_kx); qy must share batch and channels with kx")
+    if tuple(qy.shape[1:3]) != (nlat_out, nlon_out):
+        raise RuntimeError(f"qy must be (batch, nlat_out={nlat_out}, nlon_out={nlon_out}, channels)")
+    if dy is not None and (dy.shape[:3] != qy.shape[:3] or dy.shape[3] != vx.shape[3]):
+        raise RuntimeError("dy must be (batch, nlat_out, nlon_out, v channels)")
+    for name, t, c in state:
+        want = (qy.shape[0], nlat_out, nlon_out) + (() if c is None else (c,))
+        if tuple(t.shape) != want or t.dtype != torch.float32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous fp32 tensor of shape {want}")
+        _require_gpu(t, name, kx.device)
+    for name, t, dt in (("quad_weights", quad_weights, torch.float32), ("col_idx", col_idx, torch.int64), ("row_off", row_off, torch.int64), ("row_idx", row_idx, torch.int32)):
+        if t.dtype != dt or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous {dt} tensor")
+        _require_gpu(t, name, kx.device)
+    if row_off.numel() != nlat_out + 1 or row_idx.numel() != nlat_out:
+        raise RuntimeError("row_off must have nlat_out + 1 entries and row_idx nlat_out")
+
+
+@torch.library.custom_op("s2attn::forward_ring_step", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
+def forward_ring_step(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    y_acc: torch.Tensor,
+    alpha_sum_buf: torch.Tensor,
+    qdotk_max_buf: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    row_idx: torch.Tensor,
+    nlon_in: int,
+    pscale: int,
+    lon_lo_kx: int,
+    lat_halo_start: int,
+    nlat_out: int,
+    nlon_out: int,
+    n_long_rows: int,
+    max_row_len: int,
+    mid_row_len: int,
+) -> None:
+    state = (("y_acc", y_acc, vx.shape[3]), ("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None))
+    _ring_validate(kx, vx, qy, None, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out)
+    if qy.numel() == 0 or kx.numel() == 0:
+        return
+    shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_ring_forward_step(
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+            quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+        )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_forward_step")
+
+
+@forward_ring_step.register_fake
+def _(kx, vx, qy, y_acc, alpha_sum_buf, qdotk_max_buf, quad_weights, col_idx, row_off, row_idx, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out, n_long_rows, max_row_len, mid_row_len):
+    return None
+
+
+@torch.library.custom_op(
+    "s2attn::backward_ring_step_pass1", mutates_args=("alpha_sum_buf", "qdotk_max_buf", "integral_buf", "alpha_k_buf", "alpha_kvw_buf")
+)
+def backward_ring_step_pass1(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    dy: torch.Tensor,
+    alpha_sum_buf: torch.Tensor,
+    qdotk_max_buf: torch.Tensor,
+    integral_buf: torch.Tensor,
+    alpha_k_buf: torch.Tensor,
+    alpha_kvw_buf: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    row_idx: torch.Tensor,
+    nlon_in: int,
+    pscale: int,
+    lon_lo_kx: int,
+    lat_halo_start: int,
+    nlat_out: int,
+    nlon_out: int,
+    n_long_rows: int,
+    max_row_len: int,
+    mid_row_len: int,
+) -> None:
+    ck = kx.shape[3]
+    state = (("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None), ("integral_buf", integral_buf, None),
+             ("alpha_k_buf", alpha_k_buf, ck), ("alpha_kvw_buf", alpha_kvw_buf, ck))  # fmt: skip
+    _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out)
+    if qy.numel() == 0 or kx.numel() == 0:
+        return
+    shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_ring_backward_pass1(
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+            integral_buf.data_ptr(), alpha_k_buf.data_ptr(), alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(),
+            row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+        )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_backward_pass1")
+
+
+@backward_ring_step_pass1.register_fake
+def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_buf, alpha_k_buf, alpha_kvw_buf, quad_weights, col_idx, row_off, row_idx, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out, n_long_rows, max_row_len, mid_row_len):
+    return None
+
+
+@torch.library.custom_op("s2attn::backward_ring_step_pass2", mutates_args=("dkx", "dvx"))
+def backward_ring_step_pass2(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    dy: torch.Tensor,
+    alpha_sum_buf: torch.Tensor,
+    qdotk_max_buf: torch.Tensor,
+    integral_norm_buf: torch.Tensor,
+    dkx: torch.Tensor,
+    dvx: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    row_idx: torch.Tensor,
+    nlon_in: int,
+    pscale: int,
+    lon_lo_kx: int,
+    lat_halo_start: int,
+    nlat_out: int,
+    nlon_out: int,
+    n_long_rows: int,
+    max_row_len: int,
+    mid_row_len: int,
+) -> None:
+    state = (("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None), ("integral_norm_buf", integral_norm_buf, None))
+    _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out)
+    for name, t, like in (("dkx", dkx, kx), ("dvx", dvx, vx)):
+        if t.shape != like.shape or t.dtype != torch.float32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous fp32 tensor shaped like its input, {tuple(like.shape)}")
+        _require_gpu(t, name, kx.device)
+    if qy.numel() == 0 or kx.numel() == 0:
+        return
+    shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_ring_backward_pass2(
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+            integral_norm_buf.data_ptr(), dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(),
+            row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+        )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_backward_pass2")
+
+
+@backward_ring_step_pass2.register_fake
+def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_norm_buf, dkx, dvx, quad_weights, col_idx, row_off, row_idx, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out, n_long_rows, max_row_len, mid_row_len):
+    return None
