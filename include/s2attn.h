@@ -231,6 +231,42 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
                                const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
                                const int32_t *row_idx, const s2attn_ring_shape *shape, void *stream);
 
+/*
+ * The same three steps for the up-sampling (scatter) direction, nlon_out a multiple of nlon_in.  Replace
+ * attention_kernels::forward_ring_step_upsample, backward_ring_step_upsample_pass1 / _pass2
+ * (attention_interface.cpp:158-189; CUDA: attention_cuda_fwd_ring_upsample.cu:108-300,
+ * attention_cuda_bwd_ring_upsample.cu:88-240).  psi is keyed by the chunk's LOCAL input latitude: row_off has
+ * nlat_halo + 1 entries (empty rows for pole padding), col_idx = ho_local * nlon_out_global + wo_shifted with
+ * wo_shifted = (wo - first local output longitude) mod nlon_out_global.  The forward step runs three phases (scatter the
+ * chunk's maxima into max_scratch, rescale the state, scatter the sums with fp32 atomics); max_scratch is caller-owned
+ * scratch of batch * nlat_out * nlon_out floats.  Pass 1 needs the forward's FINAL qdotk_max and adds into integral,
+ * alpha_k, alpha_kvw atomically; pass 2 WRITES the chunk's dk and dv (every element, no atomics).
+ */
+typedef struct s2attn_ring_up_shape {
+    int32_t batch, nlat_halo, nlon_kx, nlat_out, nlon_out; /* as s2attn_ring_shape; nlon_out is the LOCAL output width */
+    int32_t ck, cv;
+    int32_t nlon_out_global; /* global output longitudes */
+    int32_t pscale_out;      /* global nlon_out / global nlon_in */
+    int32_t lon_lo_kx;       /* first global input longitude of the chunk */
+    int32_t lat_halo_start;  /* global input latitude of the chunk's row 0 (quadrature weight index; may be negative when
+                                the halo is padded past the pole: such rows must be empty in row_off) */
+    int32_t dtype;
+} s2attn_ring_up_shape;
+
+int s2attn_ring_forward_step_upsample(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                                      float *max_scratch, const float *quad_weights, const int64_t *col_idx,
+                                      const int64_t *row_off, const s2attn_ring_up_shape *shape, void *stream);
+
+int s2attn_ring_backward_pass1_upsample(const void *k, const void *v, const void *q, const void *dy, const float *qdotk_max,
+                                        float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                                        const int64_t *col_idx, const int64_t *row_off, const s2attn_ring_up_shape *shape,
+                                        void *stream);
+
+int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                        const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                        const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
+                                        const s2attn_ring_up_shape *shape, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -61,3 +61,59 @@ def fresh_state(batch, nlat, nlon, ck, cv, dtype, device="cpu"):
         y_acc=z(batch, nlat, nlon, cv), alpha_sum=z(batch, nlat, nlon), qdotk_max=torch.full((batch, nlat, nlon), float("-inf"), dtype=dtype, device=device),
         integral=z(batch, nlat, nlon), alpha_k=z(batch, nlat, nlon, ck), alpha_kvw=z(batch, nlat, nlon, ck),
     )  # fmt: skip
+
+
+# up-sampling direction: (in_shape, out_shape, grid_in, grid_out, theta_cutoff, local output window, chunk boundaries, halo pad)
+RING_UP_CASES = [
+    ((6, 8), (6, 16), "equiangular", "equiangular", 0.9, (0, 6, 0, 16), [0, 8], 0),  # one chunk, whole grid
+    ((6, 8), (11, 16), "equiangular", "equiangular", 0.8, (2, 6, 5, 7), [0, 3, 8], 0),  # ratio 2, unequal chunks
+    ((5, 6), (9, 18), "legendre-gauss", "equiangular", 0.9, (0, 9, 12, 6), [0, 1, 4, 6], 1),  # ratio 3, halo padded past the poles
+    ((6, 12), (12, 24), "equiangular", "legendre-gauss", 7.0, (3, 5, 20, 4), [0, 6, 12], 0),  # every point sees every point
+]
+
+
+def local_problem_upsample(case, batch=2, ck=5, cv=3, seed=0):
+    """Global tensors plus one rank's local view in the scatter direction (psi keyed by input latitude): rows = the halo's input
+    latitudes (pad rows past the poles are empty), entries restricted to the local output latitudes and re-based, output
+    longitude shifted by the window's first longitude (torch_harmonics/distributed/distributed_attention.py, _build_local_psi_upsample)."""
+    ins, outs, gi, go, tc, (lat_lo, nlat_loc, lon_lo, nlon_loc), bounds, pad = case
+    (Hi, Wi), (Ho, Wo) = ins, outs
+    col, roff = ogeo.neighborhood_csr(outs, ins, go, gi, tc)  # grids swapped: rows index the input grid
+    quad = ogeo.attention_quad_weights(Hi, Wi, gi)
+    pscale_out = Wo // Wi
+    gen = torch.Generator().manual_seed(2000 + seed)
+    k = torch.randn(batch, Hi, Wi, ck, generator=gen)
+    v = torch.randn(batch, Hi, Wi, cv, generator=gen)
+    q = torch.randn(batch, Ho, Wo, ck, generator=gen) / ck**0.5
+    dy = torch.randn(batch, Ho, Wo, cv, generator=gen)
+    # input latitudes that reach the local output rows, padded by `pad` rows on both sides (possibly past the poles)
+    ho_all = col // Wo
+    row_of = torch.repeat_interleave(torch.arange(Hi), roff[1:] - roff[:-1])
+    keep = (ho_all >= lat_lo) & (ho_all < lat_lo + nlat_loc)
+    used = row_of[keep]
+    h0, h1 = (int(used.min()) - pad, int(used.max()) + 1 + pad) if used.numel() else (0, 1)
+    rows, offs = [], [0]
+    for hg in range(h0, h1):
+        if 0 <= hg < Hi:
+            e = col[int(roff[hg]) : int(roff[hg + 1])]
+            ho = e // Wo
+            sel = (ho >= lat_lo) & (ho < lat_lo + nlat_loc)
+            e, ho = e[sel], ho[sel]
+            rows.append((ho - lat_lo) * Wo + (e - ho * Wo - lon_lo) % Wo)
+        offs.append(offs[-1] + (rows[-1].numel() if 0 <= hg < Hi else 0))
+    col_l = torch.cat(rows) if rows else torch.zeros(0, dtype=torch.int64)
+    roff_l = torch.tensor(offs, dtype=torch.int64)
+
+    def halo_block(t, lo, hi):  # rows h0..h1 of the chunk's longitudes, zeros where the halo leaves the grid
+        out = torch.zeros(t.shape[0], h1 - h0, hi - lo, t.shape[3], dtype=t.dtype)
+        a, b = max(h0, 0), min(h1, Hi)
+        out[:, a - h0 : b - h0] = t[:, a:b, lo:hi]
+        return out
+
+    return dict(
+        ins=ins, outs=outs, pscale_out=pscale_out, quad=quad, col=col, roff=roff, k=k, v=v, q=q, dy=dy, col_l=col_l, roff_l=roff_l,
+        lat_lo=lat_lo, nlat_loc=nlat_loc, lon_lo=lon_lo, nlon_loc=nlon_loc, halo=(h0, h1), halo_block=halo_block,
+        chunks=[(bounds[i], bounds[i + 1]) for i in range(len(bounds) - 1)],
+        q_l=q[:, lat_lo : lat_lo + nlat_loc, lon_lo : lon_lo + nlon_loc].contiguous(),
+        dy_l=dy[:, lat_lo : lat_lo + nlat_loc, lon_lo : lon_lo + nlon_loc].contiguous(),
+    )  # fmt: skip

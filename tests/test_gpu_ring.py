@@ -127,3 +127,100 @@ def test_ring_ops_pass_opcheck_and_leave_state_alone_without_neighbors():
     assert float(st3["alpha_sum"].abs().max()) == 0.0 and bool(torch.isinf(st3["qdotk_max"]).all()) and float(st3["y_acc"].abs().max()) == 0.0
     with pytest.raises(RuntimeError):  # chunk outside the input grid
         ops.forward_ring_step(kc, vc, qd, st3["y_acc"], st3["alpha_sum"], st3["qdotk_max"], quad, col_l, roff_l, row_idx, Wi, p["pscale"], Wi - 1, 0, p["nlat_loc"], p["nlon_loc"], *split)
+
+
+from tests.ring_util import RING_UP_CASES, local_problem_upsample  # noqa: E402
+
+
+@pytest.mark.parametrize("case", RING_UP_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
+def test_upsample_ring_steps_against_oracle_and_dense_attention(case, dtype):
+    from torch_harmonics_amd import ops
+
+    print(f"case {case} {dtype}", flush=True)
+    ck, cv = (70, 33) if case is RING_UP_CASES[1] else (5, 3)
+    p = local_problem_upsample(case, ck=ck, cv=cv)
+    for name in ("k", "v", "q", "dy", "q_l", "dy_l"):
+        p[name] = p[name].to(dtype).float()
+    B, (Hi, Wi), Wo = p["k"].shape[0], p["ins"], p["outs"][1]
+    tol = TOL if dtype == torch.float32 else dict(rtol=2e-2, atol=2e-2)
+    stol = dict(rtol=1e-5, atol=1e-5)
+    quad, col_l, roff_l = p["quad"].to(DEV), p["col_l"].to(DEV), p["roff_l"].to(DEV)
+    tail = lambda c: (Wi, Wo, p["pscale_out"], p["chunks"][c][0], p["halo"][0], p["nlat_loc"], p["nlon_loc"])  # noqa: E731
+    ogeo = lambda c: (p["quad"], p["col_l"], p["roff_l"], Wo, p["pscale_out"], p["chunks"][c][0], p["halo"][0])  # noqa: E731
+    blk = lambda t, c: p["halo_block"](t, *p["chunks"][c])  # noqa: E731
+    qd, gd = p["q_l"].to(DEV, dtype), p["dy_l"].to(DEV, dtype)
+    q64, g64 = p["q_l"].double(), p["dy_l"].double()
+    nchunk = len(p["chunks"])
+    steps = [(1 + i) % nchunk for i in range(nchunk)]
+
+    st = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    ref = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float64)
+    for c in steps:
+        kc, vc = blk(p["k"], c), blk(p["v"], c)
+        ops.forward_ring_step_upsample(kc.to(DEV, dtype), vc.to(DEV, dtype), qd, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col_l, roff_l, *tail(c))
+        ring.forward_step_upsample(kc.double(), vc.double(), q64, ref["y_acc"], ref["alpha_sum"], ref["qdotk_max"], *ogeo(c))
+        torch.cuda.synchronize()
+        seen = torch.isfinite(ref["qdotk_max"])
+        assert torch.equal(torch.isfinite(st["qdotk_max"]).cpu(), seen)
+        assert_close(f"qdotk_max after chunk {c}", st["qdotk_max"].cpu()[seen], ref["qdotk_max"][seen], **stol)
+        assert_close(f"alpha_sum after chunk {c}", st["alpha_sum"].cpu(), ref["alpha_sum"], **stol)
+        assert_close(f"y_acc after chunk {c}", st["y_acc"].cpu(), ref["y_acc"], **stol)
+
+    k, v, q = [t.double().requires_grad_(True) for t in (p["k"], p["v"], p["q"])]
+    y = oracle.dense_attention_f64(k, v, q, p["quad"], p["col"], p["roff"], 1)
+    la, na, lo, no = p["lat_lo"], p["nlat_loc"], p["lon_lo"], p["nlon_loc"]
+    win = y[:, la : la + na, lo : lo + no]
+    (win * g64).sum().backward()
+    assert_close("y", (st["y_acc"] / st["alpha_sum"][..., None]).cpu(), win.detach(), **tol)
+
+    bw = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    rbw = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float64)
+    for c in steps:
+        kc, vc = blk(p["k"], c), blk(p["v"], c)
+        ops.backward_ring_step_upsample_pass1(kc.to(DEV, dtype), vc.to(DEV, dtype), qd, gd, st["qdotk_max"], bw["integral"], bw["alpha_k"], bw["alpha_kvw"], quad, col_l, roff_l, *tail(c))
+        ring.backward_pass1_upsample(kc.double(), vc.double(), q64, g64, ref["qdotk_max"], rbw["integral"], rbw["alpha_k"], rbw["alpha_kvw"], *ogeo(c))
+        torch.cuda.synchronize()
+        assert_close(f"integral after chunk {c}", bw["integral"].cpu(), rbw["integral"], **stol)
+        assert_close(f"alpha_k after chunk {c}", bw["alpha_k"].cpu(), rbw["alpha_k"], **stol)
+        assert_close(f"alpha_kvw after chunk {c}", bw["alpha_kvw"].cpu(), rbw["alpha_kvw"], **stol)
+    S = st["alpha_sum"][..., None]
+    dq = (S * bw["alpha_kvw"] - bw["integral"][..., None] * bw["alpha_k"]) / S**2
+    assert_close("dq", dq.cpu(), q.grad[:, la : la + na, lo : lo + no], **tol)
+
+    integral_norm = (bw["integral"] / st["alpha_sum"]).contiguous()
+    dk, dv = torch.zeros_like(p["k"]), torch.zeros_like(p["v"])
+    h0, h1 = p["halo"]
+    a, b = max(h0, 0), min(h1, Hi)
+    for c in steps:
+        kc, vc = blk(p["k"], c), blk(p["v"], c)
+        dkc = torch.full(kc.shape, float("nan"), device=DEV)  # pass 2 writes every element
+        dvc = torch.full(vc.shape, float("nan"), device=DEV)
+        ops.backward_ring_step_upsample_pass2(kc.to(DEV, dtype), vc.to(DEV, dtype), qd, gd, st["alpha_sum"], st["qdotk_max"], integral_norm, dkc, dvc, quad, col_l, roff_l, *tail(c))
+        clo, chi = p["chunks"][c]
+        assert bool(torch.isfinite(dkc).all()) and bool(torch.isfinite(dvc).all())
+        dk[:, a:b, clo:chi] += dkc.cpu()[:, a - h0 : b - h0]
+        dv[:, a:b, clo:chi] += dvc.cpu()[:, a - h0 : b - h0]
+    assert_close("dk", dk, k.grad, **tol)
+    assert_close("dv", dv, v.grad, **tol)
+
+
+def test_upsample_ring_ops_pass_opcheck():
+    from torch_harmonics_amd import ops
+
+    p = local_problem_upsample(RING_UP_CASES[2])
+    B, ck, cv, Wi, Wo = p["k"].shape[0], p["k"].shape[3], p["v"].shape[3], p["ins"][1], p["outs"][1]
+    quad, col_l, roff_l = p["quad"].to(DEV), p["col_l"].to(DEV), p["roff_l"].to(DEV)
+    qd, gd = p["q_l"].to(DEV), p["dy_l"].to(DEV)
+    kc, vc = p["halo_block"](p["k"], *p["chunks"][1]).to(DEV), p["halo_block"](p["v"], *p["chunks"][1]).to(DEV)
+    tail = (Wi, Wo, p["pscale_out"], p["chunks"][1][0], p["halo"][0], p["nlat_loc"], p["nlon_loc"])
+    st = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
+    ops.forward_ring_step_upsample(kc, vc, qd, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col_l, roff_l, *tail)
+    mx = st["qdotk_max"].clamp_min(-1e30)
+    # the scatter steps add with fp32 atomics in hardware order: opcheck's repeat-and-compare needs a tolerance there
+    torch.library.opcheck(ops.forward_ring_step_upsample, (kc, vc, qd, st["y_acc"], st["alpha_sum"], mx.clone(), quad, col_l, roff_l, *tail), rtol=1e-5, atol=1e-5)
+    torch.library.opcheck(ops.backward_ring_step_upsample_pass1, (kc, vc, qd, gd, mx, st["integral"], st["alpha_k"], st["alpha_kvw"], quad, col_l, roff_l, *tail), rtol=1e-5, atol=1e-5)
+    norm = torch.zeros_like(mx)
+    torch.library.opcheck(
+        ops.backward_ring_step_upsample_pass2, (kc, vc, qd, gd, st["alpha_sum"].clamp_min(1e-30), mx, norm, torch.zeros_like(kc), torch.zeros_like(vc), quad, col_l, roff_l, *tail)
+    )

@@ -107,3 +107,44 @@ def test_split_csr_rows(name, lengths, expected):
     row_idx, row_off = _csr_from_lengths(lengths)
     assert ring.split_csr_rows(row_idx, row_off, len(lengths)) == expected
     assert tuple(ops.split_csr_rows(row_idx, row_off, len(lengths))) == expected
+
+
+from tests.ring_util import RING_UP_CASES, local_problem_upsample  # noqa: E402
+
+
+@pytest.mark.parametrize("case", RING_UP_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
+@pytest.mark.parametrize("order", ["natural", "rotated"])
+def test_upsample_chunks_fold_to_dense_attention(case, order):
+    p = local_problem_upsample(case)
+    B, ck, cv = p["k"].shape[0], p["k"].shape[3], p["v"].shape[3]
+    Hi, Wo = p["ins"][0], p["outs"][1]
+    nchunk = len(p["chunks"])
+    steps = list(range(nchunk)) if order == "natural" else [(1 + i) % nchunk for i in range(nchunk)]
+    geo = lambda c: (p["quad"], p["col_l"], p["roff_l"], Wo, p["pscale_out"], p["chunks"][c][0], p["halo"][0])  # noqa: E731
+    blk = lambda t, c: p["halo_block"](t, *p["chunks"][c]).double()  # noqa: E731
+    q_l, g_l = p["q_l"].double(), p["dy_l"].double()
+    st = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, D)
+    for c in steps:
+        ring.forward_step_upsample(blk(p["k"], c), blk(p["v"], c), q_l, st["y_acc"], st["alpha_sum"], st["qdotk_max"], *geo(c))
+    y_ref, dk_ref, dv_ref, dq_ref = _dense_reference(p)
+    torch.testing.assert_close(st["y_acc"] / st["alpha_sum"][..., None], y_ref, rtol=1e-12, atol=1e-12)
+
+    bw = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, D)
+    for c in steps:
+        ring.backward_pass1_upsample(blk(p["k"], c), blk(p["v"], c), q_l, g_l, st["qdotk_max"], bw["integral"], bw["alpha_k"], bw["alpha_kvw"], *geo(c))
+    S = st["alpha_sum"][..., None]
+    dq = (S * bw["alpha_kvw"] - bw["integral"][..., None] * bw["alpha_k"]) / S**2
+    torch.testing.assert_close(dq, dq_ref, rtol=1e-11, atol=1e-12)
+    integral_norm = bw["integral"] / st["alpha_sum"]
+    dk, dv = torch.zeros_like(p["k"], dtype=D), torch.zeros_like(p["v"], dtype=D)
+    h0, h1 = p["halo"]
+    a, b = max(h0, 0), min(h1, Hi)
+    for c in steps:
+        kc, vc = blk(p["k"], c), blk(p["v"], c)
+        dkc, dvc = torch.full_like(kc, float("nan")), torch.full_like(vc, float("nan"))  # pass 2 writes every element
+        ring.backward_pass2_upsample(kc, vc, q_l, g_l, st["alpha_sum"], st["qdotk_max"], integral_norm, dkc, dvc, *geo(c))
+        lo, hi = p["chunks"][c]
+        dk[:, a:b, lo:hi] += dkc[:, a - h0 : b - h0]
+        dv[:, a:b, lo:hi] += dvc[:, a - h0 : b - h0]
+    torch.testing.assert_close(dk, dk_ref, rtol=1e-11, atol=1e-12)
+    torch.testing.assert_close(dv, dv_ref, rtol=1e-11, atol=1e-12)

@@ -67,6 +67,13 @@ class RingShapeStruct(ctypes.Structure):
     ]
 
 
+class RingUpShapeStruct(ctypes.Structure):
+    _fields_ = [
+        (n, ctypes.c_int32)
+        for n in ("batch", "nlat_halo", "nlon_kx", "nlat_out", "nlon_out", "ck", "cv", "nlon_out_global", "pscale_out", "lon_lo_kx", "lat_halo_start", "dtype")
+    ]
+
+
 # every symbol include/s2attn.h declares: name -> (restype, argtypes)
 SYMBOLS = {
     "s2attn_last_error": (ctypes.c_char_p, []),
@@ -86,6 +93,9 @@ SYMBOLS = {
     "s2attn_ring_forward_step": (_int, [_vp] * 10 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_forward_step_upsample": (_int, [_vp] * 10 + [ctypes.POINTER(RingUpShapeStruct), _vp]),
+    "s2attn_ring_backward_pass1_upsample": (_int, [_vp] * 11 + [ctypes.POINTER(RingUpShapeStruct), _vp]),
+    "s2attn_ring_backward_pass2_upsample": (_int, [_vp] * 12 + [ctypes.POINTER(RingUpShapeStruct), _vp]),
 }
 
 _lib = None

@@ -235,6 +235,213 @@ template <typename T> __global__ __launch_bounds__(256) void pass2_kernel(const 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------------
+// Up-sampling (scatter) direction.  psi is keyed by the chunk's LOCAL input latitude hi_local (row_off has nlat_halo + 1
+// entries, empty rows for pole padding), col_idx = ho_local * nlon_out_global + wo_shifted with
+// wo_shifted = (wo - first local output longitude) mod nlon_out_global; input cell (hi_local, wi_global) is seen by the
+// local output cell (ho_local, w) with w = (wo_shifted + pscale_out * wi_global) mod nlon_out_global iff w < nlon_out.
+// The cell that normalises the softmax is not the row key here, so a step runs in three phases like the reference's
+// (attention_cuda_fwd_ring_upsample.cu:40-66): scatter the chunk's maxima, rescale the state, scatter the sums.
+// ---------------------------------------------------------------------------------------------------------------------
+struct UpArgs {
+    const void *k, *v, *q, *dy;
+    float *y_acc, *alpha_sum, *qdotk_max, *max_curr, *integral, *alpha_k, *alpha_kvw;
+    const float *integral_norm;
+    float *dk, *dv;
+    const float *quad_w;
+    const int64_t *col_idx, *row_off;
+    int B, nlat_halo, nlon_kx, Ho, Wo, ck, cv, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start;
+};
+
+__device__ inline void atomic_max_float(float *addr, float val)
+{
+    int *ai = reinterpret_cast<int *>(addr);
+    int old = *ai;
+    while (val > __int_as_float(old)) {
+        const int assumed = old;
+        old = atomicCAS(ai, assumed, __float_as_int(val));
+        if (old == assumed) break;
+    }
+}
+
+// chunk cell of this wavefront; false past the end or when its psi row is empty
+__device__ inline bool up_locate(const UpArgs &a, int &b, int &hi, int &wi_local, int &lane, int64_t &z0, int64_t &z1)
+{
+    lane = threadIdx.x & 63;
+    const long pid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (pid >= (long)a.B * a.nlat_halo * a.nlon_kx) return false;
+    wi_local = (int)(pid % a.nlon_kx);
+    hi = (int)((pid / a.nlon_kx) % a.nlat_halo);
+    b = (int)(pid / ((long)a.nlon_kx * a.nlat_halo));
+    z0 = a.row_off[hi], z1 = a.row_off[hi + 1];
+    return z1 > z0;
+}
+
+// local output cell index of entry `col` for global input longitude wi_global, or -1 when another rank owns it
+__device__ inline long up_cell(const UpArgs &a, int64_t col, int wi_global)
+{
+    const int ho = (int)(col / a.nlon_out_global);
+    int w = (int)(col - (int64_t)ho * a.nlon_out_global) + a.pscale_out * wi_global;
+    if (w >= a.nlon_out_global) w -= a.nlon_out_global;
+    return w < a.Wo ? (long)ho * a.Wo + w : -1;
+}
+
+template <typename T> __device__ inline float up_dot(const float (&x)[NCI], const T *row, int n, int lane)
+{
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NCI; i++) {
+        const int c = lane + 64 * i;
+        if (c < n) s = fmaf(x[i], ld(row + c), s);
+    }
+    return wave_sum(s);
+}
+
+template <typename T> __device__ inline void up_load(float (&x)[NCI], const T *row, int n, int lane)
+{
+#pragma unroll
+    for (int i = 0; i < NCI; i++) {
+        const int c = lane + 64 * i;
+        x[i] = c < n ? ld(row + c) : 0.f;
+    }
+}
+
+// phase 1: max_curr (a copy of qdotk_max) takes in the chunk's scores.  attention_cuda_fwd_ring_upsample.cu:108-151.
+template <typename T> __global__ __launch_bounds__(256) void up_max_kernel(const UpArgs a)
+{
+    int b, hi, wl, lane;
+    int64_t z0, z1;
+    if (!up_locate(a, b, hi, wl, lane, z0, z1)) return;
+    float kr[NCI];
+    up_load(kr, static_cast<const T *>(a.k) + (((long)b * a.nlat_halo + hi) * a.nlon_kx + wl) * a.ck, a.ck, lane);
+    const T *q = static_cast<const T *>(a.q) + (long)b * a.Ho * a.Wo * a.ck;
+    for (int64_t z = z0; z < z1; z++) {
+        const long cell = up_cell(a, a.col_idx[z], a.lon_lo_kx + wl);
+        if (cell < 0) continue;
+        const float s = up_dot(kr, q + cell * a.ck, a.ck, lane);
+        if (lane == 0) atomic_max_float(a.max_curr + (long)b * a.Ho * a.Wo + cell, s);
+    }
+}
+
+// phase 2: rescale the state of every local output cell whose maximum moved.  :153-181.
+__global__ __launch_bounds__(256) void up_rescale_kernel(const UpArgs a)
+{
+    const int lane = threadIdx.x & 63;
+    const long cell = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (cell >= (long)a.B * a.Ho * a.Wo) return;
+    const float m_old = a.qdotk_max[cell], m_new = a.max_curr[cell];
+    if (m_old == m_new) return; // untouched, including -inf == -inf
+    const float corr = __expf(m_old - m_new);
+    for (int c = lane; c < a.cv; c += 64) a.y_acc[cell * a.cv + c] *= corr;
+    if (lane == 0) {
+        a.alpha_sum[cell] *= corr;
+        a.qdotk_max[cell] = m_new;
+    }
+}
+
+// phase 3: scatter alpha = exp(q.k - max) w into alpha_sum and alpha v into y_acc.  :183-243.
+template <typename T> __global__ __launch_bounds__(256) void up_acc_kernel(const UpArgs a)
+{
+    int b, hi, wl, lane;
+    int64_t z0, z1;
+    if (!up_locate(a, b, hi, wl, lane, z0, z1)) return;
+    float kr[NCI], vr[NCI];
+    const long pt = ((long)b * a.nlat_halo + hi) * a.nlon_kx + wl;
+    up_load(kr, static_cast<const T *>(a.k) + pt * a.ck, a.ck, lane);
+    up_load(vr, static_cast<const T *>(a.v) + pt * a.cv, a.cv, lane);
+    const long boff = (long)b * a.Ho * a.Wo;
+    const T *q = static_cast<const T *>(a.q) + boff * a.ck;
+    const float w = a.quad_w[a.lat_halo_start + hi];
+    for (int64_t z = z0; z < z1; z++) {
+        const long cell = up_cell(a, a.col_idx[z], a.lon_lo_kx + wl);
+        if (cell < 0) continue;
+        const float s = up_dot(kr, q + cell * a.ck, a.ck, lane);
+        const float alpha = __expf(s - a.qdotk_max[boff + cell]) * w;
+        if (lane == 0) atomicAdd(a.alpha_sum + boff + cell, alpha);
+#pragma unroll
+        for (int i = 0; i < NCI; i++) {
+            const int c = lane + 64 * i;
+            if (c < a.cv) atomicAdd(a.y_acc + (boff + cell) * a.cv + c, alpha * vr[i]);
+        }
+    }
+}
+
+// backward pass 1: with the forward's final maximum, scatter integral, alpha_k, alpha_kvw.  attention_cuda_bwd_ring_upsample.cu:88-160.
+template <typename T> __global__ __launch_bounds__(256) void up_pass1_kernel(const UpArgs a)
+{
+    int b, hi, wl, lane;
+    int64_t z0, z1;
+    if (!up_locate(a, b, hi, wl, lane, z0, z1)) return;
+    float kr[NCI], vr[NCI];
+    const long pt = ((long)b * a.nlat_halo + hi) * a.nlon_kx + wl;
+    up_load(kr, static_cast<const T *>(a.k) + pt * a.ck, a.ck, lane);
+    up_load(vr, static_cast<const T *>(a.v) + pt * a.cv, a.cv, lane);
+    const long boff = (long)b * a.Ho * a.Wo;
+    const T *q = static_cast<const T *>(a.q) + boff * a.ck;
+    const T *g = static_cast<const T *>(a.dy) + boff * a.cv;
+    const float w = a.quad_w[a.lat_halo_start + hi];
+    for (int64_t z = z0; z < z1; z++) {
+        const long cell = up_cell(a, a.col_idx[z], a.lon_lo_kx + wl);
+        if (cell < 0) continue;
+        const float s = up_dot(kr, q + cell * a.ck, a.ck, lane);
+        const float gv = up_dot(vr, g + cell * a.cv, a.cv, lane);
+        const float alpha = __expf(s - a.qdotk_max[boff + cell]) * w;
+        const float ag = alpha * gv;
+        if (lane == 0) atomicAdd(a.integral + boff + cell, ag);
+#pragma unroll
+        for (int i = 0; i < NCI; i++) {
+            const int c = lane + 64 * i;
+            if (c < a.ck) {
+                atomicAdd(a.alpha_k + (boff + cell) * a.ck + c, alpha * kr[i]);
+                atomicAdd(a.alpha_kvw + (boff + cell) * a.ck + c, ag * kr[i]);
+            }
+        }
+    }
+}
+
+// backward pass 2: dk, dv of every chunk cell, summed over its own row and WRITTEN (no atomics).  :162-240.
+template <typename T> __global__ __launch_bounds__(256) void up_pass2_kernel(const UpArgs a)
+{
+    int b, hi, wl, lane;
+    int64_t z0, z1;
+    const bool any = up_locate(a, b, hi, wl, lane, z0, z1);
+    const long pid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    if (pid >= (long)a.B * a.nlat_halo * a.nlon_kx) return;
+    const long pt = pid; // = ((b * nlat_halo + hi) * nlon_kx + wl)
+    float kr[NCI], vr[NCI], dk[NCI], dv[NCI];
+#pragma unroll
+    for (int i = 0; i < NCI; i++) dk[i] = dv[i] = 0.f;
+    if (any) {
+        up_load(kr, static_cast<const T *>(a.k) + pt * a.ck, a.ck, lane);
+        up_load(vr, static_cast<const T *>(a.v) + pt * a.cv, a.cv, lane);
+        const long boff = (long)b * a.Ho * a.Wo;
+        const T *q = static_cast<const T *>(a.q) + boff * a.ck;
+        const T *g = static_cast<const T *>(a.dy) + boff * a.cv;
+        const float w = a.quad_w[a.lat_halo_start + hi];
+        for (int64_t z = z0; z < z1; z++) {
+            const long cell = up_cell(a, a.col_idx[z], a.lon_lo_kx + wl);
+            if (cell < 0) continue;
+            const T *qc = q + cell * a.ck, *gc = g + cell * a.cv;
+            const float s = up_dot(kr, qc, a.ck, lane);
+            const float gv = up_dot(vr, gc, a.cv, lane);
+            const float p = __expf(s - a.qdotk_max[boff + cell]) * w / a.alpha_sum[boff + cell];
+            const float sk = (gv - a.integral_norm[boff + cell]) * p;
+#pragma unroll
+            for (int i = 0; i < NCI; i++) {
+                const int c = lane + 64 * i;
+                if (c < a.ck) dk[i] = fmaf(sk, ld(qc + c), dk[i]);
+                if (c < a.cv) dv[i] = fmaf(p, ld(gc + c), dv[i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NCI; i++) {
+        const int c = lane + 64 * i;
+        if (c < a.ck) a.dk[pt * a.ck + c] = dk[i];
+        if (c < a.cv) a.dv[pt * a.cv + c] = dv[i];
+    }
+}
+
 } // namespace s2ring
 
 namespace {
@@ -336,4 +543,117 @@ extern "C" int s2attn_ring_backward_pass2(const void *k, const void *v, const vo
     a.dk = dk, a.dv = dv;
     a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off, a.row_idx = row_idx;
     return launch(PASS2, a, shape->dtype, stream);
+}
+
+namespace {
+
+int check_up(const s2attn_ring_up_shape *sh)
+{
+    if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "ring shape is null");
+    if (sh->batch < 1 || sh->nlat_halo < 1 || sh->nlon_kx < 1 || sh->nlat_out < 1 || sh->nlon_out < 1 || sh->nlon_out_global < 1)
+        return s2attn_fail(S2ATTN_E_INVALID, "batch and grid extents must be positive");
+    if (sh->ck < 1 || sh->cv < 1) return s2attn_fail(S2ATTN_E_INVALID, "channel counts must be positive");
+    if (sh->ck > MAXC || sh->cv > MAXC)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "channels above %d are not instantiated (ck=%d, cv=%d)", MAXC, sh->ck, sh->cv);
+    if (sh->pscale_out < 1 || sh->nlon_out > sh->nlon_out_global)
+        return s2attn_fail(S2ATTN_E_INVALID, "pscale_out must be positive and the local output width at most the global one");
+    if (sh->lon_lo_kx < 0 || (int64_t)sh->pscale_out * (sh->lon_lo_kx + sh->nlon_kx) > sh->nlon_out_global)
+        return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", sh->lon_lo_kx, sh->lon_lo_kx + sh->nlon_kx,
+                           sh->nlon_out_global / sh->pscale_out);
+    if (sh->dtype != S2ATTN_F32 && sh->dtype != S2ATTN_BF16 && sh->dtype != S2ATTN_F16)
+        return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
+    return S2ATTN_OK;
+}
+
+void fill_up(UpArgs &a, const s2attn_ring_up_shape *sh)
+{
+    a.B = sh->batch, a.nlat_halo = sh->nlat_halo, a.nlon_kx = sh->nlon_kx, a.Ho = sh->nlat_out, a.Wo = sh->nlon_out;
+    a.ck = sh->ck, a.cv = sh->cv, a.nlon_out_global = sh->nlon_out_global, a.pscale_out = sh->pscale_out;
+    a.lon_lo_kx = sh->lon_lo_kx, a.lat_halo_start = sh->lat_halo_start;
+}
+
+enum UpStep { UP_MAX, UP_RESCALE, UP_ACC, UP_PASS1, UP_PASS2 };
+
+template <typename T> int launch_up_t(UpStep step, const UpArgs &a, hipStream_t stream)
+{
+    const long n = step == UP_RESCALE ? (long)a.B * a.Ho * a.Wo : (long)a.B * a.nlat_halo * a.nlon_kx;
+    const long nblocks = (n + 3) / 4;
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    void (*kern)(const UpArgs) = nullptr;
+    switch (step) {
+    case UP_MAX: kern = up_max_kernel<T>; break;
+    case UP_RESCALE: kern = up_rescale_kernel; break;
+    case UP_ACC: kern = up_acc_kernel<T>; break;
+    case UP_PASS1: kern = up_pass1_kernel<T>; break;
+    default: kern = up_pass2_kernel<T>; break;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+
+int launch_up(UpStep step, const UpArgs &a, int dtype, void *stream)
+{
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (dtype == S2ATTN_F32) return launch_up_t<float>(step, a, st);
+    if (dtype == S2ATTN_BF16) return launch_up_t<__hip_bfloat16>(step, a, st);
+    return launch_up_t<__half>(step, a, st);
+}
+
+} // namespace
+
+extern "C" int s2attn_ring_forward_step_upsample(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                                                 float *max_scratch, const float *quad_weights, const int64_t *col_idx,
+                                                 const int64_t *row_off, const s2attn_ring_up_shape *shape, void *stream)
+{
+    int rc = check_up(shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!k || !v || !q || !y_acc || !alpha_sum || !qdotk_max || !max_scratch || !quad_weights || !col_idx || !row_off)
+        return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    UpArgs a = {};
+    fill_up(a, shape);
+    a.k = k, a.v = v, a.q = q, a.y_acc = y_acc, a.alpha_sum = alpha_sum, a.qdotk_max = qdotk_max, a.max_curr = max_scratch;
+    a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off;
+    const size_t bytes = sizeof(float) * (size_t)a.B * a.Ho * a.Wo;
+    const hipError_t e = hipMemcpyAsync(max_scratch, qdotk_max, bytes, hipMemcpyDeviceToDevice, static_cast<hipStream_t>(stream));
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipMemcpyAsync: %s", hipGetErrorString(e));
+    if ((rc = launch_up(UP_MAX, a, shape->dtype, stream)) != S2ATTN_OK) return rc;
+    if ((rc = launch_up(UP_RESCALE, a, shape->dtype, stream)) != S2ATTN_OK) return rc;
+    return launch_up(UP_ACC, a, shape->dtype, stream);
+}
+
+extern "C" int s2attn_ring_backward_pass1_upsample(const void *k, const void *v, const void *q, const void *dy, const float *qdotk_max,
+                                                   float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                                                   const int64_t *col_idx, const int64_t *row_off, const s2attn_ring_up_shape *shape,
+                                                   void *stream)
+{
+    const int rc = check_up(shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!k || !v || !q || !dy || !qdotk_max || !integral || !alpha_k || !alpha_kvw || !quad_weights || !col_idx || !row_off)
+        return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    UpArgs a = {};
+    fill_up(a, shape);
+    a.k = k, a.v = v, a.q = q, a.dy = dy, a.qdotk_max = const_cast<float *>(qdotk_max);
+    a.integral = integral, a.alpha_k = alpha_k, a.alpha_kvw = alpha_kvw;
+    a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off;
+    return launch_up(UP_PASS1, a, shape->dtype, stream);
+}
+
+extern "C" int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                                   const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                                   const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
+                                                   const s2attn_ring_up_shape *shape, void *stream)
+{
+    const int rc = check_up(shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!k || !v || !q || !dy || !alpha_sum || !qdotk_max || !integral_norm || !dk || !dv || !quad_weights || !col_idx || !row_off)
+        return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    UpArgs a = {};
+    fill_up(a, shape);
+    a.k = k, a.v = v, a.q = q, a.dy = dy;
+    a.alpha_sum = const_cast<float *>(alpha_sum), a.qdotk_max = const_cast<float *>(qdotk_max), a.integral_norm = integral_norm;
+    a.dk = dk, a.dv = dv;
+    a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off;
+    return launch_up(UP_PASS2, a, shape->dtype, stream);
 }

@@ -434,8 +434,10 @@ def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out
     return _lib.RingShapeStruct(B, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, vx.shape[3], nlon_in, pscale, lon_lo_kx, lat_halo_start, _DTYPE_CODE[qy.dtype])
 
 
-def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out):
-    """state: (name, tensor, trailing channel count or None) fp32 buffers shaped like the local output grid."""
+def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out, nrows=None):
+    """state: (name, tensor, trailing channel count or None) fp32 buffers shaped like the local output grid; nrows: rows of
+    the CSR (output latitudes in the gather direction, the chunk's input latitudes in the scatter direction); row_idx only
+    exists in the gather direction."""
     for name, t in (("kx", kx), ("vx", vx), ("qy", qy)) + ((("dy", dy),) if dy is not None else ()):
         if t.dim() != 4 or not t.is_contiguous():
             raise RuntimeError(f"{name} must be a contiguous 4-dimensional (batch*heads, nlat, nlon, channels) tensor")
@@ -453,12 +455,14 @@ def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_id
         if tuple(t.shape) != want or t.dtype != torch.float32 or not t.is_contiguous():
             raise RuntimeError(f"{name} must be a contiguous fp32 tensor of shape {want}")
         _require_gpu(t, name, kx.device)
-    for name, t, dt in (("quad_weights", quad_weights, torch.float32), ("col_idx", col_idx, torch.int64), ("row_off", row_off, torch.int64), ("row_idx", row_idx, torch.int32)):
+    index = (("quad_weights", quad_weights, torch.float32), ("col_idx", col_idx, torch.int64), ("row_off", row_off, torch.int64))
+    for name, t, dt in index + ((("row_idx", row_idx, torch.int32),) if row_idx is not None else ()):
         if t.dtype != dt or not t.is_contiguous():
             raise RuntimeError(f"{name} must be a contiguous {dt} tensor")
         _require_gpu(t, name, kx.device)
-    if row_off.numel() != nlat_out + 1 or row_idx.numel() != nlat_out:
-        raise RuntimeError("row_off must have nlat_out + 1 entries and row_idx nlat_out")
+    nrows = nlat_out if nrows is None else nrows
+    if row_off.numel() != nrows + 1 or (row_idx is not None and row_idx.numel() != nrows):
+        raise RuntimeError(f"row_off must have {nrows + 1} entries" + ("" if row_idx is None else f" and row_idx {nrows}"))
 
 
 @torch.library.custom_op("s2attn::forward_ring_step", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
@@ -594,4 +598,140 @@ def backward_ring_step_pass2(
 
 @backward_ring_step_pass2.register_fake
 def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_norm_buf, dkx, dvx, quad_weights, col_idx, row_off, row_idx, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out, n_long_rows, max_row_len, mid_row_len):
+    return None
+
+
+# ---- up-sampling direction (attention_interface.cpp:158-189, fake kernels attention_optimized.py:163-227) ------------
+def _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out) -> _lib.RingUpShapeStruct:
+    B, nlat_halo, nlon_kx, ck = kx.shape
+    return _lib.RingUpShapeStruct(B, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, vx.shape[3], nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, _DTYPE_CODE[qy.dtype])
+
+
+def _ring_up_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, nlat_out, nlon_out):
+    _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, None, nlat_out, nlon_out, nrows=kx.shape[1])
+
+
+@torch.library.custom_op("s2attn::forward_ring_step_upsample", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
+def forward_ring_step_upsample(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    y_acc: torch.Tensor,
+    alpha_sum_buf: torch.Tensor,
+    qdotk_max_buf: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    nlon_in: int,
+    nlon_out_global: int,
+    pscale_out: int,
+    lon_lo_kx: int,
+    lat_halo_start: int,
+    nlat_out: int,
+    nlon_out: int,
+) -> None:
+    state = (("y_acc", y_acc, vx.shape[3]), ("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None))
+    _ring_up_validate(kx, vx, qy, None, state, quad_weights, col_idx, row_off, nlat_out, nlon_out)
+    if qy.numel() == 0 or kx.numel() == 0:
+        return
+    shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    scratch = torch.empty_like(qdotk_max_buf)
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_ring_forward_step_upsample(
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(), scratch.data_ptr(),
+            quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+        )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_forward_step_upsample")
+
+
+@forward_ring_step_upsample.register_fake
+def _(kx, vx, qy, y_acc, alpha_sum_buf, qdotk_max_buf, quad_weights, col_idx, row_off, nlon_in, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out):
+    return None
+
+
+@torch.library.custom_op("s2attn::backward_ring_step_upsample_pass1", mutates_args=("integral_buf", "alpha_k_buf", "alpha_kvw_buf"))
+def backward_ring_step_upsample_pass1(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    dy: torch.Tensor,
+    qdotk_max_buf: torch.Tensor,
+    integral_buf: torch.Tensor,
+    alpha_k_buf: torch.Tensor,
+    alpha_kvw_buf: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    nlon_in: int,
+    nlon_out_global: int,
+    pscale_out: int,
+    lon_lo_kx: int,
+    lat_halo_start: int,
+    nlat_out: int,
+    nlon_out: int,
+) -> None:
+    ck = kx.shape[3]
+    state = (("qdotk_max_buf", qdotk_max_buf, None), ("integral_buf", integral_buf, None), ("alpha_k_buf", alpha_k_buf, ck), ("alpha_kvw_buf", alpha_kvw_buf, ck))
+    _ring_up_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, nlat_out, nlon_out)
+    if qy.numel() == 0 or kx.numel() == 0:
+        return
+    shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_ring_backward_pass1_upsample(
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), qdotk_max_buf.data_ptr(), integral_buf.data_ptr(), alpha_k_buf.data_ptr(),
+            alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+        )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_backward_pass1_upsample")
+
+
+@backward_ring_step_upsample_pass1.register_fake
+def _(kx, vx, qy, dy, qdotk_max_buf, integral_buf, alpha_k_buf, alpha_kvw_buf, quad_weights, col_idx, row_off, nlon_in, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out):
+    return None
+
+
+@torch.library.custom_op("s2attn::backward_ring_step_upsample_pass2", mutates_args=("dkx", "dvx"))
+def backward_ring_step_upsample_pass2(
+    kx: torch.Tensor,
+    vx: torch.Tensor,
+    qy: torch.Tensor,
+    dy: torch.Tensor,
+    alpha_sum_buf: torch.Tensor,
+    qdotk_max_buf: torch.Tensor,
+    integral_norm_buf: torch.Tensor,
+    dkx: torch.Tensor,
+    dvx: torch.Tensor,
+    quad_weights: torch.Tensor,
+    col_idx: torch.Tensor,
+    row_off: torch.Tensor,
+    nlon_in: int,
+    nlon_out_global: int,
+    pscale_out: int,
+    lon_lo_kx: int,
+    lat_halo_start: int,
+    nlat_out: int,
+    nlon_out: int,
+) -> None:
+    state = (("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None), ("integral_norm_buf", integral_norm_buf, None))
+    _ring_up_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, nlat_out, nlon_out)
+    for name, t, like in (("dkx", dkx, kx), ("dvx", dvx, vx)):
+        if t.shape != like.shape or t.dtype != torch.float32 or not t.is_contiguous():
+            raise RuntimeError(f"{name} must be a contiguous fp32 tensor shaped like its input, {tuple(like.shape)}")
+        _require_gpu(t, name, kx.device)
+    if kx.numel() == 0:
+        return
+    if qy.numel() == 0:
+        dkx.zero_()
+        dvx.zero_()
+        return
+    shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    with torch.cuda.device(kx.device):
+        rc = _lib.load().s2attn_ring_backward_pass2_upsample(
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(), integral_norm_buf.data_ptr(),
+            dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+        )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_backward_pass2_upsample")
+
+
+@backward_ring_step_upsample_pass2.register_fake
+def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_norm_buf, dkx, dvx, quad_weights, col_idx, row_off, nlon_in, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out):
     return None
