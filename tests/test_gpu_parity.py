@@ -90,6 +90,11 @@ SMALL_CASES = [
     (1, 3, 20, 20, (12, 48), (12, 48), "equiangular", "equiangular", 0.5),
     (2, 1, 100, 100, (6, 32), (6, 32), "equiangular", "equiangular", 0.9),
     (1, 2, 48, 48, (12, 96), (6, 48), "equiangular", "equiangular", 0.5),
+    # fp32 heads of 129..256 channels: two wavefronts per workgroup, one per group of 128 channels (256 and 192 channels
+    # are in SAVED_CASES below, against the float64 oracle alone: two fp32 evaluations of 256-term sums differ by more
+    # than 1e-5 from EACH OTHER)
+    (1, 2, 132, 132, (10, 64), (5, 32), "equiangular", "equiangular", 0.7),
+    (2, 1, 200, 200, (6, 36), (6, 36), "legendre-gauss", "legendre-gauss", 0.9),
     (1, 1, 128, 128, (10, 72), (5, 36), "equiangular", "legendre-gauss", 0.7),
     # head dim 32 on grids wide enough for the matrix-core kernels (nlon >= 64), incl. full-circle rows and long runs
     (1, 2, 32, 32, (24, 96), (24, 96), "equiangular", "equiangular", 0.5),

@@ -2575,31 +2575,38 @@ template <typename T> bool h16_ok(Which which, const Args &a)
 }
 
 // fp32 16-longitude matrix-core kernels, tiles of 16, 32, 64 or 128 channels: same launch geometry and the same conditions as the 16-bit family.
-template <int D> int launch_m32(Which which, const Args &a0, hipStream_t stream)
+template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream)
 {
     Args a = a0;
     a.row_first = 0;
     void (*kern)(const Args) = nullptr;
     long nblocks = 0;
+    int lds = NS > 1 ? m32_lds_bytes<D, NS>(false) : 0; // one wavefront per workgroup: static LDS
     if (which == FWD) {
-        kern = fwd_m32_kernel<D>;
+        kern = fwd_m32_kernel<D, NS>;
         nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
     } else if (which == DQ) {
-        kern = dq_m32_kernel<D>;
+        kern = dq_m32_kernel<D, NS>;
         nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
     } else {
-        kern = dkdv_m32_kernel<D>;
+        kern = dkdv_m32_kernel<D, NS>;
         nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
+        lds = NS > 1 ? m32_lds_bytes<D, NS>(true) : 0;
     }
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    if (lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * NS), lds, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
 
-// Head widths: any multiple of 4 from 16 to 128, staged in a tile of 16, 32, 64 or 128 channels (zeros past the head).
-bool m32_width(int ck, int cv) { return ck == cv && ck % 4 == 0 && ck >= 16 && ck <= 128; }
+// Head widths: any multiple of 4 from 16 to 256, staged in a tile of 16, 32, 64 or 128 channels (zeros past the head), or in
+// two channel groups of 128 worked on by two wavefronts.
+bool m32_width(int ck, int cv) { return ck == cv && ck % 4 == 0 && ck >= 16 && ck <= 256; }
 
 template <typename T> bool m32_ok(Which which, const Args &a)
 {
@@ -2638,9 +2645,10 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         return launch_dense<T>(which, a, nrows, stream);
     }
     if (m32_ok<T>(which, a)) {
-        if (a.dk_ <= 16) return launch_m32<16>(which, a, stream);
-        if (a.dk_ <= 32) return launch_m32<32>(which, a, stream);
-        return a.dk_ <= 64 ? launch_m32<64>(which, a, stream) : launch_m32<128>(which, a, stream);
+        if (a.dk_ <= 16) return launch_m32<16, 1>(which, a, stream);
+        if (a.dk_ <= 32) return launch_m32<32, 1>(which, a, stream);
+        if (a.dk_ <= 64) return launch_m32<64, 1>(which, a, stream);
+        return a.dk_ <= 128 ? launch_m32<128, 1>(which, a, stream) : launch_m32<128, 2>(which, a, stream);
     }
     return vec ? launch_p<T, true>(which, a, first, nrows - first, stream) : launch_p<T, false>(which, a, first, nrows - first, stream);
 }

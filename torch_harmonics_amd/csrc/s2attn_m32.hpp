@@ -15,6 +15,77 @@
 //   second products (V^T P^T, K^T dS^T, ...): k slot qd of instruction (kb, v) <-> position 16 kb + 4 qd + v.  B is
 //     register v of score block kb as it stands, A one float of the staged tile (lanes c read consecutive channels).
 
+// Heads wider than 128 channels: NS = 2 wavefronts per workgroup, each owning a contiguous group of D = 128 channels (its own
+// tiles, operands and output channels); the partial scores of the groups are added through LDS once per step, after which
+// both wavefronts hold the same probabilities.  One wavefront cannot hold a 256-channel step in registers.
+
+#define S2_M32_IDS(W_TILED, NROWS)                                            \
+    const int lane = NS > 1 ? (int)(threadIdx.x & 63) : (int)threadIdx.x;     \
+    const int wv = NS > 1 ? (int)(threadIdx.x >> 6) : 0;                      \
+    const int c = lane & 15, qd = lane >> 4;                                  \
+    const int BH = a.B * a.nh;                                                \
+    const int ntile = ((W_TILED) + HQ - 1) / HQ;                              \
+    int bh, id_;                                                              \
+    xcd_split(blockIdx.x, BH, ntile *(NROWS), bh, id_);                       \
+    const int grp_ = id_ / (HG * ntile);                                      \
+    const int grows_ = min(HG, (NROWS)-grp_ * HG);                            \
+    id_ -= grp_ * HG * ntile;                                                 \
+    const int wt = id_ / grows_;                                              \
+    const int rowsel = grp_ * HG + id_ % grows_;                              \
+    const int b = bh / a.nh, h = bh % a.nh;                                   \
+    const int w0 = wt * HQ;                                                   \
+    const int nvalid = min(HQ, (W_TILED)-w0);                                 \
+    const int drt = a.dk_;                 /* real head width */              \
+    const int cbase = wv * D;              /* first channel of this wavefront's group */ \
+    const int dr = min(D, drt - cbase);    /* real channels in the group */
+
+extern __shared__ float4 m32_smem[];
+
+// LDS of a workgroup: a static array when it is one wavefront (addresses are then compile-time constants), the dynamic
+// allocation of the launch when it is more (two 128-channel wavefronts need more than the 64 KB a static array may have).
+template <int BYTES, int NS> __device__ inline char *m32_lds()
+{
+    if constexpr (NS == 1) {
+        __shared__ __attribute__((aligned(16))) char buf[BYTES];
+        return buf;
+    } else {
+        return reinterpret_cast<char *>(m32_smem);
+    }
+}
+
+// LDS bytes of a kernel of this family: per wavefront two tiles (+ two rows of statistics in the dk/dv pass), then the
+// exchange area of 16 floats per lane and wavefront when there is more than one.
+template <int D, int NS> constexpr int m32_wave_bytes(bool stats) { return 2 * HK * (4 * D + 16) + (stats ? 2 * HK * 4 : 0); }
+template <int D, int NS> constexpr int m32_lds_bytes(bool stats) { return NS * m32_wave_bytes<D, NS>(stats) + (NS > 1 ? NS * 64 * 16 * 4 : 0); }
+
+// Adds the other wavefronts' partial blocks to this wavefront's: x0 (and x1 when given) hold 8 floats per lane each.
+template <int NS> __device__ inline void m32_exchange(float *xs, int wv, int lane, f4v (&x0)[2], f4v (*x1)[2])
+{
+    if constexpr (NS > 1) {
+        float4 *mine = reinterpret_cast<float4 *>(xs + (wv * 64 + lane) * 16);
+        mine[0] = make_float4(x0[0][0], x0[0][1], x0[0][2], x0[0][3]);
+        mine[1] = make_float4(x0[1][0], x0[1][1], x0[1][2], x0[1][3]);
+        if (x1) {
+            mine[2] = make_float4((*x1)[0][0], (*x1)[0][1], (*x1)[0][2], (*x1)[0][3]);
+            mine[3] = make_float4((*x1)[1][0], (*x1)[1][1], (*x1)[1][2], (*x1)[1][3]);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int o = 0; o < NS; o++) {
+            if (o == wv) continue;
+            const float4 *other = reinterpret_cast<const float4 *>(xs + (o * 64 + lane) * 16);
+            const float4 a0 = other[0], a1 = other[1];
+            x0[0] += f4v{a0.x, a0.y, a0.z, a0.w};
+            x0[1] += f4v{a1.x, a1.y, a1.z, a1.w};
+            if (x1) {
+                const float4 b0 = other[2], b1 = other[3];
+                (*x1)[0] += f4v{b0.x, b0.y, b0.z, b0.w};
+                (*x1)[1] += f4v{b1.x, b1.y, b1.z, b1.w};
+            }
+        }
+    }
+}
+
 // fp32 tile of D channels.  With a row pitch of 16 bytes modulo 128 the four-byte reads of the second products (two
 // rows 4 apart per 32 lanes, 16 consecutive floats each) fall in distinct banks.
 template <int D> struct FTile : BandTile<D / 4, 4 * D + 16> {};
@@ -95,24 +166,23 @@ template <int D> __device__ inline void m32_load_quarter(float (&op)[D / 4], con
 }
 
 // ---- forward ---------------------------------------------------------------------------------------------------
-template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args a)
+template <int D, int NS> __global__ __launch_bounds__(64 * NS) void fwd_m32_kernel(const Args a)
 {
     typedef FTile<D> Tile;
     constexpr int PITCH = Tile::PITCH, NCB = D / 16;
-    __shared__ __attribute__((aligned(16))) char Ks[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) char Vs[HK * PITCH];
-
-    S2_H16_IDS(a.Wo, a.Ho)
+    S2_M32_IDS(a.Wo, a.Ho)
+    char *lds = m32_lds<m32_lds_bytes<D, NS>(false), NS>();
+    char *Ks = lds + wv * m32_wave_bytes<D, NS>(false), *Vs = Ks + HK * PITCH;
+    float *xs = reinterpret_cast<float *>(lds + NS * m32_wave_bytes<D, NS>(false));
     const int ho = a.gorder[a.row_first + rowsel];
-    const int dr = a.dk_;              // real head width
-    const unsigned ldb = a.nh * dr * 4; // bytes between two grid points
-    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
-    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
+    const unsigned ldb = a.nh * drt * 4; // bytes between two grid points
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (drt * 4) + cbase * 4;
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (drt * 4) + cbase * 4;
     const bool mine = c < nvalid;
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
 
     float qop[D / 4];
-    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (dr * 4), qd, dr);
+    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb + (size_t)h * (drt * 4) + cbase * 4, qd, dr);
     f4v acc[NCB]; // Y^T: register v of block cb is channel 16 cb + 4 qd + v of column c
 #pragma unroll
     for (int cb = 0; cb < NCB; cb++) acc[cb] = f4v{0.f, 0.f, 0.f, 0.f};
@@ -158,6 +228,7 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
 
         f4v sc[2];
         m32_scores<D, PITCH>(sc, Ks, c, qd, qop);
+        m32_exchange<NS>(xs, wv, lane, sc, nullptr);
         // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
         const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
         float mx = -INFINITY;
@@ -204,9 +275,9 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
 
     S = h16_quarter_sum(S);
     if (mine) {
-        if (a.lse && qd == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + c] = m + fast_log2(S);
+        if (a.lse && qd == 0 && wv == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + c] = m + fast_log2(S);
         const float inv = 1.0f / S;
-        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
+        char *y = static_cast<char *>(a.y) + pt * ldb + (size_t)h * (drt * 4) + cbase * 4 + 16 * qd;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++)
             if (16 * cb + 4 * qd < dr)
@@ -216,19 +287,18 @@ template <int D> __global__ __launch_bounds__(64) void fwd_m32_kernel(const Args
 
 // ---- backward, dq pass (needs the forward's y and lse) -------------------------------------------------------------
 // Three products per step:  S^T = K Q^T,  G^T = V dY^T,  dQ^T += K^T dS^T  with dS = P o (G - I),  I = <dy, y>.
-template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args a)
+template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dq_m32_kernel(const Args a)
 {
     typedef FTile<D> Tile;
     constexpr int PITCH = Tile::PITCH, NCB = D / 16;
-    __shared__ __attribute__((aligned(16))) char Ks[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) char Vs[HK * PITCH];
-
-    S2_H16_IDS(a.Wo, a.Ho)
+    S2_M32_IDS(a.Wo, a.Ho)
+    char *lds = m32_lds<m32_lds_bytes<D, NS>(false), NS>();
+    char *Ks = lds + wv * m32_wave_bytes<D, NS>(false), *Vs = Ks + HK * PITCH;
+    float *xs = reinterpret_cast<float *>(lds + NS * m32_wave_bytes<D, NS>(false));
     const int ho = a.gorder[a.row_first + rowsel];
-    const int dr = a.dk_;
-    const unsigned ldb = a.nh * dr * 4;
-    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
-    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (dr * 4);
+    const unsigned ldb = a.nh * drt * 4;
+    const char *kx = static_cast<const char *>(a.k) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (drt * 4) + cbase * 4;
+    const char *vx = static_cast<const char *>(a.v) + ((size_t)b * a.Hi * a.Wi * a.nh + h) * (drt * 4) + cbase * 4;
     const bool mine = c < nvalid;
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? c : 0)) * a.qps;
     const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
@@ -236,7 +306,7 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
     float qop[D / 4], gop[D / 4];
     float I = 0.f;
     {
-        const size_t off = pt * ldb + (size_t)h * (dr * 4);
+        const size_t off = pt * ldb + (size_t)h * (drt * 4) + cbase * 4;
         m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + off, qd, dr);
         m32_load_quarter<D>(gop, static_cast<const char *>(a.dy) + off, qd, dr);
         float yq[D / 4];
@@ -245,6 +315,15 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
         for (int i = 0; i < D / 4; i++) I = fmaf(gop[i], yq[i], I);
     }
     I = h16_quarter_sum(I);
+    if constexpr (NS > 1) { // <dy, y> over all channel groups
+        xs[wv * 64 + lane] = I;
+        __syncthreads();
+        float t = 0.f;
+#pragma unroll
+        for (int o = 0; o < NS; o++) t += xs[o * 64 + lane];
+        I = t;
+        __syncthreads();
+    }
     const float lse = a.lse[sidx];
 
     f4v acc[NCB];
@@ -295,6 +374,7 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
         f4v sc[2], gc[2];
         m32_scores<D, PITCH>(sc, Ks, c, qd, qop);
         m32_scores<D, PITCH>(gc, Vs, c, qd, gop);
+        m32_exchange<NS>(xs, wv, lane, sc, &gc);
         const int tb = pos + 4 * qd - c;
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
@@ -320,9 +400,9 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
 
     // (stored after the walk: a global store ahead of the loop would turn the loop's scalar loads of runs and weights,
     // which the compiler only uses while nothing in the kernel can have written memory, into vector loads with waits)
-    if (mine && qd == 0) a.stats[sidx] = make_float2(lse, I);
+    if (mine && qd == 0 && wv == 0) a.stats[sidx] = make_float2(lse, I);
     if (mine) {
-        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
+        char *dq = static_cast<char *>(a.dq) + pt * ldb + (size_t)h * (drt * 4) + cbase * 4 + 16 * qd;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++)
             if (16 * cb + 4 * qd < dr) *reinterpret_cast<float4 *>(dq + 64 * cb) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
@@ -333,28 +413,26 @@ template <int D> __global__ __launch_bounds__(64) void dq_m32_kernel(const Args 
 // The wavefront owns 16 INPUT longitudes (column c = key) and walks the runs grouped by input latitude; staged rows
 // are queries.  Staged row r of a run (first row = longitude w0 - ws - len + 1) sees key c iff 0 <= r - c < len.
 // Four products per step:  S = Q K^T,  G = dY V^T  (rows = queries, columns = keys),  dV^T += dY^T P,  dK^T += Q^T dS.
-template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Args a)
+template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dkdv_m32_kernel(const Args a)
 {
     typedef FTile<D> Tile;
     constexpr int PITCH = Tile::PITCH, NCB = D / 16;
-    __shared__ __attribute__((aligned(16))) char Qs[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) char Gs[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) float Ls[HK];
-    __shared__ __attribute__((aligned(16))) float Is[HK];
-
-    S2_H16_IDS(a.Wi, a.Hi)
+    S2_M32_IDS(a.Wi, a.Hi)
+    char *lds = m32_lds<m32_lds_bytes<D, NS>(true), NS>();
+    char *Qs = lds + wv * m32_wave_bytes<D, NS>(true), *Gs = Qs + HK * PITCH;
+    float *Ls = reinterpret_cast<float *>(Gs + HK * PITCH), *Is = Ls + HK;
+    float *xs = reinterpret_cast<float *>(lds + NS * m32_wave_bytes<D, NS>(true));
     const int hi = a.sorder[a.row_first + rowsel];
-    const int dr = a.dk_;
-    const unsigned ldb = a.nh * dr * 4;
-    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (dr * 4);
-    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (dr * 4);
+    const unsigned ldb = a.nh * drt * 4;
+    const char *qy = static_cast<const char *>(a.q) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (drt * 4) + cbase * 4;
+    const char *gy = static_cast<const char *>(a.dy) + ((size_t)b * a.Ho * a.Wo * a.nh + h) * (drt * 4) + cbase * 4;
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = c < nvalid;
     const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? c : 0)) * a.kps;
 
     float kop[D / 4], vop[D / 4]; // this lane's quarter of key c
     {
-        const size_t off = pt * ldb + (size_t)h * (dr * 4);
+        const size_t off = pt * ldb + (size_t)h * (drt * 4) + cbase * 4;
         m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + off, qd, dr);
         m32_load_quarter<D>(vop, static_cast<const char *>(a.v) + off, qd, dr);
     }
@@ -419,6 +497,7 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
         f4v sc[2], gc[2];
         m32_scores<D, PITCH>(sc, Qs, c, qd, kop);
         m32_scores<D, PITCH>(gc, Gs, c, qd, vop);
+        m32_exchange<NS>(xs, wv, lane, sc, &gc);
         const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
@@ -446,7 +525,7 @@ template <int D> __global__ __launch_bounds__(64) void dkdv_m32_kernel(const Arg
     }
 
     if (mine) {
-        const size_t off = pt * ldb + (size_t)h * (dr * 4) + 16 * qd;
+        const size_t off = pt * ldb + (size_t)h * (drt * 4) + cbase * 4 + 16 * qd;
         char *dk = static_cast<char *>(a.dk) + off, *dv = static_cast<char *>(a.dv) + off;
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++) {
