@@ -131,8 +131,8 @@ int s2attn_forward_lse(const void *k, const void *v, const void *q, const float 
  * Writes dk, dv, dq (every element; no pre-zeroing needed, no atomics).
  * workspace: device scratch of s2attn_backward_workspace_bytes(shape) bytes, 8-byte aligned (16 for the matrix-core
  * shapes below): two fp32 softmax statistics per (batch, head, output point), plus, for the shapes whose dq pass works
- * from the forward's output and normaliser (16-bit storage with a head dim that is a multiple of 8, fp32 with one that is a
- * multiple of 4, from 16 to 256, ck == cv, at least 32 columns per virtual latitude), room to recompute those two when the caller does not pass them.
+ * from the forward's output and normaliser (16-bit storage with a head dim that is a multiple of 8 from 16 to 256, fp32 with
+ * one that is a multiple of 4 from 16 to 512, ck == cv, at least 32 columns per virtual latitude), room to recompute those two when the caller does not pass them.
  */
 int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape);
 

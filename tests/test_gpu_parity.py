@@ -197,6 +197,9 @@ SAVED_CASES = [
     # up to 256 channels per head on the 16-bit matrix-core kernels (fp32: wide vector kernels)
     (1, 1, 256, 256, (8, 40), (8, 40), "equiangular", "equiangular", 0.8),
     (1, 2, 192, 192, (6, 36), (6, 36), "legendre-gauss", "legendre-gauss", 0.9),
+    # fp32: three and four channel groups (16-bit storage: wide vector kernels)
+    (1, 1, 320, 320, (6, 36), (6, 36), "equiangular", "equiangular", 0.9),
+    (1, 1, 512, 512, (6, 32), (6, 32), "equiangular", "equiangular", 0.9),
     (2, 3, 64, 64, (10, 33), (10, 33), "equiangular", "equiangular", 0.8),
     (1, 1, 128, 128, (10, 40), (10, 40), "equiangular", "equiangular", 0.7),
 ]

@@ -2604,9 +2604,9 @@ template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t
     return S2ATTN_OK;
 }
 
-// Head widths: any multiple of 4 from 16 to 256, staged in a tile of 16, 32, 64 or 128 channels (zeros past the head), or in
-// two channel groups of 128 worked on by two wavefronts.
-bool m32_width(int ck, int cv) { return ck == cv && ck % 4 == 0 && ck >= 16 && ck <= 256; }
+// Head widths: any multiple of 4 from 16 to 512, staged in a tile of 16, 32, 64 or 128 channels (zeros past the head), or in
+// two to four channel groups of 128 worked on by as many wavefronts.
+bool m32_width(int ck, int cv) { return ck == cv && ck % 4 == 0 && ck >= 16 && ck <= 512; }
 
 template <typename T> bool m32_ok(Which which, const Args &a)
 {
@@ -2648,7 +2648,9 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         if (a.dk_ <= 16) return launch_m32<16, 1>(which, a, stream);
         if (a.dk_ <= 32) return launch_m32<32, 1>(which, a, stream);
         if (a.dk_ <= 64) return launch_m32<64, 1>(which, a, stream);
-        return a.dk_ <= 128 ? launch_m32<128, 1>(which, a, stream) : launch_m32<128, 2>(which, a, stream);
+        if (a.dk_ <= 128) return launch_m32<128, 1>(which, a, stream);
+        if (a.dk_ <= 256) return launch_m32<128, 2>(which, a, stream);
+        return a.dk_ <= 384 ? launch_m32<128, 3>(which, a, stream) : launch_m32<128, 4>(which, a, stream);
     }
     return vec ? launch_p<T, true>(which, a, first, nrows - first, stream) : launch_p<T, false>(which, a, first, nrows - first, stream);
 }
