@@ -58,7 +58,7 @@ template <int BYTES, int NS> __device__ inline char *m32_lds()
 template <int D, int NS> constexpr int m32_wave_bytes(bool stats) { return 2 * HK * (4 * D + 16) + (stats ? 2 * HK * 4 : 0); }
 template <int D, int NS> constexpr int m32_lds_bytes(bool stats) { return NS * m32_wave_bytes<D, NS>(stats) + (NS > 1 ? NS * 64 * 16 * 4 : 0); }
 
-// Adds the other wavefronts' partial blocks to this wavefront's: x0 (and x1 when given) hold 8 floats per lane each.
+// Replaces this wavefront's partial blocks by the sum over all wavefronts: x0 (and x1 when given) hold 8 floats per lane each.
 template <int NS> __device__ inline void m32_exchange(float *xs, int wv, int lane, f4v (&x0)[2], f4v (*x1)[2])
 {
     if constexpr (NS > 1) {
@@ -70,15 +70,17 @@ template <int NS> __device__ inline void m32_exchange(float *xs, int wv, int lan
             mine[3] = make_float4((*x1)[1][0], (*x1)[1][1], (*x1)[1][2], (*x1)[1][3]);
         }
         __syncthreads();
+        // every wavefront adds the blocks in the same order (its own included), so all of them hold bit-identical sums
+        x0[0] = x0[1] = f4v{0.f, 0.f, 0.f, 0.f};
+        if (x1) (*x1)[0] = (*x1)[1] = f4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int o = 0; o < NS; o++) {
-            if (o == wv) continue;
-            const float4 *other = reinterpret_cast<const float4 *>(xs + (o * 64 + lane) * 16);
-            const float4 a0 = other[0], a1 = other[1];
+            const float4 *part = reinterpret_cast<const float4 *>(xs + (o * 64 + lane) * 16);
+            const float4 a0 = part[0], a1 = part[1];
             x0[0] += f4v{a0.x, a0.y, a0.z, a0.w};
             x0[1] += f4v{a1.x, a1.y, a1.z, a1.w};
             if (x1) {
-                const float4 b0 = other[2], b1 = other[3];
+                const float4 b0 = part[2], b1 = part[3];
                 (*x1)[0] += f4v{b0.x, b0.y, b0.z, b0.w};
                 (*x1)[1] += f4v{b1.x, b1.y, b1.z, b1.w};
             }
