@@ -99,6 +99,58 @@ def test_module_output_and_all_gradients(case):
         assert_close("d " + name, prm.grad, params[name].grad, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("frozen", [(), ("k_weights", "v_bias"), ("input",)], ids=["all", "frozen_params", "frozen_input"])
+def test_shared_key_value_input_gradients(frozen):
+    """key is value (one tensor feeding two projections): its gradient is the sum of both projections' input gradients, with
+    any subset of the parameters or the input itself frozen."""
+    from torch_harmonics_amd import NeighborhoodAttentionS2
+
+    torch.manual_seed(SEED)
+    m = NeighborhoodAttentionS2(8, (12, 24), (6, 12), num_heads=2).to(DEV)
+    for name in frozen:
+        if name != "input":
+            getattr(m, name).requires_grad_(False)
+    xq, xkv, gout = torch.randn(2, 8, 6, 12), torch.randn(2, 8, 12, 24), torch.randn(2, 8, 6, 12)
+    dq_ = xq.clone().to(DEV).requires_grad_(True)
+    dkv = xkv.clone().to(DEV).requires_grad_("input" not in frozen)
+    m(dq_, dkv, dkv).backward(gout.to(DEV))
+    rq, rkv = xq.double().requires_grad_(True), xkv.double().requires_grad_(True)
+    ref, params = _reference_module_forward(m, rq, rkv, rkv)
+    ref.backward(gout.double())
+    tol = dict(rtol=1e-4, atol=2e-5)
+    assert_close("d query", dq_.grad, rq.grad, **tol)
+    if "input" in frozen:
+        assert dkv.grad is None
+    else:
+        assert_close("d key+value", dkv.grad, rkv.grad, **tol)
+    for name, prm in m.named_parameters():
+        if name in frozen:
+            assert prm.grad is None
+        else:
+            assert_close("d " + name, prm.grad, params[name].grad, rtol=1e-4, atol=1e-4)
+
+
+def test_self_attention_backward_under_autocast():
+    """Self-attention under bf16 autocast: the shared-input backward runs on bf16 gradients and hands back fp32 gradients."""
+    from torch_harmonics_amd import NeighborhoodAttentionS2
+
+    torch.manual_seed(SEED)
+    m = NeighborhoodAttentionS2(16, (12, 24), (12, 24), num_heads=1).to(DEV)
+    x = torch.randn(2, 16, 12, 24, device=DEV)
+    grads = []
+    for cast in (False, True):
+        xi = x.clone().requires_grad_(True)
+        m.zero_grad()
+        with torch.autocast("cuda", dtype=torch.bfloat16, enabled=cast):
+            out = m(xi)
+        out.float().square().sum().backward()
+        assert xi.grad.dtype == torch.float32 and m.k_weights.grad.dtype == torch.float32
+        grads.append([xi.grad.clone(), m.q_weights.grad.clone(), m.k_weights.grad.clone(), m.v_weights.grad.clone()])
+    for name, a, b in zip(("d input", "d q_weights", "d k_weights", "d v_weights"), grads[1], grads[0]):
+        scale = b.abs().max().item()
+        assert (a - b).abs().max().item() <= 6e-2 * scale, name
+
+
 def _small_module(nh=2, dtype=torch.float32):
     from torch_harmonics_amd import NeighborhoodAttentionS2
 

@@ -63,6 +63,46 @@ class _Linear1x1(torch.autograd.Function):
         return gx, gw, gb
 
 
+class _SharedInputLinear1x1(torch.autograd.Function):
+    """Several _Linear1x1 projections of ONE input (self-attention: q, k, v; cross-attention with key is value: k, v).  Forward
+    is one F.linear per projection; the backward accumulates the input gradient inside the GEMMs (beta = 1) instead of
+    leaving autograd to add up one full-size tensor per projection with elementwise kernels (two 2 GB adds at 721 x 1440,
+    256 channels)."""
+
+    @staticmethod
+    def forward(ctx, x, *params):  # params = (w0, b0, w1, b1, ...), biases may be None
+        weights, biases = params[0::2], params[1::2]
+        ctx.save_for_backward(x, *weights)
+        ctx.bias_dtypes = [None if b is None else b.dtype for b in biases]
+        return tuple(F.linear(x, w, b) for w, b in zip(weights, biases))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        x, *weights = ctx.saved_tensors
+        x2 = x.reshape(-1, x.shape[-1])
+        gx = None
+        out = []
+        for i, (g, w) in enumerate(zip(grads, weights)):
+            gw = gb = None
+            if g is not None:
+                g2 = g.reshape(-1, g.shape[-1])
+                if ctx.needs_input_grad[0]:
+                    if gx is None:
+                        gx = g2 @ w.to(g2.dtype)
+                    elif gx.dtype == g2.dtype:
+                        gx.addmm_(g2, w.to(g2.dtype))
+                    else:  # gradients of different dtypes (not produced by this module): plain accumulation
+                        gx = gx + (g2 @ w.to(g2.dtype)).to(gx.dtype)
+                if ctx.needs_input_grad[1 + 2 * i]:
+                    gw = _weight_grad(g2, x2.to(g2.dtype)).to(w.dtype)
+                if ctx.bias_dtypes[i] is not None and ctx.needs_input_grad[2 + 2 * i]:
+                    gb = g2.sum(0).to(ctx.bias_dtypes[i])
+            out += [gw, gb]
+        if gx is not None:
+            gx = gx.reshape(x.shape).to(x.dtype)
+        return (gx, *out)
+
+
 def _xavier_uniform(c_out: int, c_in: int, bound: float) -> nn.Parameter:
     return nn.Parameter(bound * (2 * torch.rand(c_out, c_in, 1, 1) - 1))
 
@@ -230,12 +270,20 @@ class NeighborhoodAttentionS2(nn.Module):
         # the softmax scale rides on the q projection (or on the q gain when the q/k RMS norm is on): no pass of its own
         normed = self.q_norm_weights is not None
         wq = self.q_weights.view(self.q_weights.shape[0], -1)
-        if normed:
-            query = _Linear1x1.apply(query, wq, self.q_bias)
+        bq = self.q_bias
+        if not normed:
+            wq, bq = wq * self.scale, None if bq is None else bq * self.scale
+        wk, wv = self.k_weights.view(self.k_weights.shape[0], -1), self.v_weights.view(self.v_weights.shape[0], -1)
+        # projections that share their input share one backward for the input gradient
+        if key_is_query and value_is_query:
+            query, key, value = _SharedInputLinear1x1.apply(query, wq, bq, wk, self.k_bias, wv, self.v_bias)
         else:
-            query = _Linear1x1.apply(query, wq * self.scale, None if self.q_bias is None else self.q_bias * self.scale)
-        key = _Linear1x1.apply(key, self.k_weights.view(self.k_weights.shape[0], -1), self.k_bias)
-        value = _Linear1x1.apply(value, self.v_weights.view(self.v_weights.shape[0], -1), self.v_bias)
+            query = _Linear1x1.apply(query, wq, bq)
+            if value_is_key:
+                key, value = _SharedInputLinear1x1.apply(key, wk, self.k_bias, wv, self.v_bias)
+            else:
+                key = _Linear1x1.apply(key, wk, self.k_bias)
+                value = _Linear1x1.apply(value, wv, self.v_bias)
 
         if normed:
             query = self._head_rms_norm(query, self.q_norm_weights, self.scale)
