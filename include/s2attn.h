@@ -232,6 +232,20 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
                                const int32_t *row_idx, const s2attn_ring_shape *shape, void *stream);
 
 /*
+ * Backward pass 2 of the gather direction on the transposed neighborhood: the same dk, dv as s2attn_ring_backward_pass2
+ * (attention_cuda_bwd_ring.cu:1312-1440) summed per chunk point in a fixed order and added to dk, dv without atomics.
+ * The caller supplies, once per psi and halo, the CSR entries regrouped by input latitude: for halo latitude r
+ * (global latitude lat_halo_start + r), entries t_off[r] .. t_off[r + 1] - 1 hold, for every CSR entry (row ho_local,
+ * col) with col / nlon_in == lat_halo_start + r and in CSR order, t_ho = ho_local and t_dlon = col mod nlon_in
+ * (a stable sort of the entries by col / nlon_in; t_off has nlat_halo + 1 entries).  Rows of latitudes outside the grid
+ * are empty.  The Python operator builds and caches these arrays on the device.
+ */
+int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                          const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                          const float *quad_weights, const int32_t *t_ho, const int32_t *t_dlon,
+                                          const int64_t *t_off, const s2attn_ring_shape *shape, void *stream);
+
+/*
  * The same three steps for the up-sampling (scatter) direction, nlon_out a multiple of nlon_in.  Replace
  * attention_kernels::forward_ring_step_upsample, backward_ring_step_upsample_pass1 / _pass2
  * (attention_interface.cpp:158-189; CUDA: attention_cuda_fwd_ring_upsample.cu:108-300,

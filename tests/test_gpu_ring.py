@@ -23,7 +23,7 @@ def _geo_dev(p):
 
 @pytest.mark.parametrize("case", RING_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
-def test_ring_steps_against_oracle_and_dense_attention(case, dtype):
+def test_ring_steps_against_oracle_and_dense_attention(case, dtype, monkeypatch):
     from torch_harmonics_amd import ops
 
     print(f"case {case} {dtype}", flush=True)
@@ -82,19 +82,23 @@ def test_ring_steps_against_oracle_and_dense_attention(case, dtype):
     assert_close("dq", dq.cpu(), q.grad[:, la : la + na, lo : lo + no], **tol)
 
     integral_norm = (bw["integral"] / st["alpha_sum"]).contiguous()
-    dk, dv = torch.zeros_like(p["k"]), torch.zeros_like(p["v"])
     h0, h1 = p["halo"]
-    for c in steps:
-        kc, vc = chunk_of(p, p["k"], c), chunk_of(p, p["v"], c)
-        dkc, dvc = torch.zeros(kc.shape, device=DEV), torch.zeros(vc.shape, device=DEV)
-        ops.backward_ring_step_pass2(
-            kc.to(DEV, dtype), vc.to(DEV, dtype), qd, gd, st["alpha_sum"], st["qdotk_max"], integral_norm, dkc, dvc, quad, col_l, roff_l, row_idx, *tail(c)
-        )
-        clo, chi = p["chunks"][c]
-        dk[:, h0:h1, clo:chi] += dkc.cpu()
-        dv[:, h0:h1, clo:chi] += dvc.cpu()
-    assert_close("dk", dk, k.grad, **tol)
-    assert_close("dv", dv, v.grad, **tol)
+    # pass 2 both ways: on the transposed neighborhood (what the operator runs) and straight from the CSR with atomics
+    for from_csr in (False, True):
+        monkeypatch.setattr(ops, "_RING_PASS2_FROM_CSR", from_csr)
+        dk, dv = torch.zeros_like(p["k"]), torch.zeros_like(p["v"])
+        for c in steps:
+            kc, vc = chunk_of(p, p["k"], c), chunk_of(p, p["v"], c)
+            # the step ADDS to what the arrays hold: start from a known non-zero content
+            dkc, dvc = torch.full(kc.shape, 0.5, device=DEV), torch.full(vc.shape, -0.25, device=DEV)
+            ops.backward_ring_step_pass2(
+                kc.to(DEV, dtype), vc.to(DEV, dtype), qd, gd, st["alpha_sum"], st["qdotk_max"], integral_norm, dkc, dvc, quad, col_l, roff_l, row_idx, *tail(c)
+            )
+            clo, chi = p["chunks"][c]
+            dk[:, h0:h1, clo:chi] += dkc.cpu() - 0.5
+            dv[:, h0:h1, clo:chi] += dvc.cpu() + 0.25
+        assert_close(f"dk (from_csr={from_csr})", dk, k.grad, **tol)
+        assert_close(f"dv (from_csr={from_csr})", dv, v.grad, **tol)
 
 
 def test_ring_ops_pass_opcheck_and_leave_state_alone_without_neighbors():

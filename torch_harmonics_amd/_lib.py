@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -93,6 +93,7 @@ SYMBOLS = {
     "s2attn_ring_forward_step": (_int, [_vp] * 10 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_backward_pass2_transposed": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_forward_step_upsample": (_int, [_vp] * 10 + [ctypes.POINTER(RingUpShapeStruct), _vp]),
     "s2attn_ring_backward_pass1_upsample": (_int, [_vp] * 11 + [ctypes.POINTER(RingUpShapeStruct), _vp]),
     "s2attn_ring_backward_pass2_upsample": (_int, [_vp] * 12 + [ctypes.POINTER(RingUpShapeStruct), _vp]),

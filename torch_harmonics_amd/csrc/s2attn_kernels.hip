@@ -49,7 +49,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 6; }
+extern "C" int s2attn_abi_version(void) { return 7; }
 
 namespace s2 {
 

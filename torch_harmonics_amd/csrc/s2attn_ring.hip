@@ -24,7 +24,7 @@
 namespace s2ring {
 
 constexpr int MAXC = 512;      // channels per (folded) head
-constexpr int NCI = MAXC / 64; // channels per lane
+constexpr int NCI = MAXC / 64; // channels per lane (up-sampling kernels: one wavefront per chunk cell)
 
 struct Args {
     const void *k, *v, *q, *dy;
@@ -34,6 +34,8 @@ struct Args {
     const float *quad_w;
     const int64_t *col_idx, *row_off;
     const int32_t *row_idx; // launch order of the output latitudes (may be null: natural order)
+    const int64_t *t_off;   // transposed neighborhood (pass 2): entries of halo latitude r are t_off[r] .. t_off[r + 1]
+    const int32_t *t_ho, *t_dlon;
     int B, nlat_halo, nlon_kx, Ho, Wo, ck, cv, nlon_in, pscale, lon_lo_kx, lat_halo_start;
 };
 
@@ -47,6 +49,283 @@ __device__ inline float wave_sum(float x)
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o);
     return x;
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// Gather direction.  A wavefront owns P = 64 / G consecutive output longitudes of one (batch, output latitude); the G
+// lanes of a point hold 8 consecutive channels each (G = 4 for up to 32 channels ... 64 for up to 512).  The wavefront
+// reads the CSR row 64 entries at a time, one entry per lane: the split of col into (latitude, longitude), the halo test
+// and a test whether ANY of the wavefront's points can see the entry in this chunk run once per entry in parallel; the
+// surviving entries are then taken U at a time by all points together (every point at its own shifted longitude, so the
+// P rows of K/V read for one entry are consecutive in memory), with U independent loads in flight per lane.
+// ---------------------------------------------------------------------------------------------------------------------
+constexpr int CPL = 8; // channels per lane
+
+template <int G> __device__ inline float group_sum(float x)
+{
+#pragma unroll
+    for (int o = G / 2; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    return x;
+}
+
+template <typename T> __device__ inline void unpack8(float (&x)[CPL], const T *p);
+template <> __device__ inline void unpack8<float>(float (&x)[CPL], const float *p)
+{
+    const float4 lo = reinterpret_cast<const float4 *>(p)[0], hi = reinterpret_cast<const float4 *>(p)[1];
+    x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
+}
+template <> __device__ inline void unpack8<__hip_bfloat16>(float (&x)[CPL], const __hip_bfloat16 *p)
+{
+    const uint4 r = *reinterpret_cast<const uint4 *>(p);
+    const unsigned w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) x[2 * i] = __uint_as_float(w[i] << 16), x[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+}
+template <> __device__ inline void unpack8<__half>(float (&x)[CPL], const __half *p)
+{
+    const uint4 r = *reinterpret_cast<const uint4 *>(p);
+    const unsigned w[4] = {r.x, r.y, r.z, r.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const __half2 h = *reinterpret_cast<const __half2 *>(&w[i]);
+        x[2 * i] = __low2float(h), x[2 * i + 1] = __high2float(h);
+    }
+}
+
+// channels c0 .. c0 + 7 of a row of n channels (zeros past the end); vec: n is a multiple of 8 and the row is 16-byte aligned
+template <typename T> __device__ inline void load8(float (&x)[CPL], const T *row, int c0, int n, bool vec)
+{
+    if (vec) {
+        if (c0 < n) {
+            unpack8(x, row + c0);
+        } else {
+#pragma unroll
+            for (int i = 0; i < CPL; i++) x[i] = 0.f;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < CPL; i++) x[i] = c0 + i < n ? ld(row + c0 + i) : 0.f;
+    }
+}
+
+__device__ inline void store8(float *row, const float (&x)[CPL], int c0, int n, bool vec)
+{
+    if (vec) {
+        if (c0 < n) {
+            reinterpret_cast<float4 *>(row + c0)[0] = make_float4(x[0], x[1], x[2], x[3]);
+            reinterpret_cast<float4 *>(row + c0)[1] = make_float4(x[4], x[5], x[6], x[7]);
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < CPL; i++)
+            if (c0 + i < n) row[c0 + i] = x[i];
+    }
+}
+
+// The wavefront's place: batch b, output latitude ho, first output longitude wo0 of its P points; this lane's point wo
+// (valid: inside the row) and first channel c0.  False past the end of the grid.
+template <int G> struct Place {
+    int b, ho, wo, c0, pw, pw0;
+    bool valid;
+    long out;
+    __device__ inline bool locate(const Args &a)
+    {
+        constexpr int P = 64 / G;
+        const int lane = threadIdx.x & 63;
+        const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+        const int nb = (a.Wo + P - 1) / P;
+        if (wid >= (long)a.B * a.Ho * nb) return false;
+        const int wb = (int)(wid % nb);
+        const int h = (int)((wid / nb) % a.Ho);
+        b = (int)(wid / ((long)nb * a.Ho));
+        ho = a.row_idx ? a.row_idx[h] : h;
+        const int w = wb * P + lane / G;
+        valid = w < a.Wo;
+        wo = valid ? w : a.Wo - 1;
+        c0 = (lane % G) * CPL;
+        pw = (int)(((long)a.pscale * wo) % a.nlon_in);
+        pw0 = (int)(((long)a.pscale * wb * P) % a.nlon_in);
+        out = ((long)b * a.Ho + ho) * a.Wo + wo;
+        return true;
+    }
+};
+
+// One CSR entry per lane: (longitude wi, chunk row base, quadrature weight) and whether any point of the wavefront can see it.
+template <int G> __device__ inline bool scan_entry(const Args &a, int64_t z, int64_t z1, int pw0, int &wi, int &rowbase, float &wq)
+{
+    constexpr int P = 64 / G;
+    wi = 0, rowbase = 0, wq = 0.f;
+    if (z >= z1) return false;
+    const int64_t col = a.col_idx[z];
+    int hi;
+    if ((uint64_t)col < 0x80000000ull) {
+        hi = (int)((uint32_t)col / (uint32_t)a.nlon_in);
+        wi = (int)((uint32_t)col - (uint32_t)hi * (uint32_t)a.nlon_in);
+    } else {
+        hi = (int)(col / a.nlon_in);
+        wi = (int)(col - (int64_t)hi * a.nlon_in);
+    }
+    const int hl = hi - a.lat_halo_start;
+    if (hl < 0 || hl >= a.nlat_halo) return false;
+    // first point's longitude relative to the chunk; the others follow at pscale apart, up to span further (cyclically)
+    int u = wi + pw0 - a.lon_lo_kx;
+    if (u < 0) u += a.nlon_in;
+    if (u >= a.nlon_in) u -= a.nlon_in;
+    const long span = (long)a.pscale * (P - 1);
+    if (!(u < a.nlon_kx || u + span >= a.nlon_in)) return false;
+    rowbase = hl * a.nlon_kx;
+    wq = a.quad_w[hi];
+    return true;
+}
+
+// chunk-local point of entry (wi, rowbase) for the lane's own output longitude, or -1
+__device__ inline int own_point(const Args &a, int wi, int rowbase, int pw, bool valid)
+{
+    int wip = wi + pw;
+    if (wip >= a.nlon_in) wip -= a.nlon_in;
+    const int rel = wip - a.lon_lo_kx;
+    return valid && (unsigned)rel < (unsigned)a.nlon_kx ? rowbase + rel : -1;
+}
+
+#define S2_RING_TAKE(u)                                                                                                  \
+    {                                                                                                                    \
+        const bool has = cand != 0;                                                                                      \
+        const int j = has ? __builtin_ctzll(cand) : 0;                                                                   \
+        cand &= cand - 1;                                                                                                \
+        const int wj = __builtin_amdgcn_readlane(wi, j), rj = __builtin_amdgcn_readlane(rowbase, j);                     \
+        wgt[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wq), j));                                       \
+        pt[u] = has ? own_point(a, wj, rj, pl.pw, pl.valid) : -1;                                                        \
+    }
+
+// Forward: folds the chunk into (y_acc, alpha_sum, qdotk_max).  attention_cuda_fwd_ring.cu:66-175.
+template <typename T, int G> __global__ __launch_bounds__(256) void fwd_kernel(const Args a, const bool vec)
+{
+    constexpr int U = 4;
+    Place<G> pl;
+    if (!pl.locate(a)) return;
+    const int lane = threadIdx.x & 63;
+    const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
+    const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
+    float qr[CPL], y[CPL];
+    load8(qr, static_cast<const T *>(a.q) + pl.out * a.ck, pl.c0, a.ck, vec);
+    load8(y, a.y_acc + pl.out * a.cv, pl.c0, a.cv, vec);
+    float S = a.alpha_sum[pl.out], m = a.qdotk_max[pl.out];
+    const int64_t z0 = a.row_off[pl.ho], z1 = a.row_off[pl.ho + 1];
+    for (int64_t zb = z0; zb < z1; zb += 64) {
+        int wi, rowbase;
+        float wq;
+        const bool ok = scan_entry<G>(a, zb + lane, z1, pl.pw0, wi, rowbase, wq);
+        unsigned long long cand = __ballot(ok);
+        while (cand) {
+            int pt[U];
+            float wgt[U], kk[U][CPL], vv[U][CPL], s[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) S2_RING_TAKE(u)
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const long p = pt[u] < 0 ? 0 : pt[u];
+                load8(kk[u], kx + p * a.ck, pl.c0, a.ck, vec);
+                load8(vv[u], vx + p * a.cv, pl.c0, a.cv, vec);
+            }
+            float mn = m;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float d = 0.f;
+#pragma unroll
+                for (int i = 0; i < CPL; i++) d = fmaf(qr[i], kk[u][i], d);
+                s[u] = group_sum<G>(d);
+                if (pt[u] >= 0) mn = fmaxf(mn, s[u]);
+            }
+            if (mn == -INFINITY) continue; // nothing seen yet, nothing in these entries (the condition is the same in a whole group)
+            const float corr = __expf(m - mn); // m = -inf before the first neighbor: 0
+            S *= corr;
+#pragma unroll
+            for (int i = 0; i < CPL; i++) y[i] *= corr;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float alpha = pt[u] >= 0 ? __expf(s[u] - mn) * wgt[u] : 0.f;
+                S += alpha;
+#pragma unroll
+                for (int i = 0; i < CPL; i++) y[i] = fmaf(alpha, vv[u][i], y[i]);
+            }
+            m = mn;
+        }
+    }
+    if (!pl.valid) return;
+    if (pl.c0 == 0) {
+        a.alpha_sum[pl.out] = S;
+        a.qdotk_max[pl.out] = m;
+    }
+    store8(a.y_acc + pl.out * a.cv, y, pl.c0, a.cv, vec);
+}
+
+// Backward pass 1: folds the chunk into (alpha_sum, qdotk_max, integral = sum alpha <dy, v>, alpha_k = sum alpha k,
+// alpha_kvw = sum alpha <dy, v> k).  attention_cuda_bwd_ring.cu:78-205.
+template <typename T, int G> __global__ __launch_bounds__(256) void pass1_kernel(const Args a, const bool vec)
+{
+    constexpr int U = 2;
+    Place<G> pl;
+    if (!pl.locate(a)) return;
+    const int lane = threadIdx.x & 63;
+    const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
+    const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
+    float qr[CPL], gr[CPL], ak[CPL], akg[CPL];
+    load8(qr, static_cast<const T *>(a.q) + pl.out * a.ck, pl.c0, a.ck, vec);
+    load8(gr, static_cast<const T *>(a.dy) + pl.out * a.cv, pl.c0, a.cv, vec);
+    load8(ak, a.alpha_k + pl.out * a.ck, pl.c0, a.ck, vec);
+    load8(akg, a.alpha_kvw + pl.out * a.ck, pl.c0, a.ck, vec);
+    float S = a.alpha_sum[pl.out], m = a.qdotk_max[pl.out], I = a.integral[pl.out];
+    const int64_t z0 = a.row_off[pl.ho], z1 = a.row_off[pl.ho + 1];
+    for (int64_t zb = z0; zb < z1; zb += 64) {
+        int wi, rowbase;
+        float wq;
+        const bool ok = scan_entry<G>(a, zb + lane, z1, pl.pw0, wi, rowbase, wq);
+        unsigned long long cand = __ballot(ok);
+        while (cand) {
+            int pt[U];
+            float wgt[U], kk[U][CPL], vv[U][CPL], s[U], gv[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) S2_RING_TAKE(u)
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const long p = pt[u] < 0 ? 0 : pt[u];
+                load8(kk[u], kx + p * a.ck, pl.c0, a.ck, vec);
+                load8(vv[u], vx + p * a.cv, pl.c0, a.cv, vec);
+            }
+            float mn = m;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float d = 0.f, e = 0.f;
+#pragma unroll
+                for (int i = 0; i < CPL; i++) d = fmaf(qr[i], kk[u][i], d), e = fmaf(gr[i], vv[u][i], e);
+                s[u] = group_sum<G>(d);
+                gv[u] = group_sum<G>(e);
+                if (pt[u] >= 0) mn = fmaxf(mn, s[u]);
+            }
+            if (mn == -INFINITY) continue;
+            const float corr = __expf(m - mn);
+            S *= corr, I *= corr;
+#pragma unroll
+            for (int i = 0; i < CPL; i++) ak[i] *= corr, akg[i] *= corr;
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const float alpha = pt[u] >= 0 ? __expf(s[u] - mn) * wgt[u] : 0.f;
+                const float ag = alpha * gv[u];
+                S += alpha, I += ag;
+#pragma unroll
+                for (int i = 0; i < CPL; i++) ak[i] = fmaf(alpha, kk[u][i], ak[i]), akg[i] = fmaf(ag, kk[u][i], akg[i]);
+            }
+            m = mn;
+        }
+    }
+    if (!pl.valid) return;
+    if (pl.c0 == 0) {
+        a.alpha_sum[pl.out] = S;
+        a.qdotk_max[pl.out] = m;
+        a.integral[pl.out] = I;
+    }
+    store8(a.alpha_k + pl.out * a.ck, ak, pl.c0, a.ck, vec);
+    store8(a.alpha_kvw + pl.out * a.ck, akg, pl.c0, a.ck, vec);
 }
 
 // output point of this wavefront; false past the end
@@ -74,124 +353,10 @@ __device__ inline long chunk_point(const Args &a, int64_t col, int wo, int &hi_g
     return (long)hi_local * a.nlon_kx + (wip - a.lon_lo_kx);
 }
 
-// Forward: folds the chunk into (y_acc, alpha_sum, qdotk_max).  attention_cuda_fwd_ring.cu:66-175.
-template <typename T> __global__ __launch_bounds__(256) void fwd_kernel(const Args a)
-{
-    int b, ho, wo, lane;
-    if (!locate(a, b, ho, wo, lane)) return;
-    const long out = ((long)b * a.Ho + ho) * a.Wo + wo;
-    const T *q = static_cast<const T *>(a.q) + out * a.ck;
-    const T *kx = static_cast<const T *>(a.k) + (long)b * a.nlat_halo * a.nlon_kx * a.ck;
-    const T *vx = static_cast<const T *>(a.v) + (long)b * a.nlat_halo * a.nlon_kx * a.cv;
-    float qr[NCI], y[NCI];
-#pragma unroll
-    for (int i = 0; i < NCI; i++) {
-        const int c = lane + 64 * i;
-        qr[i] = c < a.ck ? ld(q + c) : 0.f;
-        y[i] = c < a.cv ? a.y_acc[out * a.cv + c] : 0.f;
-    }
-    float S = a.alpha_sum[out], m = a.qdotk_max[out];
-    for (int64_t z = a.row_off[ho]; z < a.row_off[ho + 1]; z++) {
-        int hi;
-        const long pt = chunk_point(a, a.col_idx[z], wo, hi);
-        if (pt < 0) continue;
-        const T *kr = kx + pt * a.ck, *vr = vx + pt * a.cv;
-        float s = 0.f;
-#pragma unroll
-        for (int i = 0; i < NCI; i++) {
-            const int c = lane + 64 * i;
-            if (c < a.ck) s = fmaf(qr[i], ld(kr + c), s);
-        }
-        s = wave_sum(s);
-        const float mn = fmaxf(m, s);
-        const float alpha = __expf(s - mn) * a.quad_w[hi];
-        const float corr = __expf(m - mn); // m = -inf on the first neighbor: 0
-        S = alpha + S * corr;
-#pragma unroll
-        for (int i = 0; i < NCI; i++) {
-            const int c = lane + 64 * i;
-            if (c < a.cv) y[i] = fmaf(alpha, ld(vr + c), y[i] * corr);
-        }
-        m = mn;
-    }
-    if (lane == 0) {
-        a.alpha_sum[out] = S;
-        a.qdotk_max[out] = m;
-    }
-#pragma unroll
-    for (int i = 0; i < NCI; i++) {
-        const int c = lane + 64 * i;
-        if (c < a.cv) a.y_acc[out * a.cv + c] = y[i];
-    }
-}
-
-// Backward pass 1: folds the chunk into (alpha_sum, qdotk_max, integral = sum alpha <dy, v>, alpha_k = sum alpha k,
-// alpha_kvw = sum alpha <dy, v> k).  attention_cuda_bwd_ring.cu:78-205.
-template <typename T> __global__ __launch_bounds__(256) void pass1_kernel(const Args a)
-{
-    int b, ho, wo, lane;
-    if (!locate(a, b, ho, wo, lane)) return;
-    const long out = ((long)b * a.Ho + ho) * a.Wo + wo;
-    const T *q = static_cast<const T *>(a.q) + out * a.ck;
-    const T *g = static_cast<const T *>(a.dy) + out * a.cv;
-    const T *kx = static_cast<const T *>(a.k) + (long)b * a.nlat_halo * a.nlon_kx * a.ck;
-    const T *vx = static_cast<const T *>(a.v) + (long)b * a.nlat_halo * a.nlon_kx * a.cv;
-    float qr[NCI], gr[NCI], ak[NCI], akg[NCI];
-#pragma unroll
-    for (int i = 0; i < NCI; i++) {
-        const int c = lane + 64 * i;
-        qr[i] = c < a.ck ? ld(q + c) : 0.f;
-        gr[i] = c < a.cv ? ld(g + c) : 0.f;
-        ak[i] = c < a.ck ? a.alpha_k[out * a.ck + c] : 0.f;
-        akg[i] = c < a.ck ? a.alpha_kvw[out * a.ck + c] : 0.f;
-    }
-    float S = a.alpha_sum[out], m = a.qdotk_max[out], I = a.integral[out];
-    for (int64_t z = a.row_off[ho]; z < a.row_off[ho + 1]; z++) {
-        int hi;
-        const long pt = chunk_point(a, a.col_idx[z], wo, hi);
-        if (pt < 0) continue;
-        const T *kr = kx + pt * a.ck, *vr = vx + pt * a.cv;
-        float s = 0.f, gv = 0.f, kv[NCI];
-#pragma unroll
-        for (int i = 0; i < NCI; i++) {
-            const int c = lane + 64 * i;
-            kv[i] = c < a.ck ? ld(kr + c) : 0.f;
-            s = fmaf(qr[i], kv[i], s);
-            if (c < a.cv) gv = fmaf(gr[i], ld(vr + c), gv);
-        }
-        s = wave_sum(s);
-        gv = wave_sum(gv);
-        const float mn = fmaxf(m, s);
-        const float alpha = __expf(s - mn) * a.quad_w[hi];
-        const float corr = __expf(m - mn);
-        S = S * corr + alpha;
-        I = I * corr + alpha * gv;
-        const float ag = alpha * gv;
-#pragma unroll
-        for (int i = 0; i < NCI; i++) {
-            ak[i] = fmaf(alpha, kv[i], ak[i] * corr);
-            akg[i] = fmaf(ag, kv[i], akg[i] * corr);
-        }
-        m = mn;
-    }
-    if (lane == 0) {
-        a.alpha_sum[out] = S;
-        a.qdotk_max[out] = m;
-        a.integral[out] = I;
-    }
-#pragma unroll
-    for (int i = 0; i < NCI; i++) {
-        const int c = lane + 64 * i;
-        if (c < a.ck) {
-            a.alpha_k[out * a.ck + c] = ak[i];
-            a.alpha_kvw[out * a.ck + c] = akg[i];
-        }
-    }
-}
-
-// Backward pass 2: with the final statistics, adds this chunk's dk and dv (fp32, atomically: several output points
-// see the same input point).  attention_cuda_bwd_ring.cu:1312-1440.
-template <typename T> __global__ __launch_bounds__(256) void pass2_kernel(const Args a)
+// Backward pass 2 straight from the CSR, one wavefront per output point: with the final statistics, adds this chunk's dk and
+// dv with fp32 atomics (several output points see the same input point).  attention_cuda_bwd_ring.cu:1312-1440.
+// An atomic instruction of a wavefront covers one row of consecutive channels, the cheapest form for the L2.
+template <typename T> __global__ __launch_bounds__(256) void pass2_atomic_kernel(const Args a)
 {
     int b, ho, wo, lane;
     if (!locate(a, b, ho, wo, lane)) return;
@@ -234,6 +399,102 @@ template <typename T> __global__ __launch_bounds__(256) void pass2_kernel(const 
         }
     }
 }
+
+// Backward pass 2 on the TRANSPOSED neighborhood, no atomics: a wavefront owns P consecutive longitudes of one chunk row
+// (batch, input latitude) and walks the CSR entries that have this input latitude (t_off / t_ho / t_dlon: for every input
+// latitude of the halo, the (local output latitude, longitude offset col mod nlon_in) of those entries in CSR order).  The
+// output point of an entry for input longitude wg is wo = ((wg - dlon) mod nlon_in) / pscale when that division is exact
+// and wo is inside the local window.  dk and dv of a chunk point are summed in registers in a fixed order and added to the
+// caller's arrays once.  Same arithmetic as attention_cuda_bwd_ring.cu:1312-1440, loop order turned inside out.
+template <typename T, int G> __global__ __launch_bounds__(256) void pass2t_kernel(const Args a, const bool vec)
+{
+    constexpr int P = 64 / G, U = 2;
+    const int lane = threadIdx.x & 63;
+    const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+    const int nb = (a.nlon_kx + P - 1) / P;
+    if (wid >= (long)a.B * a.nlat_halo * nb) return;
+    const int wb = (int)(wid % nb);
+    const int hl = (int)((wid / nb) % a.nlat_halo);
+    const int b = (int)(wid / ((long)nb * a.nlat_halo));
+    const int64_t z0 = a.t_off[hl], z1 = a.t_off[hl + 1];
+    if (z0 >= z1) return; // nothing sees this latitude
+    const int w = wb * P + lane / G;
+    const bool valid = w < a.nlon_kx;
+    const int wl = valid ? w : a.nlon_kx - 1;
+    const int c0 = (lane % G) * CPL;
+    const long pt = ((long)b * a.nlat_halo + hl) * a.nlon_kx + wl;
+    float kr[CPL], vr[CPL], dk[CPL], dv[CPL];
+    load8(kr, static_cast<const T *>(a.k) + pt * a.ck, c0, a.ck, vec);
+    load8(vr, static_cast<const T *>(a.v) + pt * a.cv, c0, a.cv, vec);
+#pragma unroll
+    for (int i = 0; i < CPL; i++) dk[i] = dv[i] = 0.f;
+    const float wq = a.quad_w[a.lat_halo_start + hl];
+    const int wg = a.lon_lo_kx + wl, wg0 = a.lon_lo_kx + wb * P;
+    const long lim = (long)a.Wo * a.pscale;
+    const long obase = (long)b * a.Ho * a.Wo;
+    const T *__restrict__ qb = static_cast<const T *>(a.q) + obase * a.ck;
+    const T *__restrict__ gb = static_cast<const T *>(a.dy) + obase * a.cv;
+    for (int64_t zb = z0; zb < z1; zb += 64) {
+        const int64_t z = zb + lane;
+        int ho = 0, dl = 0;
+        bool ok = z < z1;
+        if (ok) {
+            ho = a.t_ho[z], dl = a.t_dlon[z];
+            int u = wg0 - dl; // first point's output longitude times pscale; the others follow one apart (cyclically)
+            if (u < 0) u += a.nlon_in;
+            ok = u < lim || u + (P - 1) >= a.nlon_in;
+        }
+        unsigned long long cand = __ballot(ok);
+        while (cand) {
+            long o[U];
+            bool in[U];
+            float qq[U][CPL], gg[U][CPL], S[U], m[U], In[U];
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const bool has = cand != 0;
+                const int j = has ? __builtin_ctzll(cand) : 0;
+                cand &= cand - 1;
+                const int hj = __builtin_amdgcn_readlane(ho, j), dj = __builtin_amdgcn_readlane(dl, j);
+                int t = wg - dj;
+                if (t < 0) t += a.nlon_in;
+                int wo = t;
+                bool exact = true;
+                if (a.pscale != 1) wo = t / a.pscale, exact = wo * a.pscale == t;
+                in[u] = has && valid && exact && wo < a.Wo;
+                o[u] = in[u] ? (long)hj * a.Wo + wo : 0;
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                load8(qq[u], qb + o[u] * a.ck, c0, a.ck, vec);
+                load8(gg[u], gb + o[u] * a.cv, c0, a.cv, vec);
+                S[u] = a.alpha_sum[obase + o[u]], m[u] = a.qdotk_max[obase + o[u]], In[u] = a.integral_norm[obase + o[u]];
+            }
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                float d = 0.f, e = 0.f;
+#pragma unroll
+                for (int i = 0; i < CPL; i++) d = fmaf(qq[u][i], kr[i], d), e = fmaf(gg[u][i], vr[i], e);
+                const float s = group_sum<G>(d), gv = group_sum<G>(e);
+                const float p = in[u] ? __expf(s - m[u]) * wq / S[u] : 0.f;
+                const float sk = in[u] ? (gv - In[u]) * p : 0.f;
+#pragma unroll
+                for (int i = 0; i < CPL; i++) dk[i] = fmaf(sk, qq[u][i], dk[i]), dv[i] = fmaf(p, gg[u][i], dv[i]);
+            }
+        }
+    }
+    if (!valid) return;
+    float cur[CPL];
+    load8(cur, a.dk + pt * a.ck, c0, a.ck, vec);
+#pragma unroll
+    for (int i = 0; i < CPL; i++) cur[i] += dk[i];
+    store8(a.dk + pt * a.ck, cur, c0, a.ck, vec);
+    load8(cur, a.dv + pt * a.cv, c0, a.cv, vec);
+#pragma unroll
+    for (int i = 0; i < CPL; i++) cur[i] += dv[i];
+    store8(a.dv + pt * a.cv, cur, c0, a.cv, vec);
+}
+
+#undef S2_RING_TAKE
 
 // ---------------------------------------------------------------------------------------------------------------------
 // Up-sampling (scatter) direction.  psi is keyed by the chunk's LOCAL input latitude hi_local (row_off has nlat_halo + 1
@@ -471,18 +732,44 @@ void fill(Args &a, const s2attn_ring_shape *sh)
     a.lat_halo_start = sh->lat_halo_start;
 }
 
-enum Step { FWD, PASS1, PASS2 };
+enum Step { FWD, PASS1, PASS2, PASS2T };
 
-template <typename T> int launch_t(Step step, const Args &a, hipStream_t stream)
+template <typename T, int G> int launch_g(Step step, const Args &a, hipStream_t stream)
 {
-    const long npts = (long)a.B * a.Ho * a.Wo;
-    const long nblocks = (npts + 3) / 4;
+    constexpr int P = 64 / G;
+    const long nwaves = step == PASS2T ? (long)a.B * a.nlat_halo * ((a.nlon_kx + P - 1) / P) : (long)a.B * a.Ho * ((a.Wo + P - 1) / P);
+    const long nblocks = (nwaves + 3) / 4;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    void (*kern)(const Args) = step == FWD ? fwd_kernel<T> : step == PASS1 ? pass1_kernel<T> : pass2_kernel<T>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
+    if ((long)a.nlat_halo * a.nlon_kx > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "chunk of more than 2^31 points");
+    // 16-byte rows: vector loads and stores
+    auto al = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+    bool vec = a.ck % CPL == 0 && a.cv % CPL == 0 && al(a.k) && al(a.v) && al(a.q);
+    if (step == FWD) vec = vec && al(a.y_acc);
+    if (step == PASS1) vec = vec && al(a.dy) && al(a.alpha_k) && al(a.alpha_kvw);
+    if (step == PASS2T) vec = vec && al(a.dy) && al(a.dk) && al(a.dv);
+    void (*kern)(const Args, const bool) = step == FWD ? fwd_kernel<T, G> : step == PASS1 ? pass1_kernel<T, G> : pass2t_kernel<T, G>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), 0, stream, a, vec);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
+}
+
+template <typename T> int launch_t(Step step, const Args &a, hipStream_t stream)
+{
+    if (step == PASS2) { // one wavefront per output point
+        const long nblocks = ((long)a.B * a.Ho * a.Wo + 3) / 4;
+        if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+        hipLaunchKernelGGL(pass2_atomic_kernel<T>, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+        return S2ATTN_OK;
+    }
+    const int c = a.ck > a.cv ? a.ck : a.cv; // lanes per point: 8 channels each
+    if (c <= 32) return launch_g<T, 4>(step, a, stream);
+    if (c <= 64) return launch_g<T, 8>(step, a, stream);
+    if (c <= 128) return launch_g<T, 16>(step, a, stream);
+    if (c <= 256) return launch_g<T, 32>(step, a, stream);
+    return launch_g<T, 64>(step, a, stream);
 }
 
 int launch(Step step, const Args &a, int dtype, void *stream)
@@ -543,6 +830,24 @@ extern "C" int s2attn_ring_backward_pass2(const void *k, const void *v, const vo
     a.dk = dk, a.dv = dv;
     a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off, a.row_idx = row_idx;
     return launch(PASS2, a, shape->dtype, stream);
+}
+
+extern "C" int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                                     const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                                     const float *quad_weights, const int32_t *t_ho, const int32_t *t_dlon,
+                                                     const int64_t *t_off, const s2attn_ring_shape *shape, void *stream)
+{
+    const int rc = check(shape);
+    if (rc != S2ATTN_OK) return rc;
+    if (!k || !v || !q || !dy || !alpha_sum || !qdotk_max || !integral_norm || !dk || !dv || !quad_weights || !t_ho || !t_dlon || !t_off)
+        return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    Args a = {};
+    fill(a, shape);
+    a.k = k, a.v = v, a.q = q, a.dy = dy;
+    a.alpha_sum = const_cast<float *>(alpha_sum), a.qdotk_max = const_cast<float *>(qdotk_max), a.integral_norm = integral_norm;
+    a.dk = dk, a.dv = dv;
+    a.quad_w = quad_weights, a.t_ho = t_ho, a.t_dlon = t_dlon, a.t_off = t_off;
+    return launch(PASS2T, a, shape->dtype, stream);
 }
 
 namespace {

@@ -23,7 +23,7 @@ import torch
 
 from . import _lib
 from ._attention_utils import _setup_context_attention_backward
-from .plan import get_plan
+from .plan import get_plan, get_transposed_csr
 
 _DTYPE_CODE = {torch.float32: _lib.S2ATTN_F32, torch.bfloat16: _lib.S2ATTN_BF16, torch.float16: _lib.S2ATTN_F16}
 
@@ -553,6 +553,11 @@ def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_buf, alpha_k_buf, a
     return None
 
 
+# Pass 2 runs on the transposed neighborhood (sums in registers, fixed order); True selects the library's other entry point,
+# which walks the CSR as given and adds with fp32 atomics (the reference's formulation), for comparison and tests.
+_RING_PASS2_FROM_CSR = False
+
+
 @torch.library.custom_op("s2attn::backward_ring_step_pass2", mutates_args=("dkx", "dvx"))
 def backward_ring_step_pass2(
     kx: torch.Tensor,
@@ -584,15 +589,17 @@ def backward_ring_step_pass2(
         if t.shape != like.shape or t.dtype != torch.float32 or not t.is_contiguous():
             raise RuntimeError(f"{name} must be a contiguous fp32 tensor shaped like its input, {tuple(like.shape)}")
         _require_gpu(t, name, kx.device)
-    if qy.numel() == 0 or kx.numel() == 0:
+    if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:
         return
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    head = (kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+            integral_norm_buf.data_ptr(), dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr())  # fmt: skip
     with torch.cuda.device(kx.device):
-        rc = _lib.load().s2attn_ring_backward_pass2(
-            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
-            integral_norm_buf.data_ptr(), dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(),
-            row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
-        )  # fmt: skip
+        if _RING_PASS2_FROM_CSR:
+            rc = _lib.load().s2attn_ring_backward_pass2(*head, col_idx.data_ptr(), row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
+        else:
+            t_ho, t_dlon, t_off = get_transposed_csr(col_idx, row_off, nlon_in, lat_halo_start, kx.shape[1])
+            rc = _lib.load().s2attn_ring_backward_pass2_transposed(*head, t_ho.data_ptr(), t_dlon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
     _lib.check(rc, "s2attn_ring_backward_pass2")
 
 

@@ -108,6 +108,36 @@ def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in
     return plan
 
 
+def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, nlon_in: int, lat_halo_start: int, nlat_halo: int):
+    """
+    The CSR entries regrouped by input latitude, for the ring-step backward pass 2: (t_ho int32, t_dlon int32, t_off int64
+    of nlat_halo + 1 entries) with the entries of halo latitude r (global lat_halo_start + r) at t_off[r] .. t_off[r + 1],
+    in CSR order, as (local output latitude, col mod nlon_in).  Built with device operations only (no host round trip) the
+    first time a (psi, halo) is seen, then served from the same cache as the plans.
+    """
+    key = ("transposed", col_idx.data_ptr(), row_off.data_ptr(), col_idx.numel(), row_off.numel(), col_idx._version, row_off._version,
+           str(col_idx.device), nlon_in, lat_halo_start, nlat_halo)  # fmt: skip
+    with _lock:
+        hit = _cache.get(key)
+        if hit is not None:
+            _cache.move_to_end(key)
+            return hit[:3]
+    dev, nnz, nrow = col_idx.device, col_idx.numel(), row_off.numel() - 1
+    ho = torch.repeat_interleave(torch.arange(nrow, device=dev, dtype=torch.int32), row_off[1:] - row_off[:-1], output_size=nnz)
+    hi = torch.div(col_idx, nlon_in, rounding_mode="floor")
+    order = torch.argsort(hi, stable=True)
+    hi_sorted = hi[order]
+    t_ho = ho[order].contiguous()
+    t_dlon = (col_idx - hi * nlon_in)[order].to(torch.int32).contiguous()
+    t_off = torch.searchsorted(hi_sorted, torch.arange(lat_halo_start, lat_halo_start + nlat_halo + 1, device=dev, dtype=hi.dtype)).contiguous()
+    entry = (t_ho, t_dlon, t_off, (col_idx, row_off))  # the CSR tensors stay alive with the entry: their addresses cannot be recycled
+    with _lock:
+        _cache[key] = entry
+        while len(_cache) > _MAX_ENTRIES:
+            _cache.popitem(last=False)
+    return entry[:3]
+
+
 def clear_plan_cache() -> None:
     with _lock:
         _cache.clear()
