@@ -232,17 +232,22 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
                                const int32_t *row_idx, const s2attn_ring_shape *shape, void *stream);
 
 /*
- * Backward pass 2 of the gather direction on the transposed neighborhood: the same dk, dv as s2attn_ring_backward_pass2
- * (attention_cuda_bwd_ring.cu:1312-1440) summed per chunk point in a fixed order and added to dk, dv without atomics.
- * The caller supplies, once per psi and halo, the CSR entries regrouped by input latitude: for halo latitude r
- * (global latitude lat_halo_start + r), entries t_off[r] .. t_off[r + 1] - 1 hold, for every CSR entry (row ho_local,
- * col) with col / nlon_in == lat_halo_start + r and in CSR order, t_ho = ho_local and t_dlon = col mod nlon_in
- * (a stable sort of the entries by col / nlon_in; t_off has nlat_halo + 1 entries).  Rows of latitudes outside the grid
- * are empty.  The Python operator builds and caches these arrays on the device.
+ * Regrouped psi.  Every ring kernel of this library is a gather: the cell that owns a sum walks the entries of its own
+ * latitude.  Where psi is keyed by the other grid, the caller supplies, once per psi, the CSR entries regrouped by
+ * the owner's latitude -- a STABLE sort of the entries (row r, col) by key = col / modulus:
+ *   t_off[i]  (int64, nkeys + 1 entries)  entries of key key_lo + i are t_off[i] .. t_off[i + 1] - 1, in CSR order
+ *   t_lat[z]  (int32)                     the entry's CSR row r (the partner's local latitude)
+ *   t_lon[z]  (int32)                     col mod modulus
+ * Keys outside [key_lo, key_lo + nkeys) are left out.  The Python operators build these arrays with device operations
+ * and cache them per psi.
+ *
+ * Backward pass 2 of the gather direction on the regrouped psi (modulus nlon_in, key_lo = lat_halo_start, nkeys =
+ * nlat_halo; t_lat = local output latitude): the same dk, dv as s2attn_ring_backward_pass2
+ * (attention_cuda_bwd_ring.cu:1312-1440), summed per chunk point in a fixed order and added to dk, dv without atomics.
  */
 int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                           const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
-                                          const float *quad_weights, const int32_t *t_ho, const int32_t *t_dlon,
+                                          const float *quad_weights, const int32_t *t_lat, const int32_t *t_lon,
                                           const int64_t *t_off, const s2attn_ring_shape *shape, void *stream);
 
 /*
@@ -251,10 +256,12 @@ int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const vo
  * (attention_interface.cpp:158-189; CUDA: attention_cuda_fwd_ring_upsample.cu:108-300,
  * attention_cuda_bwd_ring_upsample.cu:88-240).  psi is keyed by the chunk's LOCAL input latitude: row_off has
  * nlat_halo + 1 entries (empty rows for pole padding), col_idx = ho_local * nlon_out_global + wo_shifted with
- * wo_shifted = (wo - first local output longitude) mod nlon_out_global.  The forward step runs three phases (scatter the
- * chunk's maxima into max_scratch, rescale the state, scatter the sums with fp32 atomics); max_scratch is caller-owned
- * scratch of batch * nlat_out * nlon_out floats.  Pass 1 needs the forward's FINAL qdotk_max and adds into integral,
- * alpha_k, alpha_kvw atomically; pass 2 WRITES the chunk's dk and dv (every element, no atomics).
+ * wo_shifted = (wo - first local output longitude) mod nlon_out_global.  The reference's forward scatters in three
+ * phases (maxima, rescale, sums) with atomics; here the forward step and pass 1 gather per OUTPUT cell over psi regrouped
+ * by output latitude (modulus nlon_out_global, key_lo = 0, nkeys = nlat_out; t_lat = local input latitude), with the
+ * running maximum kept per cell: same state after every step, no scratch, no atomics.  Pass 1 needs the forward's FINAL
+ * qdotk_max and adds into integral, alpha_k, alpha_kvw; pass 2 takes psi as given and WRITES the chunk's dk and dv
+ * (every element).
  */
 typedef struct s2attn_ring_up_shape {
     int32_t batch, nlat_halo, nlon_kx, nlat_out, nlon_out; /* as s2attn_ring_shape; nlon_out is the LOCAL output width */
@@ -263,18 +270,18 @@ typedef struct s2attn_ring_up_shape {
     int32_t pscale_out;      /* global nlon_out / global nlon_in */
     int32_t lon_lo_kx;       /* first global input longitude of the chunk */
     int32_t lat_halo_start;  /* global input latitude of the chunk's row 0 (quadrature weight index; may be negative when
-                                the halo is padded past the pole: such rows must be empty in row_off) */
+                                the halo is padded past the pole: such rows must be empty in psi) */
     int32_t dtype;
 } s2attn_ring_up_shape;
 
 int s2attn_ring_forward_step_upsample(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
-                                      float *max_scratch, const float *quad_weights, const int64_t *col_idx,
-                                      const int64_t *row_off, const s2attn_ring_up_shape *shape, void *stream);
+                                      const float *quad_weights, const int32_t *t_lat, const int32_t *t_lon, const int64_t *t_off,
+                                      const s2attn_ring_up_shape *shape, void *stream);
 
 int s2attn_ring_backward_pass1_upsample(const void *k, const void *v, const void *q, const void *dy, const float *qdotk_max,
                                         float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
-                                        const int64_t *col_idx, const int64_t *row_off, const s2attn_ring_up_shape *shape,
-                                        void *stream);
+                                        const int32_t *t_lat, const int32_t *t_lon, const int64_t *t_off,
+                                        const s2attn_ring_up_shape *shape, void *stream);
 
 int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                         const float *qdotk_max, const float *integral_norm, float *dk, float *dv,

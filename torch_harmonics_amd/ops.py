@@ -598,8 +598,8 @@ def backward_ring_step_pass2(
         if _RING_PASS2_FROM_CSR:
             rc = _lib.load().s2attn_ring_backward_pass2(*head, col_idx.data_ptr(), row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
         else:
-            t_ho, t_dlon, t_off = get_transposed_csr(col_idx, row_off, nlon_in, lat_halo_start, kx.shape[1])
-            rc = _lib.load().s2attn_ring_backward_pass2_transposed(*head, t_ho.data_ptr(), t_dlon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
+            t_lat, t_lon, t_off = get_transposed_csr(col_idx, row_off, nlon_in, lat_halo_start, kx.shape[1])  # psi regrouped by input latitude
+            rc = _lib.load().s2attn_ring_backward_pass2_transposed(*head, t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
     _lib.check(rc, "s2attn_ring_backward_pass2")
 
 
@@ -639,14 +639,14 @@ def forward_ring_step_upsample(
 ) -> None:
     state = (("y_acc", y_acc, vx.shape[3]), ("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None))
     _ring_up_validate(kx, vx, qy, None, state, quad_weights, col_idx, row_off, nlat_out, nlon_out)
-    if qy.numel() == 0 or kx.numel() == 0:
+    if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
-    scratch = torch.empty_like(qdotk_max_buf)
     with torch.cuda.device(kx.device):
+        t_lat, t_lon, t_off = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)  # psi regrouped by output latitude
         rc = _lib.load().s2attn_ring_forward_step_upsample(
-            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(), scratch.data_ptr(),
-            quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+            kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+            quad_weights.data_ptr(), t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
         )  # fmt: skip
     _lib.check(rc, "s2attn_ring_forward_step_upsample")
 
@@ -680,13 +680,14 @@ def backward_ring_step_upsample_pass1(
     ck = kx.shape[3]
     state = (("qdotk_max_buf", qdotk_max_buf, None), ("integral_buf", integral_buf, None), ("alpha_k_buf", alpha_k_buf, ck), ("alpha_kvw_buf", alpha_kvw_buf, ck))
     _ring_up_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, nlat_out, nlon_out)
-    if qy.numel() == 0 or kx.numel() == 0:
+    if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
     with torch.cuda.device(kx.device):
+        t_lat, t_lon, t_off = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)
         rc = _lib.load().s2attn_ring_backward_pass1_upsample(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), qdotk_max_buf.data_ptr(), integral_buf.data_ptr(), alpha_k_buf.data_ptr(),
-            alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+            alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(), t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
         )  # fmt: skip
     _lib.check(rc, "s2attn_ring_backward_pass1_upsample")
 

@@ -108,29 +108,29 @@ def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in
     return plan
 
 
-def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, nlon_in: int, lat_halo_start: int, nlat_halo: int):
+def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, modulus: int, key_lo: int, nkeys: int):
     """
-    The CSR entries regrouped by input latitude, for the ring-step backward pass 2: (t_ho int32, t_dlon int32, t_off int64
-    of nlat_halo + 1 entries) with the entries of halo latitude r (global lat_halo_start + r) at t_off[r] .. t_off[r + 1],
-    in CSR order, as (local output latitude, col mod nlon_in).  Built with device operations only (no host round trip) the
-    first time a (psi, halo) is seen, then served from the same cache as the plans.
+    The CSR entries regrouped by key = col // modulus (the latitude named in col), for the ring-step kernels that gather
+    over the grid psi is not keyed by: (t_lat int32, t_lon int32, t_off int64 of nkeys + 1 entries) with the entries of
+    key key_lo + i at t_off[i] .. t_off[i + 1], in CSR order, as (CSR row of the entry, col mod modulus); see
+    include/s2attn.h.  Built with device operations only (no host round trip) the first time a psi is seen, then served
+    from the same cache as the plans.
     """
     key = ("transposed", col_idx.data_ptr(), row_off.data_ptr(), col_idx.numel(), row_off.numel(), col_idx._version, row_off._version,
-           str(col_idx.device), nlon_in, lat_halo_start, nlat_halo)  # fmt: skip
+           str(col_idx.device), modulus, key_lo, nkeys)  # fmt: skip
     with _lock:
         hit = _cache.get(key)
         if hit is not None:
             _cache.move_to_end(key)
             return hit[:3]
     dev, nnz, nrow = col_idx.device, col_idx.numel(), row_off.numel() - 1
-    ho = torch.repeat_interleave(torch.arange(nrow, device=dev, dtype=torch.int32), row_off[1:] - row_off[:-1], output_size=nnz)
-    hi = torch.div(col_idx, nlon_in, rounding_mode="floor")
-    order = torch.argsort(hi, stable=True)
-    hi_sorted = hi[order]
-    t_ho = ho[order].contiguous()
-    t_dlon = (col_idx - hi * nlon_in)[order].to(torch.int32).contiguous()
-    t_off = torch.searchsorted(hi_sorted, torch.arange(lat_halo_start, lat_halo_start + nlat_halo + 1, device=dev, dtype=hi.dtype)).contiguous()
-    entry = (t_ho, t_dlon, t_off, (col_idx, row_off))  # the CSR tensors stay alive with the entry: their addresses cannot be recycled
+    rows = torch.repeat_interleave(torch.arange(nrow, device=dev, dtype=torch.int32), row_off[1:] - row_off[:-1], output_size=nnz)
+    lat = torch.div(col_idx, modulus, rounding_mode="floor")
+    order = torch.argsort(lat, stable=True)
+    t_lat = rows[order].contiguous()
+    t_lon = (col_idx - lat * modulus)[order].to(torch.int32).contiguous()
+    t_off = torch.searchsorted(lat[order], torch.arange(key_lo, key_lo + nkeys + 1, device=dev, dtype=lat.dtype)).contiguous()
+    entry = (t_lat, t_lon, t_off, (col_idx, row_off))  # the CSR tensors stay alive with the entry: their addresses cannot be recycled
     with _lock:
         _cache[key] = entry
         while len(_cache) > _MAX_ENTRIES:
