@@ -50,6 +50,7 @@ struct Args {
     const int32_t *t_lat, *t_lon;     //   (partner's local latitude, off)
     int B, nlat_halo, nlon_kx, Ho, Wo, ck, cv;
     int N, scale, win_lo, win_n; // longitude relation, see the top of the file
+    int M, win_q;                // N / scale and win_n / scale (regrouped psi: the relation in partner units)
     int lat_off;                 // as given: partner's local latitude = col / N - lat_off
     int lat_halo_start;          // global input latitude of the chunk's row 0 (quadrature weights)
     int lon_lo_kx;               // first global input longitude of the chunk
@@ -130,23 +131,25 @@ __device__ inline void store8(float *row, const float (&x)[CPL], int c0, int n, 
     }
 }
 
-// The wavefront's place on a grid of nrow x ncol cells per batch: P consecutive longitudes of one row.
+// The wavefront's place on a grid of nrow x ncol cells per batch: P longitudes of one row, `stride` apart (the regrouped
+// relation only joins cells of one residue class modulo scale with an entry, so a wavefront takes its cells from one class).
 template <int G> struct Place {
     int b, row, x, x0, c0; // batch, latitude (after the launch order), this lane's longitude (clamped), the first one, first channel
     bool valid;            // the lane's longitude is inside the row
-    __device__ inline bool locate(int B, int nrow, int ncol, const int32_t *order)
+    static __host__ __device__ inline long blocks_per_row(int ncol, int stride) { return (long)stride * (((ncol + stride - 1) / stride + 64 / G - 1) / (64 / G)); }
+    __device__ inline bool locate(int B, int nrow, int ncol, const int32_t *order, int stride)
     {
         constexpr int P = 64 / G;
         const int lane = threadIdx.x & 63;
         const long wid = (long)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
-        const int nb = (ncol + P - 1) / P;
+        const int nb = (int)blocks_per_row(ncol, stride);
         if (wid >= (long)B * nrow * nb) return false;
         const int wb = (int)(wid % nb);
         const int h = (int)((wid / nb) % nrow);
         b = (int)(wid / ((long)nb * nrow));
         row = order ? order[h] : h;
-        x0 = wb * P;
-        const int w = x0 + lane / G;
+        x0 = wb % stride + stride * ((wb / stride) * P);
+        const int w = x0 + stride * (lane / G);
         valid = w < ncol;
         x = valid ? w : ncol - 1;
         c0 = (lane % G) * CPL;
@@ -164,13 +167,19 @@ template <int G, bool TR> __device__ inline bool scan_entry(const Args &a, int64
     off = 0, rowbase = 0, lat = 0;
     if (z >= z1) return false;
     if constexpr (TR) {
-        lat = a.t_lat[z], off = a.t_lon[z];
+        lat = a.t_lat[z];
         if (lat < 0 || lat >= nlat2) return false;
-        int t = x0 - off; // first cell; the others follow one apart (cyclically)
+        int t = x0 - a.t_lon[z]; // first cell; the others follow at scale apart (cyclically): one apart in partner units
         if (t < 0) t += a.N;
         int u = t - a.win_lo;
         if (u < 0) u += a.N;
-        if (!(u < a.win_n || u + (P - 1) >= a.N)) return false;
+        int q = u;
+        if (a.scale != 1) {
+            q = u / a.scale;
+            if (q * a.scale != u) return false; // this residue class never meets the entry
+        }
+        if (!(q < a.win_q || q + (P - 1) >= a.M)) return false;
+        off = q; // the first cell's partner longitude relative to the window
         rowbase = lat * pwidth;
     } else {
         const int64_t col = a.col_idx[z];
@@ -193,17 +202,14 @@ template <int G, bool TR> __device__ inline bool scan_entry(const Args &a, int64
     return true;
 }
 
-// partner cell of entry (off, rowbase) for the lane's own longitude (TR: x; as given: sx = scale * x mod N), or -1
+// partner cell of entry (off, rowbase) for the lane's own cell, or -1.  Regrouped: x = the cell's index in the wavefront,
+// off = the first cell's partner longitude relative to the window.  As given: x = scale * longitude mod N.
 template <bool TR> __device__ inline int partner(const Args &a, int off, int rowbase, int x, bool valid)
 {
     if constexpr (TR) {
-        int t = x - off;
-        if (t < 0) t += a.N;
-        const int rel = t - a.win_lo;
-        if (!valid || rel < 0 || rel >= a.win_n) return -1;
-        if (a.scale == 1) return rowbase + rel;
-        const int q = rel / a.scale;
-        return q * a.scale == rel ? rowbase + q : -1;
+        int r = off + x;
+        if (r >= a.M) r -= a.M;
+        return valid && r < a.win_q ? rowbase + r : -1;
     } else {
         int p = off + x;
         if (p >= a.N) p -= a.N;
@@ -243,10 +249,10 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd
 {
     constexpr int U = 4;
     Place<G> pl;
-    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx)) return;
+    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1)) return;
     const int lane = threadIdx.x & 63;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
-    const int xs = TR ? pl.x : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
+    const int xs = TR ? lane / G : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
     const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
     const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
     float qr[CPL], y[CPL];
@@ -310,10 +316,10 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx)) return;
+    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1)) return;
     const int lane = threadIdx.x & 63;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
-    const int xs = TR ? pl.x : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
+    const int xs = TR ? lane / G : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
     const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
     const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
     float qr[CPL], gr[CPL], ak[CPL], akg[CPL];
@@ -389,7 +395,7 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, nullptr)) return;
+    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, nullptr, TR ? a.scale : 1)) return;
     const int lane = threadIdx.x & 63;
     int64_t z0, z1;
     entry_range<TR>(a, pl.row, z0, z1);
@@ -403,7 +409,7 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
     for (int i = 0; i < CPL; i++) dk[i] = dv[i] = 0.f;
     const float wq = z0 < z1 ? a.quad_w[a.lat_halo_start + pl.row] : 0.f; // a padded row outside the grid has no entries and no weight
     const int gx = a.lon_lo_kx + pl.x, gx0 = a.lon_lo_kx + pl.x0;           // global input longitudes
-    const int xs = TR ? gx : (int)(((long)a.scale * gx) % a.N), xs0 = TR ? gx0 : (int)(((long)a.scale * gx0) % a.N);
+    const int xs = TR ? lane / G : (int)(((long)a.scale * gx) % a.N), xs0 = TR ? gx0 : (int)(((long)a.scale * gx0) % a.N);
     const long obase = (long)pl.b * a.Ho * a.Wo;
     const T *__restrict__ qb = static_cast<const T *>(a.q) + obase * a.ck;
     const T *__restrict__ gb = static_cast<const T *>(a.dy) + obase * a.cv;
@@ -542,7 +548,8 @@ int check(const s2attn_ring_shape *sh)
     if (sh->ck < 1 || sh->cv < 1) return s2attn_fail(S2ATTN_E_INVALID, "channel counts must be positive");
     if (sh->ck > MAXC || sh->cv > MAXC)
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "channels above %d are not instantiated (ck=%d, cv=%d)", MAXC, sh->ck, sh->cv);
-    if (sh->pscale < 1) return s2attn_fail(S2ATTN_E_INVALID, "pscale must be positive, got %d", sh->pscale);
+    if (sh->pscale < 1 || sh->nlon_in % sh->pscale != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "pscale must be a positive divisor of nlon_in = %d, got %d", sh->nlon_in, sh->pscale);
     if (sh->lon_lo_kx < 0 || sh->lon_lo_kx + sh->nlon_kx > sh->nlon_in)
         return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", sh->lon_lo_kx, sh->lon_lo_kx + sh->nlon_kx, sh->nlon_in);
     if ((int64_t)sh->pscale * sh->nlon_out > sh->nlon_in)
@@ -562,6 +569,7 @@ void fill(Args &a, const s2attn_ring_shape *sh, bool transposed)
         a.win_lo = 0, a.win_n = sh->pscale * sh->nlon_out;
     else
         a.win_lo = sh->lon_lo_kx, a.win_n = sh->nlon_kx;
+    a.M = a.N / a.scale, a.win_q = a.win_n / a.scale;
 }
 
 enum Step { FWD, PASS1, PASS2 };
@@ -569,7 +577,9 @@ enum Step { FWD, PASS1, PASS2 };
 template <typename T, int G, bool TR> int launch_g(Step step, const Args &a, hipStream_t stream)
 {
     constexpr int P = 64 / G;
-    const long nwaves = step == PASS2 ? (long)a.B * a.nlat_halo * ((a.nlon_kx + P - 1) / P) : (long)a.B * a.Ho * ((a.Wo + P - 1) / P);
+    const int stride = TR ? a.scale : 1;
+    const long nwaves = step == PASS2 ? (long)a.B * a.nlat_halo * Place<G>::blocks_per_row(a.nlon_kx, stride) : (long)a.B * a.Ho * Place<G>::blocks_per_row(a.Wo, stride);
+    (void)P;
     const long nblocks = (nwaves + 3) / 4;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
     if ((long)a.nlat_halo * a.nlon_kx > 0x7fffffffL || (long)a.Ho * a.Wo > 0x7fffffffL)
@@ -698,8 +708,8 @@ int check_up(const s2attn_ring_up_shape *sh)
     if (sh->ck < 1 || sh->cv < 1) return s2attn_fail(S2ATTN_E_INVALID, "channel counts must be positive");
     if (sh->ck > MAXC || sh->cv > MAXC)
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "channels above %d are not instantiated (ck=%d, cv=%d)", MAXC, sh->ck, sh->cv);
-    if (sh->pscale_out < 1 || sh->nlon_out > sh->nlon_out_global)
-        return s2attn_fail(S2ATTN_E_INVALID, "pscale_out must be positive and the local output width at most the global one");
+    if (sh->pscale_out < 1 || sh->nlon_out_global % sh->pscale_out != 0 || sh->nlon_out > sh->nlon_out_global)
+        return s2attn_fail(S2ATTN_E_INVALID, "pscale_out must be a positive divisor of nlon_out_global and the local output width at most the global one");
     if (sh->lon_lo_kx < 0 || (int64_t)sh->pscale_out * (sh->lon_lo_kx + sh->nlon_kx) > sh->nlon_out_global)
         return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", sh->lon_lo_kx, sh->lon_lo_kx + sh->nlon_kx,
                            sh->nlon_out_global / sh->pscale_out);
@@ -718,6 +728,7 @@ void fill_up(Args &a, const s2attn_ring_up_shape *sh, bool transposed)
         a.win_lo = sh->pscale_out * sh->lon_lo_kx, a.win_n = sh->pscale_out * sh->nlon_kx;
     else
         a.win_lo = 0, a.win_n = sh->nlon_out;
+    a.M = a.N / a.scale, a.win_q = a.win_n / a.scale;
 }
 
 } // namespace
