@@ -107,7 +107,7 @@ def build(verbose: bool = False) -> str:
     """Compile libs2attn.so for gfx950 with hipcc (always recompiles)."""
     csrc = os.path.join(_HERE, "csrc")
     subprocess.run(["make", "-C", csrc, "clean"], check=True, capture_output=not verbose)
-    proc = subprocess.run(["make", "-C", csrc], capture_output=True, text=True)
+    proc = subprocess.run(["make", "-C", csrc, "-j4"], capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"building libs2attn.so failed:\n{proc.stdout}\n{proc.stderr}")
     if verbose:

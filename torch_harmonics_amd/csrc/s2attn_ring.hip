@@ -78,11 +78,6 @@ template <int G> __device__ inline float group_sum(float x)
 }
 
 template <typename T> __device__ inline void unpack8(float (&x)[CPL], const T *p);
-template <> __device__ inline void unpack8<float>(float (&x)[CPL], const float *p)
-{
-    const float4 lo = reinterpret_cast<const float4 *>(p)[0], hi = reinterpret_cast<const float4 *>(p)[1];
-    x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
-}
 template <> __device__ inline void unpack8<__hip_bfloat16>(float (&x)[CPL], const __hip_bfloat16 *p)
 {
     const uint4 r = *reinterpret_cast<const uint4 *>(p);
@@ -101,43 +96,51 @@ template <> __device__ inline void unpack8<__half>(float (&x)[CPL], const __half
     }
 }
 
-// channels c0 .. c0 + 7 of a row of n channels (zeros past the end); vec: n is a multiple of 8 and the row is 16-byte aligned
-template <typename T> __device__ inline void load8(float (&x)[CPL], const T *row, int c0, int n, bool vec)
+// A lane's 8 channels are [ca, ca + 4) and [cb, cb + 4) of a row of n channels (zeros past the end).  vec: n is a multiple
+// of 8 and the rows are 16-byte aligned; 16-bit storage then has cb = ca + 4 and takes both pieces with one 16-byte load.
+template <typename T> __device__ inline void load8(float (&x)[CPL], const T *row, int ca, int cb, int n, bool vec)
 {
     if (vec) {
-        if (c0 < n) {
-            unpack8(x, row + c0);
+        if constexpr (sizeof(T) == 4) {
+            const float4 lo = ca < n ? *reinterpret_cast<const float4 *>(row + ca) : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 hi = cb < n ? *reinterpret_cast<const float4 *>(row + cb) : make_float4(0.f, 0.f, 0.f, 0.f);
+            x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
+        } else if (ca < n) {
+            unpack8(x, row + ca);
         } else {
 #pragma unroll
             for (int i = 0; i < CPL; i++) x[i] = 0.f;
         }
     } else {
 #pragma unroll
-        for (int i = 0; i < CPL; i++) x[i] = c0 + i < n ? ld(row + c0 + i) : 0.f;
+        for (int i = 0; i < 4; i++) x[i] = ca + i < n ? ld(row + ca + i) : 0.f, x[4 + i] = cb + i < n ? ld(row + cb + i) : 0.f;
     }
 }
 
-__device__ inline void store8(float *row, const float (&x)[CPL], int c0, int n, bool vec)
+__device__ inline void store8(float *row, const float (&x)[CPL], int ca, int cb, int n, bool vec)
 {
     if (vec) {
-        if (c0 < n) {
-            reinterpret_cast<float4 *>(row + c0)[0] = make_float4(x[0], x[1], x[2], x[3]);
-            reinterpret_cast<float4 *>(row + c0)[1] = make_float4(x[4], x[5], x[6], x[7]);
-        }
+        if (ca < n) *reinterpret_cast<float4 *>(row + ca) = make_float4(x[0], x[1], x[2], x[3]);
+        if (cb < n) *reinterpret_cast<float4 *>(row + cb) = make_float4(x[4], x[5], x[6], x[7]);
     } else {
 #pragma unroll
-        for (int i = 0; i < CPL; i++)
-            if (c0 + i < n) row[c0 + i] = x[i];
+        for (int i = 0; i < 4; i++) {
+            if (ca + i < n) row[ca + i] = x[i];
+            if (cb + i < n) row[cb + i] = x[4 + i];
+        }
     }
 }
 
 // The wavefront's place on a grid of nrow x ncol cells per batch: P longitudes of one row, `stride` apart (the regrouped
 // relation only joins cells of one residue class modulo scale with an entry, so a wavefront takes its cells from one class).
 template <int G> struct Place {
-    int b, row, x, x0, c0; // batch, latitude (after the launch order), this lane's longitude (clamped), the first one, first channel
-    bool valid;            // the lane's longitude is inside the row
+    int b, row, x, x0; // batch, latitude (after the launch order), this lane's longitude (clamped), the wavefront's first one
+    int ca, cb;        // the lane's channels: [ca, ca + 4) and [cb, cb + 4)
+    bool valid, first; // the lane's longitude is inside the row; first lane of its cell
     static __host__ __device__ inline long blocks_per_row(int ncol, int stride) { return (long)stride * (((ncol + stride - 1) / stride + 64 / G - 1) / (64 / G)); }
-    __device__ inline bool locate(int B, int nrow, int ncol, const int32_t *order, int stride)
+    // split: with 32-bit vector loads the G lanes of a cell take 16 consecutive bytes each, twice (channels 4 s .. and
+    // 4 G + 4 s ..), so that one load instruction of the wavefront reads whole 64-byte blocks; otherwise 8 s .. 8 s + 7.
+    __device__ inline bool locate(int B, int nrow, int ncol, const int32_t *order, int stride, bool split)
     {
         constexpr int P = 64 / G;
         const int lane = threadIdx.x & 63;
@@ -152,7 +155,10 @@ template <int G> struct Place {
         const int w = x0 + stride * (lane / G);
         valid = w < ncol;
         x = valid ? w : ncol - 1;
-        c0 = (lane % G) * CPL;
+        const int sub = lane % G;
+        first = sub == 0;
+        ca = split ? 4 * sub : CPL * sub;
+        cb = split ? 4 * G + 4 * sub : CPL * sub + 4;
         return true;
     }
 };
@@ -249,15 +255,15 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd
 {
     constexpr int U = 4;
     Place<G> pl;
-    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1)) return;
+    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
     const int xs = TR ? lane / G : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
     const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
     const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
     float qr[CPL], y[CPL];
-    load8(qr, static_cast<const T *>(a.q) + out * a.ck, pl.c0, a.ck, vec);
-    load8(y, a.y_acc + out * a.cv, pl.c0, a.cv, vec);
+    load8(qr, static_cast<const T *>(a.q) + out * a.ck, pl.ca, pl.cb, a.ck, vec);
+    load8(y, a.y_acc + out * a.cv, pl.ca, pl.cb, a.cv, vec);
     float S = a.alpha_sum[out], m = a.qdotk_max[out];
     int64_t z0, z1;
     entry_range<TR>(a, pl.row, z0, z1);
@@ -274,8 +280,8 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const long p = pt[u] < 0 ? 0 : pt[u];
-                load8(kk[u], kx + p * a.ck, pl.c0, a.ck, vec);
-                load8(vv[u], vx + p * a.cv, pl.c0, a.cv, vec);
+                load8(kk[u], kx + p * a.ck, pl.ca, pl.cb, a.ck, vec);
+                load8(vv[u], vx + p * a.cv, pl.ca, pl.cb, a.cv, vec);
             }
             float mn = m;
 #pragma unroll
@@ -302,11 +308,11 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd
         }
     }
     if (!pl.valid) return;
-    if (pl.c0 == 0) {
+    if (pl.first) {
         a.alpha_sum[out] = S;
         a.qdotk_max[out] = m;
     }
-    store8(a.y_acc + out * a.cv, y, pl.c0, a.cv, vec);
+    store8(a.y_acc + out * a.cv, y, pl.ca, pl.cb, a.cv, vec);
 }
 
 // Backward pass 1: folds the chunk into (integral = sum alpha <dy, v>, alpha_k = sum alpha k, alpha_kvw = sum alpha
@@ -316,17 +322,17 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1)) return;
+    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
     const int xs = TR ? lane / G : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
     const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
     const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
     float qr[CPL], gr[CPL], ak[CPL], akg[CPL];
-    load8(qr, static_cast<const T *>(a.q) + out * a.ck, pl.c0, a.ck, vec);
-    load8(gr, static_cast<const T *>(a.dy) + out * a.cv, pl.c0, a.cv, vec);
-    load8(ak, a.alpha_k + out * a.ck, pl.c0, a.ck, vec);
-    load8(akg, a.alpha_kvw + out * a.ck, pl.c0, a.ck, vec);
+    load8(qr, static_cast<const T *>(a.q) + out * a.ck, pl.ca, pl.cb, a.ck, vec);
+    load8(gr, static_cast<const T *>(a.dy) + out * a.cv, pl.ca, pl.cb, a.cv, vec);
+    load8(ak, a.alpha_k + out * a.ck, pl.ca, pl.cb, a.ck, vec);
+    load8(akg, a.alpha_kvw + out * a.ck, pl.ca, pl.cb, a.ck, vec);
     const bool fixed = a.fixed_max;
     float S = fixed ? 0.f : a.alpha_sum[out], m = a.qdotk_max[out], I = a.integral[out];
     int64_t z0, z1;
@@ -344,8 +350,8 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const long p = pt[u] < 0 ? 0 : pt[u];
-                load8(kk[u], kx + p * a.ck, pl.c0, a.ck, vec);
-                load8(vv[u], vx + p * a.cv, pl.c0, a.cv, vec);
+                load8(kk[u], kx + p * a.ck, pl.ca, pl.cb, a.ck, vec);
+                load8(vv[u], vx + p * a.cv, pl.ca, pl.cb, a.cv, vec);
             }
             float mn = m;
 #pragma unroll
@@ -376,15 +382,15 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
         }
     }
     if (!pl.valid) return;
-    if (pl.c0 == 0) {
+    if (pl.first) {
         if (!fixed) {
             a.alpha_sum[out] = S;
             a.qdotk_max[out] = m;
         }
         a.integral[out] = I;
     }
-    store8(a.alpha_k + out * a.ck, ak, pl.c0, a.ck, vec);
-    store8(a.alpha_kvw + out * a.ck, akg, pl.c0, a.ck, vec);
+    store8(a.alpha_k + out * a.ck, ak, pl.ca, pl.cb, a.ck, vec);
+    store8(a.alpha_kvw + out * a.ck, akg, pl.ca, pl.cb, a.ck, vec);
 }
 
 // Backward pass 2: with the final statistics, dk and dv of every chunk point, summed over the output cells that see it and
@@ -395,16 +401,15 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, nullptr, TR ? a.scale : 1)) return;
+    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, nullptr, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
     int64_t z0, z1;
     entry_range<TR>(a, pl.row, z0, z1);
     if (z0 >= z1 && !a.overwrite) return; // nothing sees this latitude
-    const int c0 = pl.c0;
     const long pt0 = ((long)pl.b * a.nlat_halo + pl.row) * a.nlon_kx + pl.x;
     float kr[CPL], vr[CPL], dk[CPL], dv[CPL];
-    load8(kr, static_cast<const T *>(a.k) + pt0 * a.ck, c0, a.ck, vec);
-    load8(vr, static_cast<const T *>(a.v) + pt0 * a.cv, c0, a.cv, vec);
+    load8(kr, static_cast<const T *>(a.k) + pt0 * a.ck, pl.ca, pl.cb, a.ck, vec);
+    load8(vr, static_cast<const T *>(a.v) + pt0 * a.cv, pl.ca, pl.cb, a.cv, vec);
 #pragma unroll
     for (int i = 0; i < CPL; i++) dk[i] = dv[i] = 0.f;
     const float wq = z0 < z1 ? a.quad_w[a.lat_halo_start + pl.row] : 0.f; // a padded row outside the grid has no entries and no weight
@@ -426,8 +431,8 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const long o = pt[u] < 0 ? 0 : pt[u];
-                load8(qq[u], qb + o * a.ck, c0, a.ck, vec);
-                load8(gg[u], gb + o * a.cv, c0, a.cv, vec);
+                load8(qq[u], qb + o * a.ck, pl.ca, pl.cb, a.ck, vec);
+                load8(gg[u], gb + o * a.cv, pl.ca, pl.cb, a.cv, vec);
                 S[u] = a.alpha_sum[obase + o], m[u] = a.qdotk_max[obase + o], In[u] = a.integral_norm[obase + o];
             }
 #pragma unroll
@@ -446,15 +451,15 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
     if (!pl.valid) return;
     if (!a.overwrite) {
         float cur[CPL];
-        load8(cur, a.dk + pt0 * a.ck, c0, a.ck, vec);
+        load8(cur, a.dk + pt0 * a.ck, pl.ca, pl.cb, a.ck, vec);
 #pragma unroll
         for (int i = 0; i < CPL; i++) dk[i] += cur[i];
-        load8(cur, a.dv + pt0 * a.cv, c0, a.cv, vec);
+        load8(cur, a.dv + pt0 * a.cv, pl.ca, pl.cb, a.cv, vec);
 #pragma unroll
         for (int i = 0; i < CPL; i++) dv[i] += cur[i];
     }
-    store8(a.dk + pt0 * a.ck, dk, c0, a.ck, vec);
-    store8(a.dv + pt0 * a.cv, dv, c0, a.cv, vec);
+    store8(a.dk + pt0 * a.ck, dk, pl.ca, pl.cb, a.ck, vec);
+    store8(a.dv + pt0 * a.cv, dv, pl.ca, pl.cb, a.cv, vec);
 }
 
 #undef S2_RING_TAKE
