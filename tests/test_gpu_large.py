@@ -204,3 +204,64 @@ def test_cfg5_bf16_sampled_rows_and_properties():
     _bf16_close("roll equivariance", y_roll, torch.roll(y, 5, 2).float())  # other tile alignment: equal up to bf16 rounding
     dk, dv, dq = ops.backward_saved(kd, vd, qd, gd, y, lse, *args)
     assert torch.isfinite(dk).all() and torch.isfinite(dv).all() and torch.isfinite(dq).all()
+
+
+@pytest.mark.parametrize("direction", ["gather", "upsample"])
+def test_ring_steps_fold_to_the_single_device_result(direction):
+    """Size-independent property at a real grid: folding the longitude chunks of K/V through the ring-step operators, in
+    any order, gives the single-device forward and backward (the chunked reduction of
+    torch_harmonics/distributed/distributed_attention.py:303-431 on one device)."""
+    from torch_harmonics_amd import ops
+    from torch_harmonics_amd.neighborhood import precompute_neighborhood_s2
+    from torch_harmonics_amd.quadrature import precompute_latitudes
+
+    up = direction == "upsample"
+    (Hi, Wi), (Ho, Wo) = ((91, 180), (181, 360)) if up else ((181, 360), (181, 360))
+    B, d, theta = 3, 32, 0.06
+    # psi is keyed by the coarser grid's latitude: output latitude, or input latitude when up-sampling (grids swapped)
+    col, roff, _ = precompute_neighborhood_s2((Ho, Wo) if up else (Hi, Wi), (Hi, Wi) if up else (Ho, Wo), "equiangular", "equiangular", theta)
+    rcol, rroff = col, roff
+    w = (2.0 * torch.pi * precompute_latitudes(Hi, "equiangular")[1].float() / Wi).contiguous().to(DEV)
+    gen = torch.Generator().manual_seed(777)
+    k, v = torch.randn(B, Hi, Wi, d, generator=gen).to(DEV), torch.randn(B, Hi, Wi, d, generator=gen).to(DEV)
+    q, dy = (torch.randn(B, Ho, Wo, d, generator=gen) / math.sqrt(d)).to(DEV), torch.randn(B, Ho, Wo, d, generator=gen).to(DEV)
+    geo = (w, col.to(DEV), roff.to(DEV), 1, Wi, Ho, Wo)
+    y, lse = ops.forward_lse(k, v, q, *geo)
+    dk, dv, dq = ops.backward_saved(k, v, q, dy, y, lse, *geo)
+
+    rcol, rroff = rcol.to(DEV), rroff.to(DEV)
+    bounds = [0, 37, 38, 120, Wi]
+    chunks = [(bounds[i], bounds[i + 1]) for i in (2, 0, 3, 1)]
+    z = lambda *s: torch.zeros(*s, device=DEV)  # noqa: E731
+    y_acc, asum, qmax = z(B, Ho, Wo, d), z(B, Ho, Wo), torch.full((B, Ho, Wo), float("-inf"), device=DEV)
+    integ, ak, akvw = z(B, Ho, Wo), z(B, Ho, Wo, d), z(B, Ho, Wo, d)
+    as2, qm2 = z(B, Ho, Wo), torch.full((B, Ho, Wo), float("-inf"), device=DEV)
+    if up:
+        tail = lambda lo: (Wi, Wo, Wo // Wi, lo, 0, Ho, Wo)  # noqa: E731
+        fwd = lambda kc, vc, lo: ops.forward_ring_step_upsample(kc, vc, q, y_acc, asum, qmax, w, rcol, rroff, *tail(lo))  # noqa: E731
+        p1 = lambda kc, vc, lo: ops.backward_ring_step_upsample_pass1(kc, vc, q, dy, qmax, integ, ak, akvw, w, rcol, rroff, *tail(lo))  # noqa: E731
+    else:
+        nnz = rroff[1:] - rroff[:-1]
+        row_idx = torch.argsort(nnz, descending=True, stable=True).to(torch.int32)
+        tail = lambda lo: (Wi, Wi // Wo, lo, 0, Ho, Wo, *ops.split_csr_rows(row_idx, rroff, Ho))  # noqa: E731
+        fwd = lambda kc, vc, lo: ops.forward_ring_step(kc, vc, q, y_acc, asum, qmax, w, rcol, rroff, row_idx, *tail(lo))  # noqa: E731
+        p1 = lambda kc, vc, lo: ops.backward_ring_step_pass1(kc, vc, q, dy, as2, qm2, integ, ak, akvw, w, rcol, rroff, row_idx, *tail(lo))  # noqa: E731
+    parts = [(k[:, :, a:b].contiguous(), v[:, :, a:b].contiguous(), a) for a, b in chunks]
+    for kc, vc, lo in parts:
+        fwd(kc, vc, lo)
+    for kc, vc, lo in parts:
+        p1(kc, vc, lo)
+    S = asum[..., None]
+    assert_close("ring y", y_acc / S, y, **TOL)
+    assert_close("ring dq", (S * akvw - integ[..., None] * ak) / S**2, dq, rtol=1e-4, atol=1e-5)
+    inorm = (integ / asum).contiguous()
+    rdk, rdv = torch.zeros_like(k), torch.zeros_like(v)
+    for (kc, vc, lo), (a, b) in zip(parts, chunks):
+        dkc, dvc = torch.zeros_like(kc), torch.zeros_like(vc)
+        if up:
+            ops.backward_ring_step_upsample_pass2(kc, vc, q, dy, asum, qmax, inorm, dkc, dvc, w, rcol, rroff, *tail(lo))
+        else:
+            ops.backward_ring_step_pass2(kc, vc, q, dy, asum, qmax, inorm, dkc, dvc, w, rcol, rroff, row_idx, *tail(lo))
+        rdk[:, :, a:b], rdv[:, :, a:b] = dkc, dvc
+    assert_close("ring dk", rdk, dk, rtol=1e-4, atol=1e-5)
+    assert_close("ring dv", rdv, dv, rtol=1e-4, atol=1e-5)

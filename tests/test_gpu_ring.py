@@ -21,13 +21,28 @@ def _geo_dev(p):
     return p["quad"].to(DEV), p["col_l"].to(DEV), p["roff_l"].to(DEV), p["row_idx"].to(DEV)
 
 
+# channel counts that are multiples of 8 take the 16-byte load paths; 32 / 64 / 128 / 256 / 512 channels = 4 / 8 / 16 / 32 / 64 lanes per cell
+VECTOR_CHANNELS = [(32, 32), (64, 128), (8, 16), (256, 40), (512, 8)]
+
+
 @pytest.mark.parametrize("case", RING_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_ring_steps_against_oracle_and_dense_attention(case, dtype, monkeypatch):
+    ck, cv = (70, 33) if case is RING_CASES[1] else (5, 3)  # one case with more than 64 channels
+    _gather_direction(case, dtype, ck, cv, monkeypatch)
+
+
+@pytest.mark.parametrize("chan", VECTOR_CHANNELS, ids=lambda c: f"ck{c[0]}cv{c[1]}")
+@pytest.mark.parametrize("case", [RING_CASES[1], RING_CASES[3]], ids=["ratio1", "ratio3"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+def test_ring_steps_vector_load_paths(case, dtype, chan, monkeypatch):
+    _gather_direction(case, dtype, *chan, monkeypatch)
+
+
+def _gather_direction(case, dtype, ck, cv, monkeypatch):
     from torch_harmonics_amd import ops
 
-    print(f"case {case} {dtype}", flush=True)
-    ck, cv = (70, 33) if case is RING_CASES[1] else (5, 3)  # one case with more than 64 channels (two per lane)
+    print(f"case {case} {dtype} ck={ck} cv={cv}", flush=True)
     p = local_problem(case, ck=ck, cv=cv)
     for name in ("k", "v", "q", "dy", "q_l", "dy_l"):  # the values the storage dtype can hold, shared by all three evaluations
         p[name] = p[name].to(dtype).float()
@@ -139,10 +154,21 @@ from tests.ring_util import RING_UP_CASES, local_problem_upsample  # noqa: E402
 @pytest.mark.parametrize("case", RING_UP_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16], ids=["f32", "bf16"])
 def test_upsample_ring_steps_against_oracle_and_dense_attention(case, dtype):
+    ck, cv = (70, 33) if case is RING_UP_CASES[1] else (5, 3)
+    _upsample_direction(case, dtype, ck, cv)
+
+
+@pytest.mark.parametrize("chan", VECTOR_CHANNELS, ids=lambda c: f"ck{c[0]}cv{c[1]}")
+@pytest.mark.parametrize("case", [RING_UP_CASES[1], RING_UP_CASES[2]], ids=["ratio2", "ratio3_padded"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
+def test_upsample_ring_steps_vector_load_paths(case, dtype, chan):
+    _upsample_direction(case, dtype, *chan)
+
+
+def _upsample_direction(case, dtype, ck, cv):
     from torch_harmonics_amd import ops
 
-    print(f"case {case} {dtype}", flush=True)
-    ck, cv = (70, 33) if case is RING_UP_CASES[1] else (5, 3)
+    print(f"case {case} {dtype} ck={ck} cv={cv}", flush=True)
     p = local_problem_upsample(case, ck=ck, cv=cv)
     for name in ("k", "v", "q", "dy", "q_l", "dy_l"):
         p[name] = p[name].to(dtype).float()
