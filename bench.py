@@ -168,6 +168,87 @@ def time_other_config(name, device, steps=3, cpu=False):
     return res
 
 
+def time_ring_steps(device, nchunk=4, reps=2):
+    """The ring-step operators on one device (all longitude chunks of K/V folded one after the other, ms for the whole fold):
+    gather direction on cfg3's tensors (B = 1, 8 heads of 32 channels folded into the batch, its grid and cutoff), up-sampling
+    361x720 -> 721x1440 with the same batch; fp32."""
+    from torch_harmonics_amd import ops
+    from torch_harmonics_amd.neighborhood import precompute_neighborhood_s2
+    from torch_harmonics_amd.quadrature import precompute_latitudes
+
+    BB, d = CONFIGS["cfg3"]["B"] * CONFIGS["cfg3"]["nh"], CONFIGS["cfg3"]["C"] // CONFIGS["cfg3"]["nh"]
+    gen = torch.Generator(device=device).manual_seed(333)
+    res = {}
+    for name, ins, outs, theta in (("gather", (721, 1440), (721, 1440), CONFIGS["cfg3"]["theta_cutoff"]), ("upsample", (361, 720), (721, 1440), 0.03)):
+        up = name == "upsample"
+        (Hi, Wi), (Ho, Wo) = ins, outs
+        col, roff, _ = precompute_neighborhood_s2(outs if up else ins, ins if up else outs, "equiangular", "equiangular", theta)
+        w = (2.0 * torch.pi * precompute_latitudes(Hi, "equiangular")[1].float() / Wi).contiguous().to(device)
+        row_idx = torch.argsort(roff[1:] - roff[:-1], descending=True, stable=True).to(torch.int32)
+        split = ops.split_csr_rows(row_idx, roff, Ho)
+        pairs = BB * (Wi if up else Wo) * col.numel()
+        col, roff, row_idx = col.to(device), roff.to(device), row_idx.to(device)
+        k = torch.randn(BB, Hi, Wi, d, device=device, generator=gen)
+        v = torch.randn(BB, Hi, Wi, d, device=device, generator=gen)
+        q = torch.randn(BB, Ho, Wo, d, device=device, generator=gen) / math.sqrt(d)
+        dy = torch.randn(BB, Ho, Wo, d, device=device, generator=gen)
+        cw = Wi // nchunk
+        parts = [(k[:, :, i * cw : (i + 1) * cw].contiguous(), v[:, :, i * cw : (i + 1) * cw].contiguous(), i * cw) for i in range(nchunk)]
+        z = lambda *s: torch.zeros(*s, device=device)  # noqa: E731
+        y_acc, asum, qmax = z(BB, Ho, Wo, d), z(BB, Ho, Wo), z(BB, Ho, Wo)
+        integ, ak, akvw, as2, qm2 = z(BB, Ho, Wo), z(BB, Ho, Wo, d), z(BB, Ho, Wo, d), z(BB, Ho, Wo), z(BB, Ho, Wo)
+        tail = (lambda lo: (Wi, Wo, Wo // Wi, lo, 0, Ho, Wo)) if up else (lambda lo: (Wi, Wi // Wo, lo, 0, Ho, Wo, *split))
+
+        def fwd():
+            y_acc.zero_(), asum.zero_(), qmax.fill_(float("-inf"))
+            for kc, vc, lo in parts:
+                if up:
+                    ops.forward_ring_step_upsample(kc, vc, q, y_acc, asum, qmax, w, col, roff, *tail(lo))
+                else:
+                    ops.forward_ring_step(kc, vc, q, y_acc, asum, qmax, w, col, roff, row_idx, *tail(lo))
+
+        def pass1():
+            integ.zero_(), ak.zero_(), akvw.zero_(), as2.zero_(), qm2.fill_(float("-inf"))
+            for kc, vc, lo in parts:
+                if up:
+                    ops.backward_ring_step_upsample_pass1(kc, vc, q, dy, qmax, integ, ak, akvw, w, col, roff, *tail(lo))
+                else:
+                    ops.backward_ring_step_pass1(kc, vc, q, dy, as2, qm2, integ, ak, akvw, w, col, roff, row_idx, *tail(lo))
+
+        grads = [(torch.zeros_like(kc), torch.zeros_like(vc)) for kc, vc, _ in parts]
+
+        def pass2():
+            for (kc, vc, lo), (dkc, dvc) in zip(parts, grads):
+                if up:
+                    ops.backward_ring_step_upsample_pass2(kc, vc, q, dy, asum, qmax, inorm, dkc, dvc, w, col, roff, *tail(lo))
+                else:
+                    ops.backward_ring_step_pass2(kc, vc, q, dy, asum, qmax, inorm, dkc, dvc, w, col, roff, row_idx, *tail(lo))
+
+        def run(f):
+            f()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(reps):
+                f()
+            torch.cuda.synchronize()
+            return 1e3 * (time.perf_counter() - t0) / reps
+
+        t_f, t_1 = run(fwd), run(pass1)
+        inorm = (integ / asum).contiguous()
+        t_2 = run(pass2)
+        # the same attention in one piece (psi keyed the same way), for scale
+        geo = (w, col, roff, 1, Wi, Ho, Wo)
+        y, lse = ops.forward_lse(k, v, q, *geo)
+        t_one = run(lambda: ops.forward_lse(k, v, q, *geo))
+        err = ((y_acc / asum[..., None]) - y).abs().max().item()
+        res[name] = {
+            "grid": f"{Hi}x{Wi} -> {Ho}x{Wo}", "theta_cutoff": theta, "pairs": pairs, "chunks": nchunk, "forward_ms": t_f, "pass1_ms": t_1, "pass2_ms": t_2,
+            "single_device_forward_ms": t_one, "max_abs_diff_to_single_device_y": err,
+        }  # fmt: skip
+        del k, v, q, dy, parts, grads, y_acc, ak, akvw, y
+    return res
+
+
 def cpu_baseline(cfg, mod, k, v, q, dy):
     """
     Times the fp32 CPU port of the reference algorithm (oracle/s2attn_oracle.c, built with the reference's
@@ -223,6 +304,8 @@ def main():
     ap.add_argument("--no-other-configs", action="store_true", help="skip the op-level timings of the other benchmark configurations")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true", help="skip the module-level (projections + permutes) timing")
+    ap.add_argument("--no-ring", action="store_true", help="skip the timing of the ring-step operators")
+    ap.add_argument("--ring-only", action="store_true", help="time the ring-step operators and nothing else (for profiling)")
     args = ap.parse_args()
 
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -239,6 +322,9 @@ def main():
     cfg = CONFIGS[args.config]
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
+    if args.ring_only:
+        print(json.dumps({"ring_steps": time_ring_steps(dev)}))
+        return
     mod, x_in, x_out, k, v, q, dy = make_workload(cfg, dev)
     (Hi, Wi), (Ho, Wo) = cfg["in_shape"], cfg["out_shape"]
     nh, B = cfg["nh"], cfg["B"]
@@ -403,6 +489,9 @@ def main():
         out["other_configs"] = {
             name: time_other_config(name, dev, cpu=(not args.no_cpu_baseline) and name in ("cfg1", "cfg2")) for name in sorted(CONFIGS) if name != args.config
         }
+
+    if not args.no_ring:
+        out["ring_steps"] = time_ring_steps(dev)
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy)

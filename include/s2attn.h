@@ -244,11 +244,14 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
  * Backward pass 2 of the gather direction on the regrouped psi (modulus nlon_in, key_lo = lat_halo_start, nkeys =
  * nlat_halo; t_lat = local output latitude): the same dk, dv as s2attn_ring_backward_pass2
  * (attention_cuda_bwd_ring.cu:1312-1440), summed per chunk point in a fixed order and added to dk, dv without atomics.
+ * row_order (here and in s2attn_ring_backward_pass2_upsample; may be null) lists the nlat_halo chunk latitudes in the
+ * order to launch them, the ones with the most entries first, which keeps the end of the launch busy.
  */
 int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                           const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
                                           const float *quad_weights, const int32_t *t_lat, const int32_t *t_lon,
-                                          const int64_t *t_off, const s2attn_ring_shape *shape, void *stream);
+                                          const int64_t *t_off, const int32_t *row_order, const s2attn_ring_shape *shape,
+                                          void *stream);
 
 /*
  * The same three steps for the up-sampling (scatter) direction, nlon_out a multiple of nlon_in.  Replace
@@ -286,7 +289,7 @@ int s2attn_ring_backward_pass1_upsample(const void *k, const void *v, const void
 int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                         const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
                                         const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
-                                        const s2attn_ring_up_shape *shape, void *stream);
+                                        const int32_t *row_order, const s2attn_ring_up_shape *shape, void *stream);
 
 #ifdef __cplusplus
 }

@@ -45,7 +45,7 @@ struct Args {
     float *dk, *dv;
     const float *quad_w;
     const int64_t *col_idx, *row_off; // psi as given: col = partner latitude * N + off
-    const int32_t *row_idx;           // launch order of the output latitudes (may be null: natural order)
+    const int32_t *row_idx;           // launch order of the owners' latitudes, longest first (may be null: natural order)
     const int64_t *t_off;             // psi regrouped by the owner's latitude: entries t_off[r] .. t_off[r + 1] of latitude r
     const int32_t *t_lat, *t_lon;     //   (partner's local latitude, off)
     int B, nlat_halo, nlon_kx, Ho, Wo, ck, cv;
@@ -401,7 +401,7 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, nullptr, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
+    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, a.row_idx, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
     int64_t z0, z1;
     entry_range<TR>(a, pl.row, z0, z1);
@@ -688,7 +688,8 @@ extern "C" int s2attn_ring_backward_pass2(const void *k, const void *v, const vo
 extern "C" int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                                      const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
                                                      const float *quad_weights, const int32_t *t_ho, const int32_t *t_dlon,
-                                                     const int64_t *t_off, const s2attn_ring_shape *shape, void *stream)
+                                                     const int64_t *t_off, const int32_t *row_order, const s2attn_ring_shape *shape,
+                                                     void *stream)
 {
     const int rc = check(shape);
     if (rc != S2ATTN_OK) return rc;
@@ -699,7 +700,7 @@ extern "C" int s2attn_ring_backward_pass2_transposed(const void *k, const void *
     a.k = k, a.v = v, a.q = q, a.dy = dy;
     a.alpha_sum = const_cast<float *>(alpha_sum), a.qdotk_max = const_cast<float *>(qdotk_max), a.integral_norm = integral_norm;
     a.dk = dk, a.dv = dv;
-    a.quad_w = quad_weights, a.t_lat = t_ho, a.t_lon = t_dlon, a.t_off = t_off;
+    a.quad_w = quad_weights, a.t_lat = t_ho, a.t_lon = t_dlon, a.t_off = t_off, a.row_idx = row_order;
     return launch<true>(PASS2, a, shape->dtype, stream);
 }
 
@@ -773,7 +774,7 @@ extern "C" int s2attn_ring_backward_pass1_upsample(const void *k, const void *v,
 extern "C" int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                                    const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
                                                    const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
-                                                   const s2attn_ring_up_shape *shape, void *stream)
+                                                   const int32_t *row_order, const s2attn_ring_up_shape *shape, void *stream)
 {
     const int rc = check_up(shape);
     if (rc != S2ATTN_OK) return rc;
@@ -784,6 +785,6 @@ extern "C" int s2attn_ring_backward_pass2_upsample(const void *k, const void *v,
     a.k = k, a.v = v, a.q = q, a.dy = dy;
     a.alpha_sum = const_cast<float *>(alpha_sum), a.qdotk_max = const_cast<float *>(qdotk_max), a.integral_norm = integral_norm;
     a.dk = dk, a.dv = dv, a.overwrite = true;
-    a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off;
+    a.quad_w = quad_weights, a.col_idx = col_idx, a.row_off = row_off, a.row_idx = row_order;
     return launch<false>(PASS2, a, shape->dtype, stream);
 }

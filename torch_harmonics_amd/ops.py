@@ -23,7 +23,7 @@ import torch
 
 from . import _lib
 from ._attention_utils import _setup_context_attention_backward
-from .plan import get_plan, get_transposed_csr
+from .plan import get_plan, get_row_order, get_transposed_csr
 
 _DTYPE_CODE = {torch.float32: _lib.S2ATTN_F32, torch.bfloat16: _lib.S2ATTN_BF16, torch.float16: _lib.S2ATTN_F16}
 
@@ -598,8 +598,8 @@ def backward_ring_step_pass2(
         if _RING_PASS2_FROM_CSR:
             rc = _lib.load().s2attn_ring_backward_pass2(*head, col_idx.data_ptr(), row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
         else:
-            t_lat, t_lon, t_off = get_transposed_csr(col_idx, row_off, nlon_in, lat_halo_start, kx.shape[1])  # psi regrouped by input latitude
-            rc = _lib.load().s2attn_ring_backward_pass2_transposed(*head, t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
+            t_lat, t_lon, t_off, t_order = get_transposed_csr(col_idx, row_off, nlon_in, lat_halo_start, kx.shape[1])  # psi regrouped by input latitude
+            rc = _lib.load().s2attn_ring_backward_pass2_transposed(*head, t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), t_order.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
     _lib.check(rc, "s2attn_ring_backward_pass2")
 
 
@@ -643,7 +643,7 @@ def forward_ring_step_upsample(
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
     with torch.cuda.device(kx.device):
-        t_lat, t_lon, t_off = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)  # psi regrouped by output latitude
+        t_lat, t_lon, t_off, _ = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)  # psi regrouped by output latitude
         rc = _lib.load().s2attn_ring_forward_step_upsample(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
             quad_weights.data_ptr(), t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
@@ -684,7 +684,7 @@ def backward_ring_step_upsample_pass1(
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
     with torch.cuda.device(kx.device):
-        t_lat, t_lon, t_off = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)
+        t_lat, t_lon, t_off, _ = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)
         rc = _lib.load().s2attn_ring_backward_pass1_upsample(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), qdotk_max_buf.data_ptr(), integral_buf.data_ptr(), alpha_k_buf.data_ptr(),
             alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(), t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
@@ -735,7 +735,8 @@ def backward_ring_step_upsample_pass2(
     with torch.cuda.device(kx.device):
         rc = _lib.load().s2attn_ring_backward_pass2_upsample(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(), integral_norm_buf.data_ptr(),
-            dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device),
+            dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr(), col_idx.data_ptr(), row_off.data_ptr(), get_row_order(row_off).data_ptr(),
+            ctypes.byref(shape), _stream_ptr(kx.device),
         )  # fmt: skip
     _lib.check(rc, "s2attn_ring_backward_pass2_upsample")
 

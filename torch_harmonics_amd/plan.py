@@ -111,9 +111,9 @@ def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in
 def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, modulus: int, key_lo: int, nkeys: int):
     """
     The CSR entries regrouped by key = col // modulus (the latitude named in col), for the ring-step kernels that gather
-    over the grid psi is not keyed by: (t_lat int32, t_lon int32, t_off int64 of nkeys + 1 entries) with the entries of
-    key key_lo + i at t_off[i] .. t_off[i + 1], in CSR order, as (CSR row of the entry, col mod modulus); see
-    include/s2attn.h.  Built with device operations only (no host round trip) the first time a psi is seen, then served
+    over the grid psi is not keyed by: (t_lat int32, t_lon int32, t_off int64 of nkeys + 1 entries, t_order int32) with the
+    entries of key key_lo + i at t_off[i] .. t_off[i + 1], in CSR order, as (CSR row of the entry, col mod modulus), and
+    t_order the keys by decreasing number of entries; see include/s2attn.h.  Built with device operations only (no host round trip) the first time a psi is seen, then served
     from the same cache as the plans.
     """
     key = ("transposed", col_idx.data_ptr(), row_off.data_ptr(), col_idx.numel(), row_off.numel(), col_idx._version, row_off._version,
@@ -122,7 +122,7 @@ def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, modulus: in
         hit = _cache.get(key)
         if hit is not None:
             _cache.move_to_end(key)
-            return hit[:3]
+            return hit[:4]
     dev, nnz, nrow = col_idx.device, col_idx.numel(), row_off.numel() - 1
     rows = torch.repeat_interleave(torch.arange(nrow, device=dev, dtype=torch.int32), row_off[1:] - row_off[:-1], output_size=nnz)
     lat = torch.div(col_idx, modulus, rounding_mode="floor")
@@ -130,12 +130,29 @@ def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, modulus: in
     t_lat = rows[order].contiguous()
     t_lon = (col_idx - lat * modulus)[order].to(torch.int32).contiguous()
     t_off = torch.searchsorted(lat[order], torch.arange(key_lo, key_lo + nkeys + 1, device=dev, dtype=lat.dtype)).contiguous()
-    entry = (t_lat, t_lon, t_off, (col_idx, row_off))  # the CSR tensors stay alive with the entry: their addresses cannot be recycled
+    t_order = torch.argsort(t_off[1:] - t_off[:-1], descending=True, stable=True).to(torch.int32).contiguous()  # launch order: longest rows first
+    entry = (t_lat, t_lon, t_off, t_order, (col_idx, row_off))  # the CSR tensors stay alive with the entry: their addresses cannot be recycled
     with _lock:
         _cache[key] = entry
         while len(_cache) > _MAX_ENTRIES:
             _cache.popitem(last=False)
-    return entry[:3]
+    return entry[:4]
+
+
+def get_row_order(row_off: torch.Tensor) -> torch.Tensor:
+    """CSR rows by decreasing number of entries (int32, on row_off's device), cached per row_off."""
+    key = ("order", row_off.data_ptr(), row_off.numel(), row_off._version, str(row_off.device))
+    with _lock:
+        hit = _cache.get(key)
+        if hit is not None:
+            _cache.move_to_end(key)
+            return hit[0]
+    order = torch.argsort(row_off[1:] - row_off[:-1], descending=True, stable=True).to(torch.int32).contiguous()
+    with _lock:
+        _cache[key] = (order, row_off)
+        while len(_cache) > _MAX_ENTRIES:
+            _cache.popitem(last=False)
+    return order
 
 
 def clear_plan_cache() -> None:
