@@ -319,3 +319,38 @@ def test_operator_argument_errors():
         ops.permute_to_nhwc(torch.randn(1, 2, 3, 4))
     with pytest.raises(RuntimeError, match="integer multiple"):
         ops.forward(k[:, :, :10].contiguous(), v[:, :, :10].contiguous(), q, *psi, 2, 10, 6, 12)
+
+
+@pytest.mark.parametrize("modulus,key_lo,nkeys", [(12, 0, 6), (12, 2, 3), (12, -2, 10), (24, 0, 3)])
+def test_regrouped_psi_is_a_stable_sort_by_latitude(modulus, key_lo, nkeys):
+    """plan.get_transposed_csr against a plain loop: the entries of key key_lo + i, in CSR order, as (CSR row, col mod modulus);
+    the launch order lists the keys by decreasing number of entries."""
+    from torch_harmonics_amd import plan
+
+    gen = torch.Generator().manual_seed(11)
+    nrow = 7
+    counts = torch.randint(0, 9, (nrow,), generator=gen)
+    roff = torch.cat([torch.zeros(1, dtype=torch.int64), counts.cumsum(0)])
+    col = torch.randint(0, 6 * 12, (int(roff[-1]),), generator=gen)  # unsorted, with duplicates
+    plan.clear_plan_cache()
+    t_lat, t_lon, t_off, t_order = plan.get_transposed_csr(col, roff, modulus, key_lo, nkeys)
+    assert t_lat.dtype == torch.int32 and t_lon.dtype == torch.int32 and t_off.dtype == torch.int64 and t_order.dtype == torch.int32
+    assert t_off.numel() == nkeys + 1
+    want = [[] for _ in range(nkeys)]
+    for r in range(nrow):
+        for z in range(int(roff[r]), int(roff[r + 1])):
+            key = int(col[z]) // modulus - key_lo
+            if 0 <= key < nkeys:
+                want[key].append((r, int(col[z]) % modulus))
+    for i in range(nkeys):
+        got = [(int(t_lat[z]), int(t_lon[z])) for z in range(int(t_off[i]), int(t_off[i + 1]))]
+        assert got == want[i], f"key {key_lo + i}"
+    lens = [len(w) for w in want]
+    assert sorted(t_order.tolist()) == list(range(nkeys))
+    assert [lens[i] for i in t_order.tolist()] == sorted(lens, reverse=True)
+    again = plan.get_transposed_csr(col, roff, modulus, key_lo, nkeys)
+    assert again[0] is t_lat  # served from the cache
+    col[0] = (int(col[0]) + modulus) % (6 * 12)  # an in-place edit changes the version counter: rebuilt
+    assert plan.get_transposed_csr(col, roff, modulus, key_lo, nkeys)[0] is not t_lat
+    order = plan.get_row_order(roff)
+    assert [int(counts[i]) for i in order.tolist()] == sorted(counts.tolist(), reverse=True)
