@@ -96,11 +96,11 @@ template <> __device__ inline void unpack8<__half>(float (&x)[CPL], const __half
     }
 }
 
-// A lane's 8 channels are [ca, ca + 4) and [cb, cb + 4) of a row of n channels (zeros past the end).  vec: n is a multiple
+// A lane's 8 channels are [ca, ca + 4) and [cb, cb + 4) of a row of n channels (zeros past the end).  VEC: n is a multiple
 // of 8 and the rows are 16-byte aligned; 16-bit storage then has cb = ca + 4 and takes both pieces with one 16-byte load.
-template <typename T> __device__ inline void load8(float (&x)[CPL], const T *row, int ca, int cb, int n, bool vec)
+template <typename T, bool VEC> __device__ inline void load8(float (&x)[CPL], const T *row, int ca, int cb, int n)
 {
-    if (vec) {
+    if constexpr (VEC) {
         if constexpr (sizeof(T) == 4) {
             const float4 lo = ca < n ? *reinterpret_cast<const float4 *>(row + ca) : make_float4(0.f, 0.f, 0.f, 0.f);
             const float4 hi = cb < n ? *reinterpret_cast<const float4 *>(row + cb) : make_float4(0.f, 0.f, 0.f, 0.f);
@@ -117,9 +117,25 @@ template <typename T> __device__ inline void load8(float (&x)[CPL], const T *row
     }
 }
 
-__device__ inline void store8(float *row, const float (&x)[CPL], int ca, int cb, int n, bool vec)
+// The same for the rows read in the inner loops.  VEC: no test against n -- the caller passes channels clamped into the
+// row (lanes past the end re-read channels 0 .. 7; what they compute meets a zero operand or is never stored).
+template <typename T, bool VEC> __device__ inline void load8_hot(float (&x)[CPL], const T *row, int ca, int cb, int n)
 {
-    if (vec) {
+    if constexpr (VEC) {
+        if constexpr (sizeof(T) == 4) {
+            const float4 lo = *reinterpret_cast<const float4 *>(row + ca), hi = *reinterpret_cast<const float4 *>(row + cb);
+            x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
+        } else {
+            unpack8(x, row + ca);
+        }
+    } else {
+        load8<T, false>(x, row, ca, cb, n);
+    }
+}
+
+template <bool VEC> __device__ inline void store8(float *row, const float (&x)[CPL], int ca, int cb, int n)
+{
+    if constexpr (VEC) {
         if (ca < n) *reinterpret_cast<float4 *>(row + ca) = make_float4(x[0], x[1], x[2], x[3]);
         if (cb < n) *reinterpret_cast<float4 *>(row + cb) = make_float4(x[4], x[5], x[6], x[7]);
     } else {
@@ -251,19 +267,22 @@ template <bool TR> __device__ inline float partner_weight(const Args &a, bool ok
 // Forward: folds the chunk into (y_acc, alpha_sum, qdotk_max) of every output cell.  attention_cuda_fwd_ring.cu:66-175;
 // TR (up-sampling, psi regrouped by output latitude): the result of the three scatter phases of
 // attention_cuda_fwd_ring_upsample.cu:108-243 with the running maximum kept per cell instead.
-template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd_kernel(const Args a, const bool vec)
+template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256) void fwd_kernel(const Args a)
 {
     constexpr int U = 4;
     Place<G> pl;
-    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
+    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
+    // channels of the inner-loop rows, clamped into the row for the unconditional vector loads
+    const int ka = VEC && pl.ca >= a.ck ? 0 : pl.ca, kb = VEC && pl.cb >= a.ck ? 4 : pl.cb;
+    const int va = VEC && pl.ca >= a.cv ? 0 : pl.ca, vb = VEC && pl.cb >= a.cv ? 4 : pl.cb;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
     const int xs = TR ? lane / G : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
     const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
     const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
     float qr[CPL], y[CPL];
-    load8(qr, static_cast<const T *>(a.q) + out * a.ck, pl.ca, pl.cb, a.ck, vec);
-    load8(y, a.y_acc + out * a.cv, pl.ca, pl.cb, a.cv, vec);
+    load8<T, VEC>(qr, static_cast<const T *>(a.q) + out * a.ck, pl.ca, pl.cb, a.ck);
+    load8<float, VEC>(y, a.y_acc + out * a.cv, pl.ca, pl.cb, a.cv);
     float S = a.alpha_sum[out], m = a.qdotk_max[out];
     int64_t z0, z1;
     entry_range<TR>(a, pl.row, z0, z1);
@@ -280,8 +299,8 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const long p = pt[u] < 0 ? 0 : pt[u];
-                load8(kk[u], kx + p * a.ck, pl.ca, pl.cb, a.ck, vec);
-                load8(vv[u], vx + p * a.cv, pl.ca, pl.cb, a.cv, vec);
+                load8_hot<T, VEC>(kk[u], kx + p * a.ck, ka, kb, a.ck);
+                load8_hot<T, VEC>(vv[u], vx + p * a.cv, va, vb, a.cv);
             }
             float mn = m;
 #pragma unroll
@@ -312,27 +331,30 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void fwd
         a.alpha_sum[out] = S;
         a.qdotk_max[out] = m;
     }
-    store8(a.y_acc + out * a.cv, y, pl.ca, pl.cb, a.cv, vec);
+    store8<VEC>(a.y_acc + out * a.cv, y, pl.ca, pl.cb, a.cv);
 }
 
 // Backward pass 1: folds the chunk into (integral = sum alpha <dy, v>, alpha_k = sum alpha k, alpha_kvw = sum alpha
 // <dy, v> k) and, with a running maximum, (alpha_sum, qdotk_max) (attention_cuda_bwd_ring.cu:78-205); with fixed_max the
 // maximum is the forward's final one and only the three sums are touched (attention_cuda_bwd_ring_upsample.cu:88-160).
-template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pass1_kernel(const Args a, const bool vec)
+template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256) void pass1_kernel(const Args a)
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
+    if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
+    // channels of the inner-loop rows, clamped into the row for the unconditional vector loads
+    const int ka = VEC && pl.ca >= a.ck ? 0 : pl.ca, kb = VEC && pl.cb >= a.ck ? 4 : pl.cb;
+    const int va = VEC && pl.ca >= a.cv ? 0 : pl.ca, vb = VEC && pl.cb >= a.cv ? 4 : pl.cb;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
     const int xs = TR ? lane / G : (int)(((long)a.scale * pl.x) % a.N), xs0 = TR ? pl.x0 : (int)(((long)a.scale * pl.x0) % a.N);
     const T *__restrict__ kx = static_cast<const T *>(a.k) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.ck;
     const T *__restrict__ vx = static_cast<const T *>(a.v) + (long)pl.b * a.nlat_halo * a.nlon_kx * a.cv;
     float qr[CPL], gr[CPL], ak[CPL], akg[CPL];
-    load8(qr, static_cast<const T *>(a.q) + out * a.ck, pl.ca, pl.cb, a.ck, vec);
-    load8(gr, static_cast<const T *>(a.dy) + out * a.cv, pl.ca, pl.cb, a.cv, vec);
-    load8(ak, a.alpha_k + out * a.ck, pl.ca, pl.cb, a.ck, vec);
-    load8(akg, a.alpha_kvw + out * a.ck, pl.ca, pl.cb, a.ck, vec);
+    load8<T, VEC>(qr, static_cast<const T *>(a.q) + out * a.ck, pl.ca, pl.cb, a.ck);
+    load8<T, VEC>(gr, static_cast<const T *>(a.dy) + out * a.cv, pl.ca, pl.cb, a.cv);
+    load8<float, VEC>(ak, a.alpha_k + out * a.ck, pl.ca, pl.cb, a.ck);
+    load8<float, VEC>(akg, a.alpha_kvw + out * a.ck, pl.ca, pl.cb, a.ck);
     const bool fixed = a.fixed_max;
     float S = fixed ? 0.f : a.alpha_sum[out], m = a.qdotk_max[out], I = a.integral[out];
     int64_t z0, z1;
@@ -350,8 +372,8 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const long p = pt[u] < 0 ? 0 : pt[u];
-                load8(kk[u], kx + p * a.ck, pl.ca, pl.cb, a.ck, vec);
-                load8(vv[u], vx + p * a.cv, pl.ca, pl.cb, a.cv, vec);
+                load8_hot<T, VEC>(kk[u], kx + p * a.ck, ka, kb, a.ck);
+                load8_hot<T, VEC>(vv[u], vx + p * a.cv, va, vb, a.cv);
             }
             float mn = m;
 #pragma unroll
@@ -389,27 +411,30 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
         }
         a.integral[out] = I;
     }
-    store8(a.alpha_k + out * a.ck, ak, pl.ca, pl.cb, a.ck, vec);
-    store8(a.alpha_kvw + out * a.ck, akg, pl.ca, pl.cb, a.ck, vec);
+    store8<VEC>(a.alpha_k + out * a.ck, ak, pl.ca, pl.cb, a.ck);
+    store8<VEC>(a.alpha_kvw + out * a.ck, akg, pl.ca, pl.cb, a.ck);
 }
 
 // Backward pass 2: with the final statistics, dk and dv of every chunk point, summed over the output cells that see it and
 // added to (or, with overwrite, written into) the caller's arrays once.  Same arithmetic as attention_cuda_bwd_ring.cu:
 // 1312-1440 (TR: psi regrouped by input latitude, loop order turned inside out) and
 // attention_cuda_bwd_ring_upsample.cu:162-240 (psi as given, keyed by the chunk's own latitude).
-template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pass2_kernel(const Args a, const bool vec)
+template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256) void pass2_kernel(const Args a)
 {
     constexpr int U = 2;
     Place<G> pl;
-    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, a.row_idx, TR ? a.scale : 1, vec && sizeof(T) == 4)) return;
+    if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
+    // channels of the inner-loop rows, clamped into the row for the unconditional vector loads
+    const int ka = VEC && pl.ca >= a.ck ? 0 : pl.ca, kb = VEC && pl.cb >= a.ck ? 4 : pl.cb;
+    const int va = VEC && pl.ca >= a.cv ? 0 : pl.ca, vb = VEC && pl.cb >= a.cv ? 4 : pl.cb;
     int64_t z0, z1;
     entry_range<TR>(a, pl.row, z0, z1);
     if (z0 >= z1 && !a.overwrite) return; // nothing sees this latitude
     const long pt0 = ((long)pl.b * a.nlat_halo + pl.row) * a.nlon_kx + pl.x;
     float kr[CPL], vr[CPL], dk[CPL], dv[CPL];
-    load8(kr, static_cast<const T *>(a.k) + pt0 * a.ck, pl.ca, pl.cb, a.ck, vec);
-    load8(vr, static_cast<const T *>(a.v) + pt0 * a.cv, pl.ca, pl.cb, a.cv, vec);
+    load8<T, VEC>(kr, static_cast<const T *>(a.k) + pt0 * a.ck, pl.ca, pl.cb, a.ck);
+    load8<T, VEC>(vr, static_cast<const T *>(a.v) + pt0 * a.cv, pl.ca, pl.cb, a.cv);
 #pragma unroll
     for (int i = 0; i < CPL; i++) dk[i] = dv[i] = 0.f;
     const float wq = z0 < z1 ? a.quad_w[a.lat_halo_start + pl.row] : 0.f; // a padded row outside the grid has no entries and no weight
@@ -431,8 +456,8 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const long o = pt[u] < 0 ? 0 : pt[u];
-                load8(qq[u], qb + o * a.ck, pl.ca, pl.cb, a.ck, vec);
-                load8(gg[u], gb + o * a.cv, pl.ca, pl.cb, a.cv, vec);
+                load8_hot<T, VEC>(qq[u], qb + o * a.ck, ka, kb, a.ck);
+                load8_hot<T, VEC>(gg[u], gb + o * a.cv, va, vb, a.cv);
                 S[u] = a.alpha_sum[obase + o], m[u] = a.qdotk_max[obase + o], In[u] = a.integral_norm[obase + o];
             }
 #pragma unroll
@@ -451,15 +476,15 @@ template <typename T, int G, bool TR> __global__ __launch_bounds__(256) void pas
     if (!pl.valid) return;
     if (!a.overwrite) {
         float cur[CPL];
-        load8(cur, a.dk + pt0 * a.ck, pl.ca, pl.cb, a.ck, vec);
+        load8<float, VEC>(cur, a.dk + pt0 * a.ck, pl.ca, pl.cb, a.ck);
 #pragma unroll
         for (int i = 0; i < CPL; i++) dk[i] += cur[i];
-        load8(cur, a.dv + pt0 * a.cv, pl.ca, pl.cb, a.cv, vec);
+        load8<float, VEC>(cur, a.dv + pt0 * a.cv, pl.ca, pl.cb, a.cv);
 #pragma unroll
         for (int i = 0; i < CPL; i++) dv[i] += cur[i];
     }
-    store8(a.dk + pt0 * a.ck, dk, pl.ca, pl.cb, a.ck, vec);
-    store8(a.dv + pt0 * a.cv, dv, pl.ca, pl.cb, a.cv, vec);
+    store8<VEC>(a.dk + pt0 * a.ck, dk, pl.ca, pl.cb, a.ck);
+    store8<VEC>(a.dv + pt0 * a.cv, dv, pl.ca, pl.cb, a.cv);
 }
 
 #undef S2_RING_TAKE
@@ -595,8 +620,12 @@ template <typename T, int G, bool TR> int launch_g(Step step, const Args &a, hip
     if (step == FWD) vec = vec && al(a.y_acc);
     if (step == PASS1) vec = vec && al(a.dy) && al(a.alpha_k) && al(a.alpha_kvw);
     if (step == PASS2) vec = vec && al(a.dy) && al(a.dk) && al(a.dv);
-    void (*kern)(const Args, const bool) = step == FWD ? fwd_kernel<T, G, TR> : step == PASS1 ? pass1_kernel<T, G, TR> : pass2_kernel<T, G, TR>;
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), 0, stream, a, vec);
+    void (*kern)(const Args) = nullptr;
+    if (vec)
+        kern = step == FWD ? fwd_kernel<T, G, TR, true> : step == PASS1 ? pass1_kernel<T, G, TR, true> : pass2_kernel<T, G, TR, true>;
+    else
+        kern = step == FWD ? fwd_kernel<T, G, TR, false> : step == PASS1 ? pass1_kernel<T, G, TR, false> : pass2_kernel<T, G, TR, false>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(256), 0, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
