@@ -70,10 +70,22 @@ __device__ inline float wave_sum(float x)
     return x;
 }
 
+// x of lane (l ^ 1), (l ^ 2) [quad permutes], (7 - l % 8) [half-row mirror], (15 - l % 16) [row mirror] by data-parallel
+// primitives: no LDS round trip
+template <int CTRL> __device__ inline float dpp_read(float x)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, 0xf, 0xf, false));
+}
+
+// sum over the G lanes of a cell, in every lane of it
 template <int G> __device__ inline float group_sum(float x)
 {
-#pragma unroll
-    for (int o = G / 2; o > 0; o >>= 1) x += __shfl_xor(x, o);
+    x += dpp_read<0xB1>(x); // quad_perm [1, 0, 3, 2]
+    x += dpp_read<0x4E>(x); // quad_perm [2, 3, 0, 1]
+    if constexpr (G >= 8) x += dpp_read<0x141>(x);  // the other quad of the 8 lanes holds its own sum in every lane
+    if constexpr (G >= 16) x += dpp_read<0x140>(x); // likewise the other half of the 16 lanes
+    if constexpr (G >= 32) x += __shfl_xor(x, 16);
+    if constexpr (G >= 64) x += __shfl_xor(x, 32);
     return x;
 }
 
@@ -302,6 +314,7 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
                 load8_hot<T, VEC>(kk[u], kx + p * a.ck, ka, kb, a.ck);
                 load8_hot<T, VEC>(vv[u], vx + p * a.cv, va, vb, a.cv);
             }
+            __builtin_amdgcn_sched_barrier(0); // every load of the step is in flight before the first use
             float mn = m;
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -375,6 +388,7 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
                 load8_hot<T, VEC>(kk[u], kx + p * a.ck, ka, kb, a.ck);
                 load8_hot<T, VEC>(vv[u], vx + p * a.cv, va, vb, a.cv);
             }
+            __builtin_amdgcn_sched_barrier(0); // every load of the step is in flight before the first use
             float mn = m;
 #pragma unroll
             for (int u = 0; u < U; u++) {
@@ -460,6 +474,7 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
                 load8_hot<T, VEC>(gg[u], gb + o * a.cv, va, vb, a.cv);
                 S[u] = a.alpha_sum[obase + o], m[u] = a.qdotk_max[obase + o], In[u] = a.integral_norm[obase + o];
             }
+            __builtin_amdgcn_sched_barrier(0); // every load of the step is in flight before the first use
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 float d = 0.f, e = 0.f;
