@@ -352,7 +352,7 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
 // maximum is the forward's final one and only the three sums are touched (attention_cuda_bwd_ring_upsample.cu:88-160).
 template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256) void pass1_kernel(const Args a)
 {
-    constexpr int U = 2;
+    constexpr int U = 3;
     Place<G> pl;
     if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
@@ -435,7 +435,7 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
 // attention_cuda_bwd_ring_upsample.cu:162-240 (psi as given, keyed by the chunk's own latitude).
 template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256) void pass2_kernel(const Args a)
 {
-    constexpr int U = 2;
+    constexpr int U = 4;
     Place<G> pl;
     if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
