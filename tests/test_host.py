@@ -354,3 +354,30 @@ def test_regrouped_psi_is_a_stable_sort_by_latitude(modulus, key_lo, nkeys):
     assert plan.get_transposed_csr(col, roff, modulus, key_lo, nkeys)[0] is not t_lat
     order = plan.get_row_order(roff)
     assert [int(counts[i]) for i in order.tolist()] == sorted(counts.tolist(), reverse=True)
+
+
+def test_ring_entry_points_reject_bad_arguments_before_touching_the_gpu():
+    lib = _lib.load()
+    ok = _lib.RingShapeStruct(2, 4, 6, 4, 8, 16, 16, 16, 2, 0, 0, _lib.S2ATTN_F32)
+    rs = lambda **kw: _lib.RingShapeStruct(**{**{f: getattr(ok, f) for f, _ in ok._fields_}, **kw})  # noqa: E731
+    null10, null13, null14 = [None] * 10, [None] * 13, [None] * 14
+    assert lib.s2attn_ring_forward_step(*null10, ctypes.byref(ok), None) == -1 and b"null" in lib.s2attn_last_error()
+    assert lib.s2attn_ring_forward_step(*null10, None, None) == -1 and b"shape" in lib.s2attn_last_error()
+    for bad, word in (
+        (rs(pscale=0), b"pscale"),
+        (rs(pscale=3), b"pscale"),  # 16 % 3 != 0
+        (rs(lon_lo_kx=12), b"leaves the input grid"),  # 12 + 6 > 16
+        (rs(nlon_out=9), b"exceeds"),  # 2 * 9 > 16
+        (rs(dtype=5), b"dtype"),
+        (rs(batch=0), b"positive"),
+        (rs(ck=0), b"channel"),
+    ):
+        assert lib.s2attn_ring_backward_pass1(*null13, ctypes.byref(bad), None) == -1 and word in lib.s2attn_last_error(), word
+    assert lib.s2attn_ring_backward_pass2(*null13, ctypes.byref(rs(ck=520)), None) == -2  # unsupported width
+    assert lib.s2attn_ring_backward_pass2_transposed(*null14, ctypes.byref(ok), None) == -1 and b"null" in lib.s2attn_last_error()
+    up = _lib.RingUpShapeStruct(2, 4, 6, 8, 16, 16, 16, 32, 2, 0, -1, _lib.S2ATTN_BF16)
+    us = lambda **kw: _lib.RingUpShapeStruct(**{**{f: getattr(up, f) for f, _ in up._fields_}, **kw})  # noqa: E731
+    assert lib.s2attn_ring_forward_step_upsample(*null10, ctypes.byref(up), None) == -1 and b"null" in lib.s2attn_last_error()
+    for bad, word in ((us(pscale_out=3), b"pscale_out"), (us(nlon_out=33), b"pscale_out"), (us(lon_lo_kx=11), b"leaves the input grid"), (us(dtype=-1), b"dtype")):
+        assert lib.s2attn_ring_backward_pass1_upsample(*[None] * 12, ctypes.byref(bad), None) == -1 and word in lib.s2attn_last_error(), word
+    assert lib.s2attn_ring_backward_pass2_upsample(*null13, ctypes.byref(up), None) == -1 and b"null" in lib.s2attn_last_error()
