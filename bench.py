@@ -301,10 +301,9 @@ def main():
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--config", default="cfg3", choices=sorted(CONFIGS))
-    ap.add_argument("--no-other-configs", action="store_true", help="skip the op-level timings of the other benchmark configurations")
+    ap.add_argument("--no-other-configs", action="store_true", help="skip the op-level timings of the other benchmark configurations and of the ring-step operators")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-module", action="store_true", help="skip the module-level (projections + permutes) timing")
-    ap.add_argument("--no-ring", action="store_true", help="skip the timing of the ring-step operators")
     ap.add_argument("--ring-only", action="store_true", help="time the ring-step operators and nothing else (for profiling)")
     args = ap.parse_args()
 
@@ -489,8 +488,6 @@ def main():
         out["other_configs"] = {
             name: time_other_config(name, dev, cpu=(not args.no_cpu_baseline) and name in ("cfg1", "cfg2")) for name in sorted(CONFIGS) if name != args.config
         }
-
-    if not args.no_ring:
         out["ring_steps"] = time_ring_steps(dev)
 
     if not args.no_cpu_baseline:
