@@ -239,7 +239,10 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
  *   t_lat[z]  (int32)                     the entry's CSR row r (the partner's local latitude)
  *   t_lon[z]  (int32)                     col mod modulus
  * Keys outside [key_lo, key_lo + nkeys) are left out.  The Python operators build these arrays with device operations
- * and cache them per psi.
+ * and cache them per psi; s2attn_ring_regroup_psi does the same on HOST arrays (like s2attn_plan_build: the caller copies
+ * the results to the device): t_lat, t_lon with room for row_off[nrows] entries, t_off [nkeys + 1], t_order [nkeys] (may
+ * be null) = the keys by decreasing number of entries, the row_order argument of the pass 2 entry points.  Returns the
+ * number of entries written or a negative error.
  *
  * Backward pass 2 of the gather direction on the regrouped psi (modulus nlon_in, key_lo = lat_halo_start, nkeys =
  * nlat_halo; t_lat = local output latitude): the same dk, dv as s2attn_ring_backward_pass2
@@ -247,6 +250,9 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
  * row_order (here and in s2attn_ring_backward_pass2_upsample; may be null) lists the nlat_halo chunk latitudes in the
  * order to launch them, the ones with the most entries first, which keeps the end of the launch busy.
  */
+int64_t s2attn_ring_regroup_psi(const int64_t *col_idx, const int64_t *row_off, int nrows, int modulus, int key_lo, int nkeys,
+                                int32_t *t_lat, int32_t *t_lon, int64_t *t_off, int32_t *t_order);
+
 int s2attn_ring_backward_pass2_transposed(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                           const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
                                           const float *quad_weights, const int32_t *t_lat, const int32_t *t_lon,

@@ -348,6 +348,16 @@ def test_regrouped_psi_is_a_stable_sort_by_latitude(modulus, key_lo, nkeys):
     lens = [len(w) for w in want]
     assert sorted(t_order.tolist()) == list(range(nkeys))
     assert [lens[i] for i in t_order.tolist()] == sorted(lens, reverse=True)
+    # the library's host builder gives the same arrays
+    lib = _lib.load()
+    h_lat, h_lon = torch.full((col.numel(),), -7, dtype=torch.int32), torch.full((col.numel(),), -7, dtype=torch.int32)
+    h_off, h_order = torch.zeros(nkeys + 1, dtype=torch.int64), torch.zeros(nkeys, dtype=torch.int32)
+    n = lib.s2attn_ring_regroup_psi(col.data_ptr(), roff.data_ptr(), nrow, modulus, key_lo, nkeys, h_lat.data_ptr(), h_lon.data_ptr(), h_off.data_ptr(), h_order.data_ptr())
+    lo, hi = int(t_off[0]), int(t_off[-1])  # the torch builder keeps every entry and points into the window; the host builder keeps the window only
+    assert n == hi - lo and int(h_off[0]) == 0
+    assert torch.equal(h_off, t_off - lo)
+    assert torch.equal(h_lat[:n], t_lat[lo:hi]) and torch.equal(h_lon[:n], t_lon[lo:hi])
+    assert torch.equal(h_order, t_order)
     again = plan.get_transposed_csr(col, roff, modulus, key_lo, nkeys)
     assert again[0] is t_lat  # served from the cache
     col[0] = (int(col[0]) + modulus) % (6 * 12)  # an in-place edit changes the version counter: rebuilt

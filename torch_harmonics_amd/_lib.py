@@ -93,6 +93,7 @@ SYMBOLS = {
     "s2attn_ring_forward_step": (_int, [_vp] * 10 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_regroup_psi": (_i64, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),
     "s2attn_ring_backward_pass2_transposed": (_int, [_vp] * 14 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_forward_step_upsample": (_int, [_vp] * 10 + [ctypes.POINTER(RingUpShapeStruct), _vp]),
     "s2attn_ring_backward_pass1_upsample": (_int, [_vp] * 12 + [ctypes.POINTER(RingUpShapeStruct), _vp]),

@@ -209,3 +209,42 @@ extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off,
     ndense[1] = order_rows(scost, scatter_order);
     return S2ATTN_OK;
 }
+
+// Regrouped psi for the ring-step kernels (see include/s2attn.h): a stable counting sort of the CSR entries by the
+// latitude named in col, on host arrays like the plan builder.  Entries whose key is outside [key_lo, key_lo + nkeys)
+// are left out; t_lat / t_lon need room for nnz entries.  Returns the number of entries written, or a negative error.
+extern "C" int64_t s2attn_ring_regroup_psi(const int64_t *col_idx, const int64_t *row_off, int nrows, int modulus, int key_lo, int nkeys,
+                                           int32_t *t_lat, int32_t *t_lon, int64_t *t_off, int32_t *t_order)
+{
+    if (!col_idx || !row_off || !t_lat || !t_lon || !t_off) return s2attn_fail(S2ATTN_E_INVALID, "null array pointer");
+    if (nrows < 0 || modulus < 1 || nkeys < 0) return s2attn_fail(S2ATTN_E_INVALID, "nrows and nkeys must not be negative, modulus must be positive");
+    const int64_t nnz = row_off[nrows];
+    for (int r = 0; r < nrows; r++)
+        if (row_off[r] > row_off[r + 1] || row_off[r] < 0) return s2attn_fail(S2ATTN_E_INVALID, "row_off must start at or above 0 and not decrease (row %d)", r);
+    auto key_of = [&](int64_t col) -> int64_t { // floor division: a negative col never maps into the window by accident
+        const int64_t q = col / modulus;
+        return (col % modulus != 0 && col < 0 ? q - 1 : q) - key_lo;
+    };
+    std::vector<int64_t> count((size_t)nkeys + 1, 0);
+    for (int64_t z = 0; z < nnz; z++) {
+        const int64_t k = key_of(col_idx[z]);
+        if (k >= 0 && k < nkeys) count[(size_t)k + 1]++;
+    }
+    for (int i = 0; i < nkeys; i++) count[(size_t)i + 1] += count[(size_t)i];
+    for (int i = 0; i <= nkeys; i++) t_off[i] = count[(size_t)i];
+    std::vector<int64_t> cursor(count.begin(), count.end() - (nkeys >= 0 ? 1 : 0));
+    for (int r = 0; r < nrows; r++) {
+        for (int64_t z = row_off[r]; z < row_off[r + 1]; z++) {
+            const int64_t col = col_idx[z], k = key_of(col);
+            if (k < 0 || k >= nkeys) continue;
+            const int64_t at = cursor[(size_t)k]++;
+            t_lat[at] = r;
+            t_lon[at] = (int32_t)(col - (k + key_lo) * modulus);
+        }
+    }
+    if (t_order) { // keys by decreasing number of entries, ties in key order
+        std::iota(t_order, t_order + nkeys, 0);
+        std::stable_sort(t_order, t_order + nkeys, [&](int32_t a, int32_t b) { return t_off[a + 1] - t_off[a] > t_off[b + 1] - t_off[b]; });
+    }
+    return t_off[nkeys];
+}
