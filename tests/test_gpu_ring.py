@@ -254,3 +254,46 @@ def test_upsample_ring_ops_pass_opcheck():
     torch.library.opcheck(
         ops.backward_ring_step_upsample_pass2, (kc, vc, qd, gd, st["alpha_sum"].clamp_min(1e-30), mx, norm, torch.zeros_like(kc), torch.zeros_like(vc), quad, col_l, roff_l, *tail)
     )
+
+
+def test_pass2_on_psi_regrouped_by_the_host_builder_is_bitwise_the_operator():
+    """s2attn_ring_regroup_psi (host arrays, what a C caller uses) feeds s2attn_ring_backward_pass2_transposed the same entries
+    in the same order as the operator's device-built arrays: identical dk, dv bit for bit."""
+    import ctypes
+
+    from torch_harmonics_amd import _lib, ops
+
+    case = RING_CASES[2]
+    p = local_problem(case, ck=16, cv=8)
+    B, Wi = p["k"].shape[0], p["ins"][1]
+    quad, col_l, roff_l, row_idx = _geo_dev(p)
+    split = ops.split_csr_rows(p["row_idx"], p["roff_l"], p["nlat_loc"])
+    c = 1
+    kc, vc = chunk_of(p, p["k"], c).to(DEV), chunk_of(p, p["v"], c).to(DEV)
+    qd, gd = p["q_l"].to(DEV), p["dy_l"].to(DEV)
+    gen = torch.Generator().manual_seed(5)
+    stat = lambda: (torch.rand(B, p["nlat_loc"], p["nlon_loc"], generator=gen) + 0.5).to(DEV)  # noqa: E731
+    asum, qmax, inorm = stat(), stat(), stat()
+    tail = (Wi, p["pscale"], p["chunks"][c][0], p["halo"][0], p["nlat_loc"], p["nlon_loc"], *split)
+    dk0, dv0 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.backward_ring_step_pass2(kc, vc, qd, gd, asum, qmax, inorm, dk0, dv0, quad, col_l, roff_l, row_idx, *tail)
+
+    lib = _lib.load()
+    nlat_halo, nnz = kc.shape[1], p["col_l"].numel()
+    t_lat, t_lon = torch.zeros(nnz, dtype=torch.int32), torch.zeros(nnz, dtype=torch.int32)
+    t_off, t_order = torch.zeros(nlat_halo + 1, dtype=torch.int64), torch.zeros(nlat_halo, dtype=torch.int32)
+    n = lib.s2attn_ring_regroup_psi(p["col_l"].data_ptr(), p["roff_l"].data_ptr(), p["nlat_loc"], Wi, p["halo"][0], nlat_halo,
+                                    t_lat.data_ptr(), t_lon.data_ptr(), t_off.data_ptr(), t_order.data_ptr())  # fmt: skip
+    assert n >= 0
+    d_lat, d_lon, d_off, d_order = [t.to(DEV) for t in (t_lat, t_lon, t_off, t_order)]
+    shape = _lib.RingShapeStruct(B, nlat_halo, kc.shape[2], p["nlat_loc"], p["nlon_loc"], 16, 8, Wi, p["pscale"], p["chunks"][c][0], p["halo"][0], _lib.S2ATTN_F32)
+    dk1, dv1 = torch.zeros_like(kc), torch.zeros_like(vc)
+    rc = lib.s2attn_ring_backward_pass2_transposed(
+        kc.data_ptr(), vc.data_ptr(), qd.data_ptr(), gd.data_ptr(), asum.data_ptr(), qmax.data_ptr(), inorm.data_ptr(), dk1.data_ptr(), dv1.data_ptr(),
+        quad.data_ptr(), d_lat.data_ptr(), d_lon.data_ptr(), d_off.data_ptr(), d_order.data_ptr(), ctypes.byref(shape),
+        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream),
+    )  # fmt: skip
+    _lib.check(rc, "s2attn_ring_backward_pass2_transposed")
+    torch.cuda.synchronize()
+    assert float(dk0.abs().max()) > 0
+    assert torch.equal(dk0, dk1) and torch.equal(dv0, dv1)
