@@ -129,22 +129,6 @@ template <typename T, bool VEC> __device__ inline void load8(float (&x)[CPL], co
     }
 }
 
-// The same for the rows read in the inner loops.  VEC: no test against n -- the caller passes channels clamped into the
-// row (lanes past the end re-read channels 0 .. 7; what they compute meets a zero operand or is never stored).
-template <typename T, bool VEC> __device__ inline void load8_hot(float (&x)[CPL], const T *row, int ca, int cb, int n)
-{
-    if constexpr (VEC) {
-        if constexpr (sizeof(T) == 4) {
-            const float4 lo = *reinterpret_cast<const float4 *>(row + ca), hi = *reinterpret_cast<const float4 *>(row + cb);
-            x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
-        } else {
-            unpack8(x, row + ca);
-        }
-    } else {
-        load8<T, false>(x, row, ca, cb, n);
-    }
-}
-
 template <bool VEC> __device__ inline void store8(float *row, const float (&x)[CPL], int ca, int cb, int n)
 {
     if constexpr (VEC) {
@@ -236,32 +220,54 @@ template <int G, bool TR> __device__ inline bool scan_entry(const Args &a, int64
     return true;
 }
 
-// partner cell of entry (off, rowbase) for the lane's own cell, or -1.  Regrouped: x = the cell's index in the wavefront,
-// off = the first cell's partner longitude relative to the window.  As given: x = scale * longitude mod N.
-template <bool TR> __device__ inline int partner(const Args &a, int off, int rowbase, int x, bool valid)
+// index of the lane's partner inside the partner row of entry `off` (relative to the window), or -1.  Regrouped: x = the
+// cell's index in the wavefront, off = the first cell's partner longitude relative to the window.  As given: x = scale *
+// longitude mod N.
+template <bool TR> __device__ inline int partner(const Args &a, int off, int x, bool valid)
 {
     if constexpr (TR) {
         int r = off + x;
         if (r >= a.M) r -= a.M;
-        return valid && r < a.win_q ? rowbase + r : -1;
+        return valid && r < a.win_q ? r : -1;
     } else {
         int p = off + x;
         if (p >= a.N) p -= a.N;
         const int rel = p - a.win_lo;
-        return valid && (unsigned)rel < (unsigned)a.win_n ? rowbase + rel : -1;
+        return valid && (unsigned)rel < (unsigned)a.win_n ? rel : -1;
     }
 }
 
-// takes the next surviving entry of the batch: its partner cell for this lane (or -1) and, for W, its quadrature weight
+// takes the next surviving entry of the batch: the start of its partner row (the same for the whole wavefront), this lane's
+// partner inside that row (or -1) and, for W, the entry's quadrature weight
 #define S2_RING_TAKE(u, W)                                                                                               \
     {                                                                                                                    \
         const bool has = cand != 0;                                                                                      \
         const int j = has ? __builtin_ctzll(cand) : 0;                                                                   \
         cand &= cand - 1;                                                                                                \
-        const int oj = __builtin_amdgcn_readlane(off, j), rj = __builtin_amdgcn_readlane(rowbase, j);                    \
+        const int oj = __builtin_amdgcn_readlane(off, j);                                                                \
+        rb[u] = __builtin_amdgcn_readlane(rowbase, j);                                                                   \
         if (W) wgt[u] = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wq), j));                                \
-        pt[u] = has ? partner<TR>(a, oj, rj, xs, pl.valid) : -1;                                                         \
+        pt[u] = has ? partner<TR>(a, oj, xs, pl.valid) : -1;                                                             \
     }
+
+// Channels of row r (an index inside a run of rows that starts at the wavefront-uniform pointer `rows`, n channels each).
+// VEC: the address is the uniform row start plus a 32-bit byte offset per lane (the launcher checks that a run of rows
+// stays below 2 GiB and r below 2^24), which spares the 64-bit address arithmetic per load.
+template <typename T, bool VEC> __device__ inline void load_row(float (&x)[CPL], const T *rows, int r, int n, int ca, int cb)
+{
+    if constexpr (VEC) {
+        const char *base = reinterpret_cast<const char *>(rows);
+        const unsigned o = __umul24((unsigned)r, (unsigned)(n * sizeof(T)));
+        if constexpr (sizeof(T) == 4) {
+            const float4 lo = *reinterpret_cast<const float4 *>(base + (o + 4u * ca)), hi = *reinterpret_cast<const float4 *>(base + (o + 4u * cb));
+            x[0] = lo.x, x[1] = lo.y, x[2] = lo.z, x[3] = lo.w, x[4] = hi.x, x[5] = hi.y, x[6] = hi.z, x[7] = hi.w;
+        } else {
+            unpack8(x, reinterpret_cast<const T *>(base + (o + 2u * ca)));
+        }
+    } else {
+        load8<T, false>(x, rows + (size_t)r * n, ca, cb, n);
+    }
+}
 
 // entries of the owner's latitude `row`
 template <bool TR> __device__ inline void entry_range(const Args &a, int row, int64_t &z0, int64_t &z1)
@@ -285,7 +291,8 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
     Place<G> pl;
     if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
-    // channels of the inner-loop rows, clamped into the row for the unconditional vector loads
+    // channels of the inner-loop rows, clamped into the row: the vector loads there are unconditional (lanes past the end
+    // re-read channels 0 .. 7; what they compute meets a zero operand or is never stored)
     const int ka = VEC && pl.ca >= a.ck ? 0 : pl.ca, kb = VEC && pl.cb >= a.ck ? 4 : pl.cb;
     const int va = VEC && pl.ca >= a.cv ? 0 : pl.ca, vb = VEC && pl.cb >= a.cv ? 4 : pl.cb;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
@@ -304,15 +311,15 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
         const float wq = partner_weight<TR>(a, ok, lat);
         unsigned long long cand = __ballot(ok);
         while (cand) {
-            int pt[U];
+            int pt[U], rb[U];
             float wgt[U], kk[U][CPL], vv[U][CPL], s[U];
 #pragma unroll
             for (int u = 0; u < U; u++) S2_RING_TAKE(u, true)
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const long p = pt[u] < 0 ? 0 : pt[u];
-                load8_hot<T, VEC>(kk[u], kx + p * a.ck, ka, kb, a.ck);
-                load8_hot<T, VEC>(vv[u], vx + p * a.cv, va, vb, a.cv);
+                const int r = pt[u] < 0 ? 0 : pt[u];
+                load_row<T, VEC>(kk[u], kx + (long)rb[u] * a.ck, r, a.ck, ka, kb);
+                load_row<T, VEC>(vv[u], vx + (long)rb[u] * a.cv, r, a.cv, va, vb);
             }
             __builtin_amdgcn_sched_barrier(0); // every load of the step is in flight before the first use
             float mn = m;
@@ -324,11 +331,12 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
                 s[u] = group_sum<G>(d);
                 if (pt[u] >= 0) mn = fmaxf(mn, s[u]);
             }
-            if (mn == -INFINITY) continue; // nothing seen yet and nothing in these entries (the same in a whole lane group)
-            const float corr = __expf(m - mn); // m = -inf before the first neighbor: 0
-            S *= corr;
+            if (__any(mn > m)) { // a maximum moved somewhere in the wavefront; m = -inf before the first neighbor: factor 0
+                const float corr = mn > m ? __expf(m - mn) : 1.f;
+                S *= corr;
 #pragma unroll
-            for (int i = 0; i < CPL; i++) y[i] *= corr;
+                for (int i = 0; i < CPL; i++) y[i] *= corr;
+            }
 #pragma unroll
             for (int u = 0; u < U; u++) {
                 const float alpha = pt[u] >= 0 ? __expf(s[u] - mn) * wgt[u] : 0.f;
@@ -356,7 +364,8 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
     Place<G> pl;
     if (!pl.locate(a.B, a.Ho, a.Wo, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
-    // channels of the inner-loop rows, clamped into the row for the unconditional vector loads
+    // channels of the inner-loop rows, clamped into the row: the vector loads there are unconditional (lanes past the end
+    // re-read channels 0 .. 7; what they compute meets a zero operand or is never stored)
     const int ka = VEC && pl.ca >= a.ck ? 0 : pl.ca, kb = VEC && pl.cb >= a.ck ? 4 : pl.cb;
     const int va = VEC && pl.ca >= a.cv ? 0 : pl.ca, vb = VEC && pl.cb >= a.cv ? 4 : pl.cb;
     const long out = ((long)pl.b * a.Ho + pl.row) * a.Wo + pl.x;
@@ -378,15 +387,15 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
         const float wq = partner_weight<TR>(a, ok, lat);
         unsigned long long cand = __ballot(ok);
         while (cand) {
-            int pt[U];
+            int pt[U], rb[U];
             float wgt[U], kk[U][CPL], vv[U][CPL], s[U], gv[U];
 #pragma unroll
             for (int u = 0; u < U; u++) S2_RING_TAKE(u, true)
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const long p = pt[u] < 0 ? 0 : pt[u];
-                load8_hot<T, VEC>(kk[u], kx + p * a.ck, ka, kb, a.ck);
-                load8_hot<T, VEC>(vv[u], vx + p * a.cv, va, vb, a.cv);
+                const int r = pt[u] < 0 ? 0 : pt[u];
+                load_row<T, VEC>(kk[u], kx + (long)rb[u] * a.ck, r, a.ck, ka, kb);
+                load_row<T, VEC>(vv[u], vx + (long)rb[u] * a.cv, r, a.cv, va, vb);
             }
             __builtin_amdgcn_sched_barrier(0); // every load of the step is in flight before the first use
             float mn = m;
@@ -399,9 +408,8 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
                 gv[u] = group_sum<G>(e);
                 if (pt[u] >= 0 && !fixed) mn = fmaxf(mn, s[u]);
             }
-            if (mn == -INFINITY) continue;
-            if (!fixed) {
-                const float corr = __expf(m - mn);
+            if (__any(mn > m)) { // never with a fixed maximum
+                const float corr = mn > m ? __expf(m - mn) : 1.f;
                 S *= corr, I *= corr;
 #pragma unroll
                 for (int i = 0; i < CPL; i++) ak[i] *= corr, akg[i] *= corr;
@@ -439,7 +447,8 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
     Place<G> pl;
     if (!pl.locate(a.B, a.nlat_halo, a.nlon_kx, a.row_idx, TR ? a.scale : 1, VEC && sizeof(T) == 4)) return;
     const int lane = threadIdx.x & 63;
-    // channels of the inner-loop rows, clamped into the row for the unconditional vector loads
+    // channels of the inner-loop rows, clamped into the row: the vector loads there are unconditional (lanes past the end
+    // re-read channels 0 .. 7; what they compute meets a zero operand or is never stored)
     const int ka = VEC && pl.ca >= a.ck ? 0 : pl.ca, kb = VEC && pl.cb >= a.ck ? 4 : pl.cb;
     const int va = VEC && pl.ca >= a.cv ? 0 : pl.ca, vb = VEC && pl.cb >= a.cv ? 4 : pl.cb;
     int64_t z0, z1;
@@ -462,17 +471,18 @@ template <typename T, int G, bool TR, bool VEC> __global__ __launch_bounds__(256
         const bool ok = scan_entry<G, TR>(a, zb + lane, z1, xs0, a.Ho, a.Wo, off, rowbase, lat);
         unsigned long long cand = __ballot(ok);
         while (cand) {
-            int pt[U];
+            int pt[U], rb[U];
             float wgt[1], qq[U][CPL], gg[U][CPL], S[U], m[U], In[U];
             (void)wgt;
 #pragma unroll
             for (int u = 0; u < U; u++) S2_RING_TAKE(u, false)
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const long o = pt[u] < 0 ? 0 : pt[u];
-                load8_hot<T, VEC>(qq[u], qb + o * a.ck, ka, kb, a.ck);
-                load8_hot<T, VEC>(gg[u], gb + o * a.cv, va, vb, a.cv);
-                S[u] = a.alpha_sum[obase + o], m[u] = a.qdotk_max[obase + o], In[u] = a.integral_norm[obase + o];
+                const int r = pt[u] < 0 ? 0 : pt[u];
+                load_row<T, VEC>(qq[u], qb + (long)rb[u] * a.ck, r, a.ck, ka, kb);
+                load_row<T, VEC>(gg[u], gb + (long)rb[u] * a.cv, r, a.cv, va, vb);
+                const long o = obase + rb[u] + r;
+                S[u] = a.alpha_sum[o], m[u] = a.qdotk_max[o], In[u] = a.integral_norm[o];
             }
             __builtin_amdgcn_sched_barrier(0); // every load of the step is in flight before the first use
 #pragma unroll
@@ -629,6 +639,9 @@ template <typename T, int G, bool TR> int launch_g(Step step, const Args &a, hip
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
     if ((long)a.nlat_halo * a.nlon_kx > 0x7fffffffL || (long)a.Ho * a.Wo > 0x7fffffffL)
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "more than 2^31 points per batch entry");
+    const long wmax = a.nlon_kx > a.Wo ? a.nlon_kx : a.Wo; // 32-bit byte offsets inside one latitude row
+    if (wmax >= (1L << 24) || wmax * (a.ck > a.cv ? a.ck : a.cv) * 4 > 0x7fffffffL)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "a latitude row of %ld points is too long", wmax);
     // 16-byte rows: vector loads and stores
     auto al = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
     bool vec = a.ck % CPL == 0 && a.cv % CPL == 0 && al(a.k) && al(a.v) && al(a.q);
