@@ -194,7 +194,8 @@ int s2attn_permute_to_nchw(const void *src, void *dst, int64_t B, int64_t H, int
  *                                                      input longitudes lon_lo_kx .. + nlon_kx
  *   q, dy        [batch, nlat_out, nlon_out, ck / cv]   local output points
  *   y_acc        [batch, nlat_out, nlon_out, cv] fp32;  alpha_sum, qdotk_max, integral(_norm) [batch, nlat_out, nlon_out] fp32
- *   alpha_k, alpha_kvw [batch, nlat_out, nlon_out, ck] fp32;   dk, dv: fp32, shaped like k, v (ADDED to, atomically)
+ *   alpha_k, alpha_kvw [batch, nlat_out, nlon_out, ck] fp32;   dk, dv: fp32, shaped like k, v (ADDED to; with fp32 atomics
+ *                                                      in s2attn_ring_backward_pass2, plainly in ..._pass2_transposed)
  *   quad_weights [global nlat_in] fp32, indexed by global input latitude
  *   col_idx, row_off: the local CSR in device memory, int64: row_off has nlat_out + 1 entries, col_idx = hi_global *
  *     nlon_in + wi with wi already shifted by pscale * (first local output longitude); row_idx (int32, nlat_out entries,
