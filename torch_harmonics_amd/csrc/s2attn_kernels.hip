@@ -34,6 +34,14 @@
 
 #include "s2attn_internal.h"
 
+// This file is compiled three times (see the Makefile), so that the three groups of kernel instantiations build side by
+// side: S2_PART 1 = everything but the launchers of the 16-longitude matrix-core families, 2 = the 16-bit family
+// (s2attn_h16.hpp), 3 = the fp32 family (s2attn_m32.hpp).  S2_PART 0 (the default) is the whole library in one unit.
+#ifndef S2_PART
+#define S2_PART 0
+#endif
+
+#if S2_PART <= 1
 // ---------------------------------------------------------------------------------
 // error reporting
 // ---------------------------------------------------------------------------------
@@ -50,6 +58,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
 extern "C" int s2attn_abi_version(void) { return 7; }
+#endif
 
 namespace s2 {
 
@@ -2388,6 +2397,106 @@ template <typename E> __global__ __launch_bounds__(256) void transpose_kernel(co
 } // namespace s2
 
 // ---------------------------------------------------------------------------------
+// launchers of the two 16-longitude matrix-core families: declared everywhere, defined (and instantiated for every
+// shape the dispatch below names) in their own compilation of this file
+// ---------------------------------------------------------------------------------
+namespace s2 {
+
+enum Which { FWD, DQ, DKDV };
+
+template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream);
+template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream);
+
+#if S2_PART == 0 || S2_PART == 2
+// 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
+// dq pass exists only in the form that takes the forward's y and lse.
+template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream)
+{
+    if constexpr (std::is_same<T, float>::value) {
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "16-bit kernels asked for fp32 storage");
+    } else {
+        Args a = a0;
+        a.row_first = 0;
+        void (*kern)(const Args) = nullptr;
+        long nblocks = 0;
+        if (which == FWD) {
+            kern = fwd_h16_kernel<T, D, PAD>;
+            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+        } else if (which == DQ) {
+            kern = dq_h16_kernel<T, D, PAD>;
+            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+        } else {
+            kern = dkdv_h16_kernel<T, D, PAD>;
+            nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
+        }
+        if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+        return S2ATTN_OK;
+    }
+}
+#endif
+#if S2_PART == 2
+#define S2_H16_INSTANCES(T)                                                      \
+    template int launch_h16<T, 32, false>(Which, const Args &, hipStream_t);    \
+    template int launch_h16<T, 64, false>(Which, const Args &, hipStream_t);    \
+    template int launch_h16<T, 128, false>(Which, const Args &, hipStream_t);   \
+    template int launch_h16<T, 32, true>(Which, const Args &, hipStream_t);     \
+    template int launch_h16<T, 64, true>(Which, const Args &, hipStream_t);     \
+    template int launch_h16<T, 128, true>(Which, const Args &, hipStream_t);    \
+    template int launch_h16<T, 256, true>(Which, const Args &, hipStream_t);
+S2_H16_INSTANCES(bf16_t)
+S2_H16_INSTANCES(f16_t)
+S2_H16_INSTANCES(float) // never reached (fp32 storage takes the other families); only its error return is compiled
+#undef S2_H16_INSTANCES
+#endif
+
+#if S2_PART == 0 || S2_PART == 3
+// fp32 16-longitude matrix-core kernels, tiles of 16, 32, 64 or 128 channels: same launch geometry and the same conditions as the 16-bit family.
+template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream)
+{
+    Args a = a0;
+    a.row_first = 0;
+    void (*kern)(const Args) = nullptr;
+    long nblocks = 0;
+    int lds = NS > 1 ? m32_lds_bytes<D, NS>(false) : 0; // one wavefront per workgroup: static LDS
+    if (which == FWD) {
+        kern = fwd_m32_kernel<D, NS>;
+        nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+    } else if (which == DQ) {
+        kern = dq_m32_kernel<D, NS>;
+        nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+    } else {
+        kern = dkdv_m32_kernel<D, NS>;
+        nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
+        lds = NS > 1 ? m32_lds_bytes<D, NS>(true) : 0;
+    }
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    if (lds > 48 * 1024) {
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * NS), lds, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+#endif
+#if S2_PART == 3
+template int launch_m32<16, 1>(Which, const Args &, hipStream_t);
+template int launch_m32<32, 1>(Which, const Args &, hipStream_t);
+template int launch_m32<64, 1>(Which, const Args &, hipStream_t);
+template int launch_m32<128, 1>(Which, const Args &, hipStream_t);
+template int launch_m32<128, 2>(Which, const Args &, hipStream_t);
+template int launch_m32<128, 3>(Which, const Args &, hipStream_t);
+template int launch_m32<128, 4>(Which, const Args &, hipStream_t);
+#endif
+
+} // namespace s2
+
+#if S2_PART <= 1
+// ---------------------------------------------------------------------------------
 // host side
 // ---------------------------------------------------------------------------------
 namespace {
@@ -2417,8 +2526,6 @@ int check_shape(const s2attn_shape *sh)
 int esize(int dtype) { return dtype == S2ATTN_F32 ? 4 : 2; }
 
 bool aligned(const void *p, size_t n) { return (reinterpret_cast<uintptr_t>(p) % n) == 0; }
-
-enum Which { FWD, DQ, DKDV };
 
 template <typename T, int P, bool VEC> int launch_one(Which which, const Args &a0, int row_first, int row_count, hipStream_t stream)
 {
@@ -2531,35 +2638,6 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
     return S2ATTN_OK;
 }
 
-// 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
-// dq pass exists only in the form that takes the forward's y and lse.
-template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream)
-{
-    if constexpr (std::is_same<T, float>::value) {
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "16-bit kernels asked for fp32 storage");
-    } else {
-        Args a = a0;
-        a.row_first = 0;
-        void (*kern)(const Args) = nullptr;
-        long nblocks = 0;
-        if (which == FWD) {
-            kern = fwd_h16_kernel<T, D, PAD>;
-            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
-        } else if (which == DQ) {
-            kern = dq_h16_kernel<T, D, PAD>;
-            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
-        } else {
-            kern = dkdv_h16_kernel<T, D, PAD>;
-            nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
-        }
-        if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
-        const hipError_t e = hipGetLastError();
-        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
-        return S2ATTN_OK;
-    }
-}
-
 // Head widths: any multiple of 8 from 16 to 256, staged in a tile of 32, 64, 128 or 256 channels (zeros past the head).
 bool h16_width(int ck, int cv) { return ck == cv && ck % 8 == 0 && ck >= 16 && ck <= 256; }
 
@@ -2572,36 +2650,6 @@ template <typename T> bool h16_ok(Which which, const Args &a)
     for (const void *p : ptrs)
         if (p && !aligned(p, 16)) return false;
     return true;
-}
-
-// fp32 16-longitude matrix-core kernels, tiles of 16, 32, 64 or 128 channels: same launch geometry and the same conditions as the 16-bit family.
-template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream)
-{
-    Args a = a0;
-    a.row_first = 0;
-    void (*kern)(const Args) = nullptr;
-    long nblocks = 0;
-    int lds = NS > 1 ? m32_lds_bytes<D, NS>(false) : 0; // one wavefront per workgroup: static LDS
-    if (which == FWD) {
-        kern = fwd_m32_kernel<D, NS>;
-        nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
-    } else if (which == DQ) {
-        kern = dq_m32_kernel<D, NS>;
-        nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
-    } else {
-        kern = dkdv_m32_kernel<D, NS>;
-        nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
-        lds = NS > 1 ? m32_lds_bytes<D, NS>(true) : 0;
-    }
-    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    if (lds > 48 * 1024) {
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
-        if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
-    }
-    hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * NS), lds, stream, a);
-    const hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
-    return S2ATTN_OK;
 }
 
 // Head widths: any multiple of 4 from 16 to 512, staged in a tile of 16, 32, 64 or 128 channels (zeros past the head), or in
@@ -2874,3 +2922,4 @@ extern "C" int s2attn_permute_to_nchw(const void *src, void *dst, int64_t B, int
 {
     return permute(src, dst, B, H * W, C, elem_size, stream); // [HW, C] -> [C, HW]
 }
+#endif // S2_PART <= 1
