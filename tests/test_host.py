@@ -391,3 +391,16 @@ def test_ring_entry_points_reject_bad_arguments_before_touching_the_gpu():
     for bad, word in ((us(pscale_out=3), b"pscale_out"), (us(nlon_out=33), b"pscale_out"), (us(lon_lo_kx=11), b"leaves the input grid"), (us(dtype=-1), b"dtype")):
         assert lib.s2attn_ring_backward_pass1_upsample(*[None] * 12, ctypes.byref(bad), None) == -1 and word in lib.s2attn_last_error(), word
     assert lib.s2attn_ring_backward_pass2_upsample(*null13, ctypes.byref(up), None) == -1 and b"null" in lib.s2attn_last_error()
+
+
+def test_bench_refuses_more_than_one_gpu_with_a_message():
+    """bench.py measures one GPU; --gpus N > 1 (or a multi-rank environment) exits with a message that says so, before any GPU use."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for argv, env in ((["--gpus", "2"], {}), ([], {"WORLD_SIZE": "4"})):
+        proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *argv], capture_output=True, text=True, env={**os.environ, **env}, timeout=300)
+        assert proc.returncode == 2
+        assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
