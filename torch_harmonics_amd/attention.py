@@ -31,6 +31,10 @@ def _weight_grad(g: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     slices = max(1, min(64, n // 8192))
     if slices == 1:
         return g.t() @ x
+    for s in range(slices, slices // 2, -1):  # a slice count that divides n leaves no remainder GEMM and no extra add
+        if n % s == 0:
+            slices = s
+            break
     rows = n // slices
     main = slices * rows
     out = torch.bmm(g[:main].view(slices, rows, -1).transpose(1, 2), x[:main].view(slices, rows, -1)).sum(0)
