@@ -297,3 +297,37 @@ def test_pass2_on_psi_regrouped_by_the_host_builder_is_bitwise_the_operator():
     torch.cuda.synchronize()
     assert float(dk0.abs().max()) > 0
     assert torch.equal(dk0, dk1) and torch.equal(dv0, dv1)
+
+
+def test_ring_steps_with_an_empty_local_psi_are_no_ops():
+    """A rank whose output rows see no input point at all (an empty col_idx): every step returns without touching the state; pass 2
+    of the up-sampling direction still writes every element (zeros)."""
+    from torch_harmonics_amd import ops
+
+    B, ck, cv, Ho, Wo, Hh, Wk = 2, 8, 8, 3, 6, 4, 5
+    z = lambda *s: torch.zeros(*s, device=DEV)  # noqa: E731
+    kc, vc, q, dy = torch.randn(B, Hh, Wk, ck, device=DEV), torch.randn(B, Hh, Wk, cv, device=DEV), torch.randn(B, Ho, Wo, ck, device=DEV), torch.randn(B, Ho, Wo, cv, device=DEV)
+    quad = torch.ones(16, device=DEV)
+    col = torch.zeros(0, dtype=torch.int64, device=DEV)
+    roff, row_idx = torch.zeros(Ho + 1, dtype=torch.int64, device=DEV), torch.arange(Ho, dtype=torch.int32, device=DEV)
+    st = fresh_state(B, Ho, Wo, ck, cv, torch.float32, DEV)
+    tail = (12, 2, 3, 0, Ho, Wo, 0, 0, 0)
+    ops.forward_ring_step(kc, vc, q, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col, roff, row_idx, *tail)
+    ops.backward_ring_step_pass1(kc, vc, q, dy, st["alpha_sum"], st["qdotk_max"], st["integral"], st["alpha_k"], st["alpha_kvw"], quad, col, roff, row_idx, *tail)
+    dk, dv = torch.full_like(kc, 2.0), torch.full_like(vc, 3.0)
+    ops.backward_ring_step_pass2(kc, vc, q, dy, st["alpha_sum"] + 1, st["qdotk_max"].clamp_min(0), z(B, Ho, Wo), dk, dv, quad, col, roff, row_idx, *tail)
+    torch.cuda.synchronize()
+    assert float(st["y_acc"].abs().max()) == 0 and float(st["alpha_sum"].abs().max()) == 0 and bool(torch.isinf(st["qdotk_max"]).all())
+    assert float(st["integral"].abs().max()) == 0 and float(st["alpha_k"].abs().max()) == 0
+    assert bool((dk == 2.0).all()) and bool((dv == 3.0).all())  # the gather direction ADDS: untouched
+    # up-sampling direction: psi keyed by the chunk's input latitudes
+    roff_up = torch.zeros(Hh + 1, dtype=torch.int64, device=DEV)
+    up_tail = (6, 12, 2, 0, 0, Ho, Wo)
+    st = fresh_state(B, Ho, Wo, ck, cv, torch.float32, DEV)
+    ops.forward_ring_step_upsample(kc, vc, q, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col, roff_up, *up_tail)
+    ops.backward_ring_step_upsample_pass1(kc, vc, q, dy, st["qdotk_max"], st["integral"], st["alpha_k"], st["alpha_kvw"], quad, col, roff_up, *up_tail)
+    dk, dv = torch.full_like(kc, float("nan")), torch.full_like(vc, float("nan"))
+    ops.backward_ring_step_upsample_pass2(kc, vc, q, dy, st["alpha_sum"] + 1, st["qdotk_max"].clamp_min(0), z(B, Ho, Wo), dk, dv, quad, col, roff_up, *up_tail)
+    torch.cuda.synchronize()
+    assert float(st["y_acc"].abs().max()) == 0 and float(st["alpha_sum"].abs().max()) == 0 and float(st["integral"].abs().max()) == 0
+    assert float(dk.abs().max()) == 0 and float(dv.abs().max()) == 0

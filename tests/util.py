@@ -35,6 +35,8 @@ def assert_close(name, got, want, rtol, atol):
     got = got.detach().double().cpu()
     want = want.detach().double().cpu()
     assert got.shape == want.shape, f"{name}: shape {tuple(got.shape)} vs {tuple(want.shape)}"
+    if got.numel() == 0:
+        return
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
     err = (got - want).abs()
     bound = atol + rtol * want.abs()

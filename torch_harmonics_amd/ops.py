@@ -489,7 +489,7 @@ def forward_ring_step(
 ) -> None:
     state = (("y_acc", y_acc, vx.shape[3]), ("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None))
     _ring_validate(kx, vx, qy, None, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out)
-    if qy.numel() == 0 or kx.numel() == 0:
+    if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:  # nothing to fold in
         return
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
     with torch.cuda.device(kx.device):
@@ -536,7 +536,7 @@ def backward_ring_step_pass1(
     state = (("alpha_sum_buf", alpha_sum_buf, None), ("qdotk_max_buf", qdotk_max_buf, None), ("integral_buf", integral_buf, None),
              ("alpha_k_buf", alpha_k_buf, ck), ("alpha_kvw_buf", alpha_kvw_buf, ck))  # fmt: skip
     _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out)
-    if qy.numel() == 0 or kx.numel() == 0:
+    if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:  # nothing to fold in
         return
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
     with torch.cuda.device(kx.device):
@@ -727,7 +727,7 @@ def backward_ring_step_upsample_pass2(
         _require_gpu(t, name, kx.device)
     if kx.numel() == 0:
         return
-    if qy.numel() == 0:
+    if qy.numel() == 0 or col_idx.numel() == 0:  # no output cell sees the chunk: the step still writes every element
         dkx.zero_()
         dvx.zero_()
         return
