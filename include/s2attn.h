@@ -76,6 +76,10 @@ int s2attn_abi_version(void);
  *     gather_off  [nvout+1]   gather_runs  [4*nruns]   gather_order  [nvout]
  *     scatter_off [nvin+1]    scatter_runs [4*nruns]   scatter_order [nvin]
  *     ndense [2]  number of long-run latitudes at the front of gather_order and of scatter_order
+ *     gather_order_mixed [nvout], scatter_order_mixed [nvin]  (either may be null) the same latitudes with the long-run and
+ *                 the short-run ones interleaved in proportion to their work: the launch order of the kernels that put
+ *                 long runs on the matrix cores and short runs on the vector ALU (fp32 heads of 32 channels on at least
+ *                 64 longitudes), so that both kinds of workgroups share a SIMD for the whole launch
  * The caller copies the six arrays to the device and passes them, with the two counts, in s2attn_plan.
  */
 int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
@@ -84,7 +88,7 @@ int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_
 int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
                       int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
                       int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order,
-                      int32_t *ndense);
+                      int32_t *ndense, int32_t *gather_order_mixed, int32_t *scatter_order_mixed);
 
 typedef struct s2attn_plan {
     const int32_t *gather_off;    /* device, [nvout+1]  */
@@ -94,8 +98,10 @@ typedef struct s2attn_plan {
     const int32_t *scatter_runs;  /* device, [4*nruns]  (backward only) */
     const int32_t *scatter_order; /* device, [nvin]     (backward only) */
     int64_t nruns;
-    int32_t gather_ndense;  /* leading entries of gather_order that go to the dense kernels  */
-    int32_t scatter_ndense; /* leading entries of scatter_order that go to the dense kernels */
+    int32_t gather_ndense;  /* leading entries of gather_order that are long-run latitudes  */
+    int32_t scatter_ndense; /* leading entries of scatter_order that are long-run latitudes */
+    const int32_t *gather_order_mixed;  /* device, [nvout], may be null: see s2attn_plan_build */
+    const int32_t *scatter_order_mixed; /* device, [nvin],  may be null */
 } s2attn_plan;
 
 typedef struct s2attn_shape {

@@ -404,3 +404,24 @@ def test_bench_refuses_more_than_one_gpu_with_a_message():
         proc = subprocess.run([sys.executable, os.path.join(root, "bench.py"), *argv], capture_output=True, text=True, env={**os.environ, **env}, timeout=300)
         assert proc.returncode == 2
         assert "one GPU" in proc.stderr and proc.stdout.strip() == ""
+
+
+def test_mixed_launch_order_is_the_same_latitudes_interleaved_by_work():
+    """gather_order_mixed / scatter_order_mixed: permutations of the latitudes in which the long-run list and the short-run list
+    each keep their own order, both are spread over the whole launch, and neither list's handed-out share of work runs ahead of
+    the other's by more than one latitude."""
+    from oracle import geometry as ogeo
+
+    ins = outs = (48, 96)
+    col, roff = ogeo.neighborhood_csr(ins, outs, "equiangular", "equiangular", 3 * torch.pi / 47)
+    arrays, nruns, ndense, mixed = build_host_plan(col, roff, ins[0], ins[1], outs[0], outs[1], with_mixed=True)
+    plain = build_host_plan(col, roff, ins[0], ins[1], outs[0], outs[1])
+    assert all(torch.equal(a, b) for a, b in zip(arrays, plain[0])) and plain[1:] == (nruns, ndense)
+    for order, mix, nd in ((arrays[2], mixed[0], ndense[0]), (arrays[5], mixed[1], ndense[1])):
+        order, mix = order.tolist(), mix.tolist()
+        assert sorted(mix) == list(range(len(order)))
+        assert 0 < nd < len(order), "the case must have both kinds of latitudes"
+        dense, vec = order[:nd], order[nd:]
+        assert [r for r in mix if r in set(dense)] == dense and [r for r in mix if r in set(vec)] == vec
+        where_dense = [i for i, r in enumerate(mix) if r in set(dense)]
+        assert where_dense[0] <= 1 and where_dense[-1] >= len(mix) // 2  # spread out, not a prefix

@@ -15,7 +15,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -33,6 +33,8 @@ class PlanStruct(ctypes.Structure):
         ("nruns", _i64),
         ("gather_ndense", ctypes.c_int32),
         ("scatter_ndense", ctypes.c_int32),
+        ("gather_order_mixed", _vp),
+        ("scatter_order_mixed", _vp),
     ]
 
 
@@ -79,7 +81,7 @@ SYMBOLS = {
     "s2attn_last_error": (ctypes.c_char_p, []),
     "s2attn_abi_version": (_int, []),
     "s2attn_plan_count": (_i64, [_vp, _vp, _i64, _int, _int, _int, _int]),
-    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_forward_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_saved": (_int, [_vp] * 11 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),

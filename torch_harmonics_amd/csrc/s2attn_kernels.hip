@@ -57,7 +57,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 7; }
+extern "C" int s2attn_abi_version(void) { return 8; }
 #endif
 
 namespace s2 {
@@ -276,6 +276,7 @@ struct Args {
     const void *ysaved; // backward with saved statistics: the forward output
     const float *quad_w;
     const int *goff, *gorder, *soff, *sorder;
+    const int *gorder_mixed, *sorder_mixed; // launch orders for the hybrid kernels (may be null)
     const Run *gruns, *sruns;
     int B, nh, Hi, Wi, Ho, Wo, dk_, dv_;
     int kps; // nlon_in / nlon_out when the input grid is the finer one, else 1; see key_point()
@@ -2619,6 +2620,9 @@ template <typename T> int launch_dense(Which which, const Args &a0, int row_coun
     if (row_count <= 0) return S2ATTN_OK;
     Args a = a0;
     a.row_first = 0;
+    // long-run and short-run latitudes interleaved: matrix-core-heavy and vector-heavy workgroups side by side
+    if (a.gorder_mixed) a.gorder = a.gorder_mixed;
+    if (a.sorder_mixed) a.sorder = a.sorder_mixed;
     void (*kern)(const Args) = nullptr;
     long nblocks = 0;
     if (which == FWD) {
@@ -2719,6 +2723,8 @@ void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const f
     a.soff = plan->scatter_off;
     a.sruns = reinterpret_cast<const Run *>(plan->scatter_runs);
     a.sorder = plan->scatter_order;
+    a.gorder_mixed = plan->gather_order_mixed;
+    a.sorder_mixed = plan->scatter_order_mixed;
     a.B = sh->batch;
     a.nh = sh->num_heads;
     const bool up = sh->nlon_out % sh->nlon_in == 0 && sh->nlon_out != sh->nlon_in;

@@ -23,10 +23,11 @@ _lock = threading.Lock()
 
 
 class Plan:
-    """Six int32 arrays on one device plus the ctypes view the library takes."""
+    """Six int32 arrays plus the two interleaved launch orders on one device, and the ctypes view the library takes."""
 
-    def __init__(self, arrays, nruns, ndense, keepalive):
+    def __init__(self, arrays, nruns, ndense, keepalive, mixed):
         self.gather_off, self.gather_runs, self.gather_order, self.scatter_off, self.scatter_runs, self.scatter_order = arrays
+        self.gather_order_mixed, self.scatter_order_mixed = mixed
         self.nruns = nruns
         self.gather_ndense, self.scatter_ndense = ndense
         self._keepalive = keepalive
@@ -40,17 +41,21 @@ class Plan:
             nruns,
             self.gather_ndense,
             self.scatter_ndense,
+            self.gather_order_mixed.data_ptr(),
+            self.scatter_order_mixed.data_ptr(),
         )
 
 
-def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int):
+def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int, with_mixed: bool = False):
     """
     Runs the library's host builder on CPU copies of the CSR.  Returns
     ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns, (gather_ndense, scatter_ndense))
     as CPU int32 tensors; gather_runs has shape (nruns, 4) = (virtual input latitude, ws, len, real input latitude),
     grouped by virtual output latitude; scatter_runs (virtual output latitude, ws, len, real output latitude), grouped by
     virtual input latitude.  Virtual latitude = real latitude * ratio + column class on the finer of the two grids (see
-    include/s2attn.h); the first *_ndense entries of each order are the latitudes with long runs.
+    include/s2attn.h); the first *_ndense entries of each order are the latitudes with long runs.  with_mixed: a fourth
+    element (gather_order_mixed, scatter_order_mixed), the same latitudes with long-run and short-run ones interleaved in
+    proportion to their work (the launch order of the kernels that split their work between matrix cores and vector ALU).
     """
     lib = _lib.load()
     ci = col_idx.detach().to(device="cpu", dtype=torch.int64).contiguous()
@@ -73,8 +78,14 @@ def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, 
         torch.zeros(nvin, dtype=torch.int32),
     ]
     ndense = torch.zeros(2, dtype=torch.int32)
-    rc = lib.s2attn_plan_build(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays], ndense.data_ptr())
+    mixed = (torch.zeros(nvout, dtype=torch.int32), torch.zeros(nvin, dtype=torch.int32))
+    rc = lib.s2attn_plan_build(
+        ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays], ndense.data_ptr(),
+        mixed[0].data_ptr() if with_mixed else None, mixed[1].data_ptr() if with_mixed else None,
+    )  # fmt: skip
     _lib.check(rc, "s2attn_plan_build")
+    if with_mixed:
+        return arrays, int(nruns), (int(ndense[0]), int(ndense[1])), mixed
     return arrays, int(nruns), (int(ndense[0]), int(ndense[1]))
 
 
@@ -98,9 +109,9 @@ def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in
         if plan is not None:
             _cache.move_to_end(key)
             return plan
-    arrays, nruns, ndense = build_host_plan(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    arrays, nruns, ndense, mixed = build_host_plan(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out, with_mixed=True)
     dev = col_idx.device
-    plan = Plan([a.to(dev) for a in arrays], nruns, ndense, (col_idx, row_off))
+    plan = Plan([a.to(dev) for a in arrays], nruns, ndense, (col_idx, row_off), [m.to(dev) for m in mixed])
     with _lock:
         _cache[key] = plan
         while len(_cache) > _MAX_ENTRIES:
