@@ -408,8 +408,7 @@ def test_bench_refuses_more_than_one_gpu_with_a_message():
 
 def test_mixed_launch_order_is_the_same_latitudes_interleaved_by_work():
     """gather_order_mixed / scatter_order_mixed: permutations of the latitudes in which the long-run list and the short-run list
-    each keep their own order, both are spread over the whole launch, and neither list's handed-out share of work runs ahead of
-    the other's by more than one latitude."""
+    each keep their own order and the long-run latitudes are spread over the launch instead of forming its prefix."""
     from oracle import geometry as ogeo
 
     ins = outs = (48, 96)
