@@ -202,10 +202,23 @@ def test_product_neighborhood_equals_oracle(ins, outs, gi, go, tc):
     assert torch.equal(row, torch.repeat_interleave(torch.arange(outs[0]), roff[1:] - roff[:-1]))
 
 
-def test_product_neighborhood_at_benchmark_resolution():
-    col, roff, _ = precompute_neighborhood_s2((721, 1440), (721, 1440), theta_cutoff=3 * math.pi / 720)
-    lens = roff[1:] - roff[:-1]
-    assert col.numel() == 99625 and int(lens.min()) == 29 and int(lens.max()) == 5760 and int(lens.median()) == 41
+@pytest.mark.parametrize(
+    "ins,outs,gi,go,tc,nnz,lens",
+    [
+        ((721, 1440), (721, 1440), "equiangular", "equiangular", 3 * math.pi / 720, 99625, (29, 41, 5760)),
+        ((721, 1440), (360, 720), "equiangular", "legendre-gauss", 2 * math.pi / 359, 77422, (48, 72, 6271)),
+        ((361, 720), (361, 720), "legendre-gauss", "legendre-gauss", 8 * math.pi / 360, 237317, (197, 287, 5562)),
+    ],
+    ids=["cfg3", "cfg4", "cfg5"],
+)
+def test_product_neighborhood_at_benchmark_resolution(ins, outs, gi, go, tc, nnz, lens):
+    """The band-limited builder against the restatement of the reference's full-grid loop, entry by entry, at the three
+    large benchmark grids (its latitude band and slack are what could go wrong at 721 rows and not at 128)."""
+    col, roff, _ = precompute_neighborhood_s2(ins, outs, gi, go, tc)
+    col_o, roff_o = ogeo.neighborhood_csr(ins, outs, gi, go, tc)
+    assert torch.equal(roff, roff_o) and torch.equal(col, col_o)
+    n = roff[1:] - roff[:-1]
+    assert col.numel() == nnz and (int(n.min()), int(n.median()), int(n.max())) == lens  # torch's median: the lower middle element
 
 
 # ---- module ---------------------------------------------------------------------------------------
@@ -424,3 +437,30 @@ def test_mixed_launch_order_is_the_same_latitudes_interleaved_by_work():
         assert [r for r in mix if r in set(dense)] == dense and [r for r in mix if r in set(vec)] == vec
         where_dense = [i for i, r in enumerate(mix) if r in set(dense)]
         assert where_dense[0] <= 1 and where_dense[-1] >= len(mix) // 2  # spread out, not a prefix
+
+
+def test_plan_cache_keys_accept_inference_tensors():
+    """psi buffers created or moved under torch.inference_mode() have no version counter; the cache keys must not read one."""
+    from torch_harmonics_amd import plan
+
+    with torch.inference_mode():
+        roff = torch.tensor([0, 2, 3], dtype=torch.int64)
+        col = torch.tensor([0, 1, 5], dtype=torch.int64)
+    assert roff.is_inference() and plan._version(roff) == 0 and plan._version(col) == 0
+    normal = torch.zeros(3, dtype=torch.int64)
+    v0 = plan._version(normal)
+    normal.add_(1)
+    assert plan._version(normal) == v0 + 1
+    order = plan.get_row_order(roff)  # a cached lookup keyed by an inference tensor
+    assert order.tolist() == [0, 1] and plan.get_row_order(roff) is order
+    plan.clear_plan_cache()
+
+
+@pytest.mark.parametrize("n", [100, 16384, 16384 * 3 + 7, 8192 * 64 + 13, 70001])
+def test_weight_gradient_split_reduction(n):
+    """g^T x with the reduction over n split into slices (taken from n >= 16384) equals the plain product, remainder rows included."""
+    from torch_harmonics_amd.attention import _weight_grad
+
+    gen = torch.Generator().manual_seed(n)
+    g, x = torch.randn(n, 6, generator=gen, dtype=torch.float64), torch.randn(n, 5, generator=gen, dtype=torch.float64)
+    torch.testing.assert_close(_weight_grad(g, x), g.t() @ x, rtol=1e-12, atol=1e-9)

@@ -22,6 +22,11 @@ _cache = OrderedDict()
 _lock = threading.Lock()
 
 
+def _version(t: torch.Tensor) -> int:
+    """Version counter of a tensor for the cache keys; inference tensors have none (reading it raises) and cannot be edited in place while tracked."""
+    return 0 if t.is_inference() else t._version
+
+
 class Plan:
     """Six int32 arrays plus the two interleaved launch orders on one device, and the ctypes view the library takes."""
 
@@ -96,8 +101,8 @@ def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in
         row_off.data_ptr(),
         col_idx.numel(),
         row_off.numel(),
-        col_idx._version,
-        row_off._version,
+        _version(col_idx),
+        _version(row_off),
         str(col_idx.device),
         nlat_in,
         nlon_in,
@@ -127,7 +132,7 @@ def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, modulus: in
     t_order the keys by decreasing number of entries; see include/s2attn.h.  Built with device operations only (no host round trip) the first time a psi is seen, then served
     from the same cache as the plans.
     """
-    key = ("transposed", col_idx.data_ptr(), row_off.data_ptr(), col_idx.numel(), row_off.numel(), col_idx._version, row_off._version,
+    key = ("transposed", col_idx.data_ptr(), row_off.data_ptr(), col_idx.numel(), row_off.numel(), _version(col_idx), _version(row_off),
            str(col_idx.device), modulus, key_lo, nkeys)  # fmt: skip
     with _lock:
         hit = _cache.get(key)
@@ -152,7 +157,7 @@ def get_transposed_csr(col_idx: torch.Tensor, row_off: torch.Tensor, modulus: in
 
 def get_row_order(row_off: torch.Tensor) -> torch.Tensor:
     """CSR rows by decreasing number of entries (int32, on row_off's device), cached per row_off."""
-    key = ("order", row_off.data_ptr(), row_off.numel(), row_off._version, str(row_off.device))
+    key = ("order", row_off.data_ptr(), row_off.numel(), _version(row_off), str(row_off.device))
     with _lock:
         hit = _cache.get(key)
         if hit is not None:
