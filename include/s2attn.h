@@ -1,5 +1,5 @@
 /*
- * s2attn: spherical neighborhood attention (gather direction) for AMD gfx950.
+ * s2attn: spherical neighborhood attention (self-attention, down-sampling and up-sampling) for AMD gfx950.
  *
  * Plain C ABI of libs2attn.so.  No torch types cross this boundary: device
  * buffers are raw pointers, sizes are ints, the stream is a hipStream_t passed
@@ -174,6 +174,23 @@ int s2attn_backward_saved(const void *k, const void *v, const void *q, const voi
 int s2attn_backward_dq_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
                              const float *quad_weights, void *dq, void *workspace, const s2attn_plan *plan,
                              const s2attn_shape *shape, void *stream);
+
+/*
+ * s2attn_backward_saved for callers that cannot allocate device memory (code under HIP graph capture, tight loops,
+ * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and same results as
+ * s2attn_backward_saved minus the workspace: the two statistics per (batch, head, output point) live in a device array
+ * built into the library, S2ATTN_NOALLOC_SCRATCH_BYTES large (every GPU the library runs on holds its copy until the
+ * process ends).  Shapes whose s2attn_backward_workspace_bytes() exceed that return S2ATTN_E_UNSUPPORTED (64 MiB holds
+ * 8.3 M output points x heads x batch entries with fp32 heads of 32 channels on wide grids, e.g. 721 x 1440 x 8 heads).
+ * Calls no hipMalloc / hipFree.  The first call on a device looks the array's address up (hipGetSymbolAddress): make
+ * that call outside a graph capture.  All calls on one GPU share the array: calls that overlap there (two streams, two
+ * threads) race; calls on one stream are ordered by the stream.
+ */
+#define S2ATTN_NOALLOC_SCRATCH_BYTES (64 * 1024 * 1024)
+
+int s2attn_backward_saved_noalloc(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
+                                  const float *quad_weights, void *dk, void *dv, void *dq, const s2attn_plan *plan,
+                                  const s2attn_shape *shape, void *stream);
 
 /*
  * Layout conversion.  Replace attention_kernels::permute_to_nhwc / permute_to_nchw

@@ -15,7 +15,8 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 8
+ABI_VERSION = 9
+NOALLOC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 _vp = ctypes.c_void_p
 _i64 = ctypes.c_int64
@@ -85,6 +86,7 @@ SYMBOLS = {
     "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_forward_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_saved": (_int, [_vp] * 11 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
+    "s2attn_backward_saved_noalloc": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_dq_saved": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
     "s2attn_backward": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),

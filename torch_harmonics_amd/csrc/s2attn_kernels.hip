@@ -30,6 +30,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 #include <type_traits>
 
 #include "s2attn_internal.h"
@@ -57,7 +58,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 8; }
+extern "C" int s2attn_abi_version(void) { return 9; }
 #endif
 
 namespace s2 {
@@ -2889,6 +2890,46 @@ extern "C" int s2attn_backward(const void *k, const void *v, const void *q, cons
     const int rc = s2attn_backward_dq(k, v, q, dy, quad_weights, dq, workspace, plan, shape, stream);
     if (rc != S2ATTN_OK) return rc;
     return s2attn_backward_dkdv(k, v, q, dy, quad_weights, dk, dv, workspace, plan, shape, stream);
+}
+
+// ---------------------------------------------------------------------------------
+// backward from saved statistics for callers that cannot allocate: the workspace is a device array of this library
+// ---------------------------------------------------------------------------------
+static __device__ __align__(256) unsigned char scratch[S2ATTN_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void *g_scratch_ptr[MAX_DEVICES] = {}; // address of `scratch` on each device, looked up once per device
+} // namespace
+
+extern "C" int s2attn_backward_saved_noalloc(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
+                                             const float *quad_weights, void *dk, void *dv, void *dq, const s2attn_plan *plan,
+                                             const s2attn_shape *shape, void *stream)
+{
+    const int64_t need = s2attn_backward_workspace_bytes(shape);
+    if (need < 0) return (int)need;
+    if (need > (int64_t)S2ATTN_NOALLOC_SCRATCH_BYTES)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "this shape needs %lld bytes of backward workspace, the built-in scratch array holds %lld; use s2attn_backward_saved with a caller-allocated workspace",
+                           (long long)need, (long long)S2ATTN_NOALLOC_SCRATCH_BYTES);
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipGetDevice: %s", hipGetErrorString(e));
+    if (dev < 0 || dev >= MAX_DEVICES) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "device ordinal %d is outside the %d this library keeps a scratch address for", dev, MAX_DEVICES);
+    void *ws = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        if (!g_scratch_ptr[dev]) { // every device holds its own copy of the array at its own address
+            void *p = nullptr;
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !p) return s2attn_fail(S2ATTN_E_LAUNCH, "hipGetSymbolAddress(scratch): %s", hipGetErrorString(e));
+            g_scratch_ptr[dev] = p;
+        }
+        ws = g_scratch_ptr[dev];
+    }
+    // the dq pass writes both statistics of every (batch, head, output point) before the dk/dv pass reads them, so
+    // nothing of a previous call's contents is ever read and nothing needs clearing
+    return s2attn_backward_saved(k, v, q, dy, y, lse, quad_weights, dk, dv, dq, ws, plan, shape, stream);
 }
 
 namespace {
