@@ -357,7 +357,7 @@ def main():
     shape = _lib.ShapeStruct(B, nh, Hi, Wi, Ho, Wo, k.shape[3] // nh, v.shape[3] // nh, _lib.S2ATTN_BF16 if bf16 else _lib.S2ATTN_F32)
     y = torch.empty(q.shape[:3] + (v.shape[3],), device=dev, dtype=k.dtype)
     dk, dv, dq = torch.empty_like(k), torch.empty_like(v), torch.empty_like(q)
-    ws = torch.empty(lib.s2attn_backward_workspace_bytes(ctypes.byref(shape)) // 4, device=dev)
+    ws = torch.empty(lib.s2attn_backward_saved_workspace_bytes(ctypes.byref(shape)) // 4, device=dev)
     lse = torch.empty((B, nh, Ho, Wo), device=dev)
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     pl, sh = ctypes.byref(plan.struct), ctypes.byref(shape)

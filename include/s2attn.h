@@ -71,37 +71,71 @@ int s2attn_abi_version(void);
  * the longest latitudes first is the load balancing for the ~200:1 spread of row lengths between the poles and
  * the equator.  Any CSR is representable (worst case every entry is its own run).
  *
+ * The plan is ONE position-independent array of int32 (the "blob"): a header of S2ATTN_PLAN_HEADER_INTS ints (counts, and
+ * the offset in ints of every array inside the blob) followed by the arrays, each starting on a 16-byte boundary:
+ *     gather_off  [nvout+1]   gather_runs  [4*nruns]   gather_order  [nvout]   gather_order_mixed  [nvout]
+ *     scatter_off [nvin+1]    scatter_runs [4*nruns]   scatter_order [nvin]    scatter_order_mixed [nvin]
+ *     *_order_mixed: the same latitudes with the long-run and the short-run ones interleaved in proportion to their work
+ *     gather_items  [2*n]  scatter_items [2*n]   work lists of the kernels that put long runs on the matrix cores and short
+ *                 runs on the vector ALU (fp32 heads of 32 channels on at least 64 longitudes): (latitude, pair) with
+ *                 pair = -1 for a single latitude, else the index of a PAIR of adjacent short-run latitudes (latitude,
+ *                 latitude + 1) that one wavefront works together; long-run and short-run units interleaved by work
+ *     *_pair_off [npairs+1], *_pair_runs [8 * ...]   merged runs of each pair: (lat, ws, len, aux, dA, lenA, dB, lenB) =
+ *                 the union band in the form of a run of that grouping; band position i belongs to the first latitude of
+ *                 the pair iff dA <= i < dA + lenA, to the second iff dB <= i < dB + lenB (len < 32)
+ * The builder runs on the host; the caller copies the blob to the device unchanged (it can also be stored and reused:
+ * it depends only on the CSR and the four grid extents) and passes the device address with a host copy of the header.
+ *
  * s2attn_plan_count   number of runs the CSR decomposes into, or a negative error.
- * s2attn_plan_build   fills caller-allocated host arrays:
- *     gather_off  [nvout+1]   gather_runs  [4*nruns]   gather_order  [nvout]
- *     scatter_off [nvin+1]    scatter_runs [4*nruns]   scatter_order [nvin]
- *     ndense [2]  number of long-run latitudes at the front of gather_order and of scatter_order
- *     gather_order_mixed [nvout], scatter_order_mixed [nvin]  (either may be null) the same latitudes with the long-run and
- *                 the short-run ones interleaved in proportion to their work: the launch order of the kernels that put
- *                 long runs on the matrix cores and short runs on the vector ALU (fp32 heads of 32 channels on at least
- *                 64 longitudes), so that both kinds of workgroups share a SIMD for the whole launch
- * The caller copies the six arrays to the device and passes them, with the two counts, in s2attn_plan.
+ * s2attn_plan_size    number of int32 in the blob of this CSR, or a negative error.
+ * s2attn_plan_build   fills blob_out[blob_ints] (host memory; blob_ints as returned by s2attn_plan_size).
  */
-int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
-                          int nlat_out, int nlon_out);
+#define S2ATTN_PLAN_HEADER_INTS 32
+#define S2ATTN_PLAN_MAGIC 0x53324132 /* "S2A2" */
+enum {
+    S2ATTN_PH_MAGIC = 0,
+    S2ATTN_PH_TOTAL = 1, /* ints in the blob */
+    S2ATTN_PH_NVOUT = 2,
+    S2ATTN_PH_NVIN = 3,
+    S2ATTN_PH_NRUNS = 4,
+    S2ATTN_PH_GATHER_NDENSE = 5,  /* leading entries of gather_order that are long-run latitudes */
+    S2ATTN_PH_SCATTER_NDENSE = 6, /* the same for scatter_order */
+    S2ATTN_PH_GATHER_OFF = 8,
+    S2ATTN_PH_GATHER_RUNS = 9,
+    S2ATTN_PH_GATHER_ORDER = 10,
+    S2ATTN_PH_GATHER_ORDER_MIXED = 11,
+    S2ATTN_PH_SCATTER_OFF = 12,
+    S2ATTN_PH_SCATTER_RUNS = 13,
+    S2ATTN_PH_SCATTER_ORDER = 14,
+    S2ATTN_PH_SCATTER_ORDER_MIXED = 15,
+    S2ATTN_PH_GATHER_NITEMS = 16,
+    S2ATTN_PH_GATHER_ITEMS = 17,
+    S2ATTN_PH_GATHER_PAIR_OFF = 18,
+    S2ATTN_PH_GATHER_PAIR_RUNS = 19,
+    S2ATTN_PH_GATHER_NPAIRS = 20,
+    S2ATTN_PH_SCATTER_NITEMS = 21,
+    S2ATTN_PH_SCATTER_ITEMS = 22,
+    S2ATTN_PH_SCATTER_PAIR_OFF = 23,
+    S2ATTN_PH_SCATTER_PAIR_RUNS = 24,
+    S2ATTN_PH_SCATTER_NPAIRS = 25,
+    S2ATTN_PH_NLAT_IN = 28, /* the grid extents the plan was built for: checked against the shape of every call */
+    S2ATTN_PH_NLON_IN = 29,
+    S2ATTN_PH_NLAT_OUT = 30,
+    S2ATTN_PH_NLON_OUT = 31
+};
 
-int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
-                      int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
-                      int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order,
-                      int32_t *ndense, int32_t *gather_order_mixed, int32_t *scatter_order_mixed);
+int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in, int nlat_out,
+                          int nlon_out);
+
+int64_t s2attn_plan_size(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in, int nlat_out,
+                         int nlon_out);
+
+int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in, int nlat_out,
+                      int nlon_out, int32_t *blob_out, int64_t blob_ints);
 
 typedef struct s2attn_plan {
-    const int32_t *gather_off;    /* device, [nvout+1]  */
-    const int32_t *gather_runs;   /* device, [4*nruns]  */
-    const int32_t *gather_order;  /* device, [nvout]    */
-    const int32_t *scatter_off;   /* device, [nvin+1]   (backward only) */
-    const int32_t *scatter_runs;  /* device, [4*nruns]  (backward only) */
-    const int32_t *scatter_order; /* device, [nvin]     (backward only) */
-    int64_t nruns;
-    int32_t gather_ndense;  /* leading entries of gather_order that are long-run latitudes  */
-    int32_t scatter_ndense; /* leading entries of scatter_order that are long-run latitudes */
-    const int32_t *gather_order_mixed;  /* device, [nvout], may be null: see s2attn_plan_build */
-    const int32_t *scatter_order_mixed; /* device, [nvin],  may be null */
+    const int32_t *data;                     /* device copy of the blob */
+    int32_t header[S2ATTN_PLAN_HEADER_INTS]; /* host copy of the blob's first S2ATTN_PLAN_HEADER_INTS ints */
 } s2attn_plan;
 
 typedef struct s2attn_shape {
@@ -138,8 +172,11 @@ int s2attn_forward_lse(const void *k, const void *v, const void *q, const float 
  * workspace: device scratch of s2attn_backward_workspace_bytes(shape) bytes, 8-byte aligned (16 for the matrix-core
  * shapes below): two fp32 softmax statistics per (batch, head, output point), plus, for the shapes whose dq pass works
  * from the forward's output and normaliser (16-bit storage with a head dim that is a multiple of 8 from 16 to 256, fp32 with
- * one that is a multiple of 4 from 16 to 512, ck == cv, at least 32 columns per virtual latitude), room to recompute those two when the caller does not pass them.
+ * one that is a multiple of 4 from 16 to 512, ck == cv, at least 32 columns per virtual latitude), room for that output
+ * and normaliser, which this entry point first recomputes with the forward kernel.  s2attn_backward_saved and its two
+ * halves, which are handed both, need only the statistics: s2attn_backward_saved_workspace_bytes(shape).
  */
+int64_t s2attn_backward_saved_workspace_bytes(const s2attn_shape *shape);
 int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape);
 
 int s2attn_backward(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, void *dk,
@@ -163,7 +200,7 @@ int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void
 /*
  * Backward from saved forward results: y (the forward output) and lse (from s2attn_forward_lse) make the softmax
  * final from the first neighbor on, which saves one of the four matrix products of the dq pass and all running-maximum
- * bookkeeping.  Same outputs as s2attn_backward to rounding; same workspace.  Shapes that run on the vector kernels
+ * bookkeeping.  Same outputs as s2attn_backward to rounding; workspace of s2attn_backward_saved_workspace_bytes().  Shapes that run on the vector kernels
  * (other head dims, ck != cv, narrow grids, unaligned tensors) ignore y and lse and take the
  * s2attn_backward path.
  */
@@ -180,7 +217,7 @@ int s2attn_backward_dq_saved(const void *k, const void *v, const void *q, const 
  * harnesses that forbid hipMalloc).  It has no counterpart in the reference.  Same arguments and same results as
  * s2attn_backward_saved minus the workspace: the two statistics per (batch, head, output point) live in a device array
  * built into the library, S2ATTN_NOALLOC_SCRATCH_BYTES large (every GPU the library runs on holds its copy until the
- * process ends).  Shapes whose s2attn_backward_workspace_bytes() exceed that return S2ATTN_E_UNSUPPORTED (64 MiB holds
+ * process ends).  Shapes whose s2attn_backward_saved_workspace_bytes() exceed that return S2ATTN_E_UNSUPPORTED (64 MiB holds
  * 8.3 M output points x heads x batch entries with fp32 heads of 32 channels on wide grids, e.g. 721 x 1440 x 8 heads).
  * Calls no hipMalloc / hipFree.  The first call on a device looks the array's address up (hipGetSymbolAddress): make
  * that call outside a graph capture.  All calls on one GPU share the array: calls that overlap there (two streams, two

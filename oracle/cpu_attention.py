@@ -148,18 +148,20 @@ def is_upsample(Wi, Wo):
     return Wo % Wi == 0 and Wi % Wo != 0
 
 
-def dense_attention_f64(k, v, q, quad_weights, col_idx, row_off, nh):
+def dense_attention_f64(k, v, q, quad_weights, col_idx, row_off, nh, dtype=torch.float64):
     """
     Textbook formulation, differentiable: softmax over the masked neighborhood of
     q.k + log(quad weight), times v, in float64.  Small grids only (dense mask).  Serves both
     directions: the mask is the only thing that differs (attention_torch.py:74-125 and 582-650).
+    dtype=torch.float32 evaluates the same expression in single precision (what plain fp32 arithmetic
+    makes of the inputs: the yardstick for shapes where 1e-5 is below fp32's own reach).
     """
     B, Hi, Wi, Ho, Wo, Ck, Cv = _dims(k, v, q, nh)
     M = (dense_mask_upsample if is_upsample(Wi, Wo) else dense_mask)(col_idx, row_off, Hi, Wi, Ho, Wo)
-    kd = k.to(torch.float64).reshape(B, Hi * Wi, nh, Ck).permute(0, 2, 1, 3)
-    vd = v.to(torch.float64).reshape(B, Hi * Wi, nh, Cv).permute(0, 2, 1, 3)
-    qd = q.to(torch.float64).reshape(B, Ho * Wo, nh, Ck).permute(0, 2, 1, 3)
-    logw = torch.log(quad_weights.to(torch.float64)).reshape(Hi, 1).expand(Hi, Wi).reshape(1, 1, 1, Hi * Wi)
+    kd = k.to(dtype).reshape(B, Hi * Wi, nh, Ck).permute(0, 2, 1, 3)
+    vd = v.to(dtype).reshape(B, Hi * Wi, nh, Cv).permute(0, 2, 1, 3)
+    qd = q.to(dtype).reshape(B, Ho * Wo, nh, Ck).permute(0, 2, 1, 3)
+    logw = torch.log(quad_weights.to(torch.float64)).to(dtype).reshape(Hi, 1).expand(Hi, Wi).reshape(1, 1, 1, Hi * Wi)
     scores = qd @ kd.transpose(-1, -2) + logw
     scores = scores.masked_fill(~M.reshape(1, 1, Ho * Wo, Hi * Wi), float("-inf"))
     y = torch.softmax(scores, dim=-1) @ vd

@@ -41,7 +41,7 @@ def test_library_loads_and_exports_every_declared_symbol():
 def test_entry_points_reject_bad_arguments_before_touching_the_gpu():
     lib = _lib.load()
     shape = _lib.ShapeStruct(1, 2, 4, 8, 4, 8, 8, 8, _lib.S2ATTN_F32)
-    plan = _lib.PlanStruct(None, None, None, None, None, None, 0)
+    plan = _lib.PlanStruct()
     rc = lib.s2attn_forward(None, None, None, None, None, ctypes.byref(plan), ctypes.byref(shape), None)
     assert rc == -1 and b"null" in lib.s2attn_last_error()
     bad = _lib.ShapeStruct(1, 2, 4, 9, 4, 6, 8, 8, _lib.S2ATTN_F32)  # 9 % 6 != 0
@@ -133,6 +133,94 @@ def test_plan_covers_exactly_the_csr_pairs(ins, outs, gi, go, tc):
         lens = (roff[1:] - roff[:-1]).tolist()
         assert all(lens[gorder[i]] >= lens[gorder[i + 1]] for i in range(outs[0] - 1)), "rows must be ordered longest first"
     assert nruns <= col.numel()
+
+
+def _pairs_from_items(plan, Hi, Wi, Ho, Wo):
+    """Expands the hybrid kernels' work lists the way those kernels walk them: an item is one latitude (its runs) or a pair
+    of adjacent latitudes whose merged bands carry, per band position, which of the two latitudes it belongs to."""
+    up = Wo % Wi == 0 and Wo != Wi
+    psk, psq, W = (1, Wo // Wi, Wi) if up else (Wi // Wo, 1, Wo)
+    goff, gruns, _, soff, sruns, _ = [a.numpy() for a in plan.arrays()]
+    gather, scatter = Counter(), Counter()
+    seen = {"GATHER": [], "SCATTER": []}
+    for side, out in (("GATHER", gather), ("SCATTER", scatter)):
+        items, poff, pruns = [a.numpy() for a in plan.items(side)]
+        off, runs = (goff, gruns) if side == "GATHER" else (soff, sruns)
+        for lat, pair in items.tolist():
+            members = []  # (own latitude, other latitude, aux, ws, len) in the single-run form of this grouping
+            if pair < 0:
+                seen[side].append(lat)
+                members = [(lat, int(r[0]), int(r[1]), int(r[2])) for r in runs[off[lat] : off[lat + 1]]]
+            else:
+                seen[side] += [lat, lat + 1]
+                for other, ws, ln, aux, dA, lenA, dB, lenB in pruns[poff[pair] : poff[pair + 1]].tolist():
+                    assert 1 <= ln < 32 and 0 <= ws < W
+                    for own, d, l in ((lat, dA, lenA), (lat + 1, dB, lenB)):
+                        if l == 0:
+                            continue
+                        assert 0 <= d and d + l <= ln
+                        # a run (ws', l) of the same grouping: gather bands start at ws + d, scatter bands END d before the union's end
+                        members.append((own, other, (ws + d) % W if side == "GATHER" else (ws + ln - d - l) % W, l))
+            for own, other, ws, ln in members:
+                for j in range(W):
+                    for t in range(ln):
+                        if side == "GATHER":  # own = virtual output latitude, other = virtual input latitude
+                            out[(own // psq, j * psq + own % psq, other // psk, ((ws + t + j) % W) * psk + other % psk)] += 1
+                        else:  # own = virtual input latitude, other = virtual output latitude
+                            out[(other // psq, ((j - ws - t) % W) * psq + other % psq, own // psk, j * psk + own % psk)] += 1
+    return gather, scatter, seen
+
+
+@pytest.mark.parametrize(
+    "ins,outs,gi,go,tc",
+    [
+        ((24, 128), (24, 128), "equiangular", "equiangular", 2.5 * math.pi / 23),
+        ((33, 160), (33, 160), "legendre-gauss", "legendre-gauss", 0.2),
+        ((48, 256), (24, 128), "equiangular", "legendre-gauss", 0.3),
+        ((20, 128), (41, 256), "equiangular", "equiangular", 0.35),  # up-sampling
+        ((6, 12), (6, 12), "equiangular", "equiangular", None),  # too narrow for pairs: single latitudes only
+    ],
+)
+def test_plan_work_lists_with_latitude_pairs_cover_exactly_the_csr_pairs(ins, outs, gi, go, tc):
+    from torch_harmonics_amd.plan import build_host_blob
+
+    up = outs[1] % ins[1] == 0 and outs[1] != ins[1]
+    if up:
+        col, roff, _ = precompute_neighborhood_s2(outs, ins, go, gi, tc)
+    else:
+        col, roff, _ = precompute_neighborhood_s2(ins, outs, gi, go, tc)
+    plan = build_host_blob(col, roff, ins[0], ins[1], outs[0], outs[1])
+    ref = _pairs_from_csr(col, roff, ins[1], outs[1])
+    gather, scatter, seen = _pairs_from_items(plan, ins[0], ins[1], outs[0], outs[1])
+    assert gather == ref and scatter == ref
+    h, PH = plan.header, _lib.PH
+    assert sorted(seen["GATHER"]) == list(range(h[PH["NVOUT"]])) and sorted(seen["SCATTER"]) == list(range(h[PH["NVIN"]]))
+    if ins[1] >= 128:
+        assert h[PH["GATHER_NPAIRS"]] > 0 and h[PH["SCATTER_NPAIRS"]] > 0, "the case is meant to form pairs"
+    else:
+        assert h[PH["GATHER_NPAIRS"]] == 0 and h[PH["SCATTER_NPAIRS"]] == 0
+
+
+def test_plan_blob_is_self_describing():
+    from torch_harmonics_amd.plan import build_host_blob, plan_from_blob
+
+    col, roff, _ = precompute_neighborhood_s2((12, 24), (6, 12), "equiangular", "equiangular", 0.6)
+    plan = build_host_blob(col, roff, 12, 24, 6, 12)
+    h, PH = plan.header, _lib.PH
+    assert h[PH["MAGIC"]] == _lib.PLAN_MAGIC and h[PH["TOTAL"]] == plan.blob.numel() and plan.blob.dtype == torch.int32
+    assert (h[PH["NLAT_IN"]], h[PH["NLON_IN"]], h[PH["NLAT_OUT"]], h[PH["NLON_OUT"]]) == (12, 24, 6, 12)
+    assert plan.blob[:32].tolist() == list(h)
+    again = plan_from_blob(plan.blob.clone(), h, 12, 24, 6, 12)
+    assert all(torch.equal(a, b) for a, b in zip(again.arrays(), plan.arrays()))
+    with pytest.raises(RuntimeError, match="grid extents"):
+        plan_from_blob(plan.blob, h, 12, 24, 6, 24)
+    with pytest.raises(RuntimeError, match="header"):
+        plan_from_blob(plan.blob[:-4], h, 12, 24, 6, 12)
+    # the library refuses a plan made for other grids, before anything is launched
+    lib = _lib.load()
+    shape = _lib.ShapeStruct(1, 1, 12, 24, 6, 24, 8, 8, _lib.S2ATTN_F32)
+    rc = lib.s2attn_forward(1, 1, 1, 1, 1, ctypes.byref(plan.struct), ctypes.byref(shape), None)
+    assert rc == -1 and b"built for" in lib.s2attn_last_error()
 
 
 def test_plan_handles_arbitrary_unsorted_csr_with_duplicates():
@@ -239,7 +327,9 @@ def test_module_state_and_defaults():
         "q_norm_weights": (2,),
         "k_norm_weights": (2,),
     }
-    assert {n for n, _ in m.named_buffers()} == {"quad_weights", "psi_row_idx", "psi_col_idx", "psi_roff_idx"}
+    # the reference's four non-persistent buffers, plus the run-length plan of psi (also non-persistent: not in the state_dict)
+    assert {n for n, _ in m.named_buffers()} == {"quad_weights", "psi_row_idx", "psi_col_idx", "psi_roff_idx", "psi_plan"}
+    assert m.psi_plan.dtype == torch.int32 and m.psi_plan[:32].tolist() == m._psi_plan_header
     assert m.theta_cutoff == pytest.approx(math.pi / 5) and m.scale == pytest.approx(1 / math.sqrt(2))
     assert m.quad_weights.dtype == torch.float32 and m.quad_weights.shape == (12,)
     assert m.psi_roff_idx.shape == (7,) and not m.upsample

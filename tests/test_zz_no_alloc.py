@@ -41,7 +41,7 @@ def _run(lib, prob, noalloc, poison=None):
     if noalloc:
         _lib.check(lib.s2attn_backward_saved_noalloc(*head, pl, sh, stream), "s2attn_backward_saved_noalloc")
     else:
-        nbytes = lib.s2attn_backward_workspace_bytes(sh)
+        nbytes = lib.s2attn_backward_saved_workspace_bytes(sh)
         ws = torch.full(((nbytes + 3) // 4,), float("nan"), device=DEV)
         _lib.check(lib.s2attn_backward_saved(*head, ws.data_ptr(), pl, sh, stream), "s2attn_backward_saved")
     torch.cuda.synchronize()
@@ -72,10 +72,10 @@ def test_noalloc_backward_matches_the_workspace_entry_point_twice():
 def test_noalloc_backward_rejects_shapes_beyond_its_scratch():
     """Checked on the host before anything touches a GPU."""
     lib = _lib.load()
-    shape = _lib.ShapeStruct(4, 16, 361, 720, 361, 720, 64, 64, _lib.S2ATTN_BF16)  # needs 133 MB of statistics alone
-    assert lib.s2attn_backward_workspace_bytes(ctypes.byref(shape)) > _lib.NOALLOC_SCRATCH_BYTES
-    plan = _lib.PlanStruct(None, None, None, None, None, None, 0)
+    shape = _lib.ShapeStruct(4, 16, 361, 720, 361, 720, 64, 64, _lib.S2ATTN_BF16)  # needs 133 MB of statistics
+    assert lib.s2attn_backward_saved_workspace_bytes(ctypes.byref(shape)) > _lib.NOALLOC_SCRATCH_BYTES
+    plan = _lib.PlanStruct()
     rc = lib.s2attn_backward_saved_noalloc(*([None] * 10), ctypes.byref(plan), ctypes.byref(shape), None)
     assert rc == -2 and b"scratch" in lib.s2attn_last_error()
     fits = _lib.ShapeStruct(1, 8, 721, 1440, 721, 1440, 32, 32, _lib.S2ATTN_F32)  # the 721 x 1440, 8-head benchmark shape
-    assert lib.s2attn_backward_workspace_bytes(ctypes.byref(fits)) <= _lib.NOALLOC_SCRATCH_BYTES
+    assert lib.s2attn_backward_saved_workspace_bytes(ctypes.byref(fits)) <= _lib.NOALLOC_SCRATCH_BYTES

@@ -13,9 +13,10 @@ import threading
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libs2attn.so")
+TORCH_LIB_PATH = os.path.join(_HERE, "_C.so")  # libtorch registration of the operators (csrc/s2attn_torch.cpp)
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 9
+ABI_VERSION = 10
 NOALLOC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 _vp = ctypes.c_void_p
@@ -23,20 +24,27 @@ _i64 = ctypes.c_int64
 _int = ctypes.c_int
 
 
+PLAN_HEADER_INTS = 32
+PLAN_MAGIC = 0x53324132
+# index of each field in the plan header (include/s2attn.h, S2ATTN_PH_*)
+PH = dict(
+    MAGIC=0, TOTAL=1, NVOUT=2, NVIN=3, NRUNS=4, GATHER_NDENSE=5, SCATTER_NDENSE=6,
+    GATHER_OFF=8, GATHER_RUNS=9, GATHER_ORDER=10, GATHER_ORDER_MIXED=11,
+    SCATTER_OFF=12, SCATTER_RUNS=13, SCATTER_ORDER=14, SCATTER_ORDER_MIXED=15,
+    GATHER_NITEMS=16, GATHER_ITEMS=17, GATHER_PAIR_OFF=18, GATHER_PAIR_RUNS=19, GATHER_NPAIRS=20,
+    SCATTER_NITEMS=21, SCATTER_ITEMS=22, SCATTER_PAIR_OFF=23, SCATTER_PAIR_RUNS=24, SCATTER_NPAIRS=25,
+    NLAT_IN=28, NLON_IN=29, NLAT_OUT=30, NLON_OUT=31,
+)  # fmt: skip
+
+
 class PlanStruct(ctypes.Structure):
-    _fields_ = [
-        ("gather_off", _vp),
-        ("gather_runs", _vp),
-        ("gather_order", _vp),
-        ("scatter_off", _vp),
-        ("scatter_runs", _vp),
-        ("scatter_order", _vp),
-        ("nruns", _i64),
-        ("gather_ndense", ctypes.c_int32),
-        ("scatter_ndense", ctypes.c_int32),
-        ("gather_order_mixed", _vp),
-        ("scatter_order_mixed", _vp),
-    ]
+    """s2attn_plan: device address of the plan blob and a host copy of its header."""
+
+    _fields_ = [("data", _vp), ("header", ctypes.c_int32 * PLAN_HEADER_INTS)]
+
+    @classmethod
+    def make(cls, data_ptr, header):
+        return cls(data_ptr, (ctypes.c_int32 * PLAN_HEADER_INTS)(*[int(x) for x in header]))
 
 
 class ShapeStruct(ctypes.Structure):
@@ -82,13 +90,15 @@ SYMBOLS = {
     "s2attn_last_error": (ctypes.c_char_p, []),
     "s2attn_abi_version": (_int, []),
     "s2attn_plan_count": (_i64, [_vp, _vp, _i64, _int, _int, _int, _int]),
-    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _i64, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "s2attn_plan_size": (_i64, [_vp, _vp, _i64, _int, _int, _int, _int]),
+    "s2attn_plan_build": (_int, [_vp, _vp, _i64, _int, _int, _int, _int, _vp, _i64]),
     "s2attn_forward": (_int, [_vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_forward_lse": (_int, [_vp, _vp, _vp, _vp, _vp, _vp, ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_saved": (_int, [_vp] * 11 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_saved_noalloc": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_dq_saved": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
+    "s2attn_backward_saved_workspace_bytes": (_i64, [ctypes.POINTER(ShapeStruct)]),
     "s2attn_backward": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_dq": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
     "s2attn_backward_dkdv": (_int, [_vp] * 8 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(ShapeStruct), _vp]),
@@ -121,7 +131,7 @@ def build(verbose: bool = False) -> str:
 
 
 def is_built() -> bool:
-    return os.path.exists(LIB_PATH)
+    return os.path.exists(LIB_PATH) and os.path.exists(TORCH_LIB_PATH)
 
 
 def load():
@@ -146,6 +156,27 @@ def load():
             raise RuntimeError(f"libs2attn.so has ABI version {got}, this package expects {ABI_VERSION}; rebuild it")
         _lib = lib
     return _lib
+
+
+_torch_ops_loaded = False
+
+
+def load_torch_ops() -> None:
+    """Loads _C.so, whose static initialisers register attention_kernels::{forward, backward, permute_to_nhwc, permute_to_nchw}
+    and s2attn_kernels::{forward_lse, backward_saved} with the dispatcher; raises if it is not built."""
+    global _torch_ops_loaded
+    if _torch_ops_loaded:
+        return
+    load()  # the C ABI library it links against
+    with _lock:
+        if _torch_ops_loaded:
+            return
+        if not os.path.exists(TORCH_LIB_PATH):
+            raise RuntimeError(f"{TORCH_LIB_PATH} is not built. Run `make -C {os.path.join(_HERE, 'csrc')}`; this package has no fallback implementation.")
+        import torch
+
+        torch.ops.load_library(TORCH_LIB_PATH)
+        _torch_ops_loaded = True
 
 
 def check(rc: int, what: str) -> None:

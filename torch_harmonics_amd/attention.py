@@ -18,6 +18,7 @@ from ._attention_utils import _check_dtypes_match, _check_extent, _check_ndim
 from ._layout import to_nchw, to_nhwc
 from .neighborhood import precompute_neighborhood_s2
 from .ops import neighborhood_s2_attention
+from .plan import build_host_blob
 from .quadrature import precompute_latitudes
 
 __all__ = ["NeighborhoodAttentionS2"]
@@ -204,6 +205,12 @@ class NeighborhoodAttentionS2(nn.Module):
         self.register_buffer("psi_row_idx", row_idx, persistent=False)
         self.register_buffer("psi_col_idx", col_idx, persistent=False)
         self.register_buffer("psi_roff_idx", row_off, persistent=False)
+        # The kernels consume psi as a run-length plan (include/s2attn.h).  It is built here, on the host, from the CSR that was
+        # just computed, and travels with the module as one more buffer, so no forward ever copies psi back from the device
+        # (the reference re-sorts the CSR rows on the device in every call, attention_cuda_utils.cu:74-113).
+        plan = build_host_blob(col_idx, row_off, self.nlat_in, self.nlon_in, self.nlat_out, self.nlon_out)
+        self.register_buffer("psi_plan", plan.blob, persistent=False)
+        self._psi_plan_header = list(plan.header)
 
         # projections are 1x1; stored in convolution shape, drawn in the order q, k, v, proj
         bound_qk = math.sqrt(6.0 / (self.in_channels + self.k_channels))
@@ -294,8 +301,9 @@ class NeighborhoodAttentionS2(nn.Module):
             key = self._head_rms_norm(key, self.k_norm_weights)
 
         out = self.attention_handle(
-            key, value, query, self.quad_weights, self.psi_col_idx, self.psi_roff_idx, self.num_heads, self.nlon_in, self.nlat_out, self.nlon_out
-        )
+            key, value, query, self.quad_weights, self.psi_col_idx, self.psi_roff_idx, self.num_heads, self.nlon_in, self.nlat_out, self.nlon_out,
+            self.psi_plan, self._psi_plan_header,
+        )  # fmt: skip
 
         out = _Linear1x1.apply(out, self.proj_weights.view(self.proj_weights.shape[0], -1), self.proj_bias)
         return to_nchw(out)

@@ -58,7 +58,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 9; }
+extern "C" int s2attn_abi_version(void) { return 10; }
 #endif
 
 namespace s2 {
@@ -269,6 +269,8 @@ template <int P> __device__ inline float dot_row(const float (&a)[P], const floa
     return (s0 + s1) + (s2 + s3);
 }
 
+struct PRun;
+
 struct Args {
     const void *k, *v, *q, *dy;
     void *y, *dk, *dv, *dq;
@@ -277,8 +279,12 @@ struct Args {
     const void *ysaved; // backward with saved statistics: the forward output
     const float *quad_w;
     const int *goff, *gorder, *soff, *sorder;
-    const int *gorder_mixed, *sorder_mixed; // launch orders for the hybrid kernels (may be null)
+    const int *gorder_mixed, *sorder_mixed; // launch orders with long-run and short-run latitudes interleaved
     const Run *gruns, *sruns;
+    // work lists of the hybrid kernels: (latitude, pair index or -1) per workgroup row, merged runs of the pairs (see s2attn_pair.hpp)
+    const int *gitems, *sitems, *gpoff, *spoff;
+    const PRun *gpruns, *spruns;
+    int n_gitems, n_sitems;
     int B, nh, Hi, Wi, Ho, Wo, dk_, dv_;
     int kps; // nlon_in / nlon_out when the input grid is the finer one, else 1; see key_point()
     int qps; // nlon_out / nlon_in when the output grid is the finer one, else 1; see query_point()
@@ -1539,14 +1545,30 @@ __device__ inline int kappa(int v, int half) { return 8 * (v / 4) + 4 * half + (
 // latitude/head, fetched into registers with one 16-byte load per lane per 8 rows.  Matrix-core tiles use the first
 // 32 rows; the vector path for short runs uses all 40 (32 columns + up to 9 neighbors - 1).
 constexpr int MR = 40;  // rows of the LDS tile
-constexpr int VC = 9;   // neighbors per vector-path chunk (MT - 1 + VC <= MR)
-constexpr int LMIN = 32; // runs at least this long go through the matrix cores (measured optimum on cfg3: flat between 24 and 40)
+constexpr int VC = S2_VC;   // neighbors per vector-path chunk (MT - 1 + VC <= MR)
+constexpr int LMIN = S2_LMIN; // runs at least this long go through the matrix cores (measured optimum on cfg3: flat between 24 and 40)
+static_assert(MT - 1 + VC <= MR, "a vector chunk must fit the staged tile");
+// Vector path of the forward: the running maximum m is only the reference point of the exponentials (any m gives the same
+// y = sum p v / sum p), so it is moved, and the accumulators rescaled, only when a score exceeds it by more than this
+// (log2 domain: probabilities stay below 2^8); after a query's first neighbor that is rare.
+constexpr float RESCALE_THR = 8.0f;
 
 template <typename T> struct Tile40 {
     typedef typename Vec4<T>::type raw_t;
     raw_t raw[5];
+    // Tiles that do not cross longitude W - 1 (all but one or two per latitude) are addressed as a wave-uniform base
+    // (scalar registers) plus one per-lane byte offset that never changes, so a load costs no vector instruction besides
+    // itself; only the wrapping tile computes a column per lane and load.
     __device__ inline void fetch(const T *src, unsigned ld, int c0, int W, int lane, bool fifth)
     {
+        const unsigned lane_off = (unsigned)(lane >> 3) * ld + 4u * (unsigned)(lane & 7);
+        if (c0 + MR <= W) {
+            const T *base = src + (size_t)c0 * ld;
+#pragma unroll
+            for (int it = 0; it < 4; it++) raw[it] = *reinterpret_cast<const raw_t *>(base + (size_t)(it * 8) * ld + lane_off);
+            if (fifth) raw[4] = *reinterpret_cast<const raw_t *>(base + (size_t)32 * ld + lane_off);
+            return;
+        }
         const int colA = c0 + (lane >> 3), cb = 4 * (lane & 7);
 #pragma unroll
         for (int it = 0; it < 4; it++) {
@@ -1589,6 +1611,8 @@ __device__ inline int run_stride(int len) { return run_is_dense(len) ? MT : VC; 
     const int w0 = wt * MT;                                                   \
     const int nvalid = min(MT, (W_TILED)-w0);
 
+#include "s2attn_pair.hpp"
+
 // forward, head dim 32.  Lane (j, half) keeps channels 8g + 4 half + e (g, e < 4) of query j: that is the
 // accumulator layout of the matrix-core product, and the vector path for short runs uses the same one (each half
 // computes half of a dot product, one cross-half exchange completes it).
@@ -1596,9 +1620,14 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
 {
     __shared__ __attribute__((aligned(16))) float Ks[MR * MLK];
     __shared__ __attribute__((aligned(16))) float Vs[MR * MLK];
+    __shared__ __attribute__((aligned(16))) int Rs[8 * S2_PAIR_MAX_RUNS]; // merged runs of a latitude pair
 
     S2_MFMA_IDS(a.Wo)
-    const int ho = a.gorder[a.row_first + rowsel];
+    const int ho = a.gitems[2 * rowsel], pair = a.gitems[2 * rowsel + 1];
+    if (pair >= 0) { // two adjacent short-run latitudes in one wavefront
+        fwd_pair<T>(a, Ks, Vs, Rs, lane, b, h, w0, nvalid, ho, pair);
+        return;
+    }
     const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
@@ -1713,47 +1742,41 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], acc, 0, 0, 0);
             }
         } else {
-            // ---- vector chunk: neighbors pos .. pos + L - 1, query j reads staged rows j + t ----
+            // ---- vector chunk: neighbors pos .. pos + L - 1, query j reads staged rows j + t; one pass, lazy maximum ----
             const int L = min(VC, len - pos);
-            float s[VC];
-            float cm = NEG_BIG;
 #pragma unroll
             for (int t = 0; t < VC; t++) {
-                s[t] = NEG_BIG;
                 if (t < L) {
+                    float4 x[4], z[4];
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        x[g] = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
+                        z[g] = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
+                    }
                     float part = 0.f;
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const float4 x = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
-                        part = fmaf(qb[4 * g], x.x, part);
-                        part = fmaf(qb[4 * g + 1], x.y, part);
-                        part = fmaf(qb[4 * g + 2], x.z, part);
-                        part = fmaf(qb[4 * g + 3], x.w, part);
+                        part = fmaf(qb[4 * g], x[g].x, part);
+                        part = fmaf(qb[4 * g + 1], x[g].y, part);
+                        part = fmaf(qb[4 * g + 2], x[g].z, part);
+                        part = fmaf(qb[4 * g + 3], x[g].w, part);
                     }
-                    s[t] = xor32_sum(part);
-                    cm = fmaxf(cm, s[t]);
-                }
-            }
-            const float mn = fmaxf(m, cm);
-            if (__any(mn > m)) {
-                const float corr = fast_exp2(m - mn);
-                S *= corr;
+                    const float sv = xor32_sum(part);
+                    if (__any(sv > m + RESCALE_THR)) {
+                        const float mn = sv > m + RESCALE_THR ? sv : m, corr = fast_exp2(m - mn);
+                        S *= corr;
 #pragma unroll
-                for (int v = 0; v < 16; v++) acc[v] *= corr;
-            }
-            m = mn;
-#pragma unroll
-            for (int t = 0; t < VC; t++) {
-                if (t < L) {
-                    const float p = fast_exp2(s[t] - mn) * w;
+                        for (int v = 0; v < 16; v++) acc[v] *= corr;
+                        m = mn;
+                    }
+                    const float p = fast_exp2(sv - m) * w;
                     S += p;
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
-                        const float4 x = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
-                        acc[4 * g] = fmaf(p, x.x, acc[4 * g]);
-                        acc[4 * g + 1] = fmaf(p, x.y, acc[4 * g + 1]);
-                        acc[4 * g + 2] = fmaf(p, x.z, acc[4 * g + 2]);
-                        acc[4 * g + 3] = fmaf(p, x.w, acc[4 * g + 3]);
+                        acc[4 * g] = fmaf(p, z[g].x, acc[4 * g]);
+                        acc[4 * g + 1] = fmaf(p, z[g].y, acc[4 * g + 1]);
+                        acc[4 * g + 2] = fmaf(p, z[g].z, acc[4 * g + 2]);
+                        acc[4 * g + 3] = fmaf(p, z[g].w, acc[4 * g + 3]);
                     }
                 }
             }
@@ -1779,231 +1802,6 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     }
 }
 
-// backward dq + statistics: same ownership as the forward (lane (j, half): query j, channels 8g + 4 half + e).
-// Matrix-core tile, four products:  S^T = K Q^T,  G^T = V dY^T,  A_k^T += K^T P^T,  A_kg^T += K^T (P o G)^T  (the A
-// operands of the last two are column reads of the K tile, the B operands the probability registers); short runs take
-// the vector path on the same accumulators.  Online softmax across tiles and chunks.
-template <typename T> __global__ __launch_bounds__(64) void dq_mfma_kernel(const Args a)
-{
-    __shared__ __attribute__((aligned(16))) float Ks[MR * MLK];
-    __shared__ __attribute__((aligned(16))) float Vs[MR * MLK];
-
-    S2_MFMA_IDS(a.Wo)
-    const int ho = a.gorder[a.row_first + rowsel];
-    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
-    const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
-    const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
-    const bool mine = j < nvalid;
-    const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? j : 0)) * a.qps;
-
-    float qb[16], gb[16];
-    {
-        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 4 * half;
-        const T *grow = static_cast<const T *>(a.dy) + pt * ldv + (size_t)h * 32 + 4 * half;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float4 x = load4(qrow + 8 * g);
-            const float4 z = load4(grow + 8 * g);
-            qb[4 * g] = x.x * LOG2E, qb[4 * g + 1] = x.y * LOG2E, qb[4 * g + 2] = x.z * LOG2E, qb[4 * g + 3] = x.w * LOG2E;
-            gb[4 * g] = z.x, gb[4 * g + 1] = z.y, gb[4 * g + 2] = z.z, gb[4 * g + 3] = z.w;
-        }
-    }
-    f16v Ak, Akg;
-#pragma unroll
-    for (int v = 0; v < 16; v++) {
-        Ak[v] = 0.f;
-        Akg[v] = 0.f;
-    }
-    float m = NEG_BIG, S = 0.f, Ag = 0.f;
-
-    int ri = a.goff[ho];
-    const int rend = a.goff[ho + 1];
-    int pos = 0;
-    Run run = {0, 0, 0, 0};
-    Tile40<T> kt, vt;
-    auto fetch = [&](const Run &rn, int p) {
-        const int c0 = (rn.ws + w0 + p) % a.Wi;
-        const bool fifth = !run_is_dense(rn.len);
-        kt.fetch(kx + (size_t)key_row(a, rn.lat, rn.pad) * ldk, ldk * a.kps, c0, a.Wi, lane, fifth);
-        vt.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, lane, fifth);
-    };
-    if (ri < rend) {
-        run = a.gruns[ri];
-        fetch(run, 0);
-        kt.commit(Ks, lane, !run_is_dense(run.len));
-        vt.commit(Vs, lane, !run_is_dense(run.len));
-    }
-    __syncthreads();
-    settle(qb);
-    settle(gb);
-
-    while (ri < rend) {
-        const float w = a.quad_w[run.pad];
-        const int len = run.len;
-        int nri = ri, npos = pos + run_stride(len);
-        Run nrun = run;
-        if (run_done(len, npos)) {
-            nri++;
-            npos = 0;
-            if (nri < rend) nrun = a.gruns[nri];
-        }
-        const bool more = nri < rend;
-        if (more) fetch(nrun, npos);
-
-        const float *kq = Ks + j * MLK + 4 * half;
-        const float *vq = Vs + j * MLK + 4 * half;
-        if (run_is_dense(len)) {
-            const int u0 = pos;
-            f16v sc, gc;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                sc[v] = 0.f;
-                gc[v] = 0.f;
-            }
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4 x = *reinterpret_cast<const float4 *>(kq + 8 * g);
-                const float4 z = *reinterpret_cast<const float4 *>(vq + 8 * g);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, qb[4 * g + 0], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, gb[4 * g + 0], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, qb[4 * g + 1], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, gb[4 * g + 1], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, qb[4 * g + 2], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, gb[4 * g + 2], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, qb[4 * g + 3], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, gb[4 * g + 3], gc, 0, 0, 0);
-            }
-            const bool edge = (u0 < MT - 1) || (u0 + MT - 1 >= len);
-            if (edge) {
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    const int t = u0 + kappa(v, half) - j;
-                    sc[v] = (t >= 0 && t < len) ? sc[v] : NEG_BIG;
-                }
-            }
-            float mx = sc[0];
-#pragma unroll
-            for (int v = 1; v < 16; v++) mx = fmaxf(mx, sc[v]);
-            mx = xor32_max(mx);
-            const float mn = fmaxf(m, mx);
-            if (__any(mn > m)) {
-                const float corr = fast_exp2(m - mn);
-                S *= corr;
-                Ag *= corr;
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    Ak[v] *= corr;
-                    Akg[v] *= corr;
-                }
-            }
-            m = mn;
-            float rs = 0.f, rg = 0.f;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                float p = fast_exp2(sc[v] - mn) * w;
-                if (edge) p = (sc[v] == NEG_BIG) ? 0.f : p;
-                const float pg = p * gc[v];
-                sc[v] = p;
-                gc[v] = pg;
-                rs += p;
-                rg += pg;
-            }
-            rs = xor32_sum(rs);
-            rg = xor32_sum(rg);
-            S += rs;
-            Ag += rg;
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float x = Ks[kappa(v, half) * MLK + j];
-                Ak = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], Ak, 0, 0, 0);
-                Akg = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], Akg, 0, 0, 0);
-            }
-        } else {
-            const int L = min(VC, len - pos);
-            float s[VC], gd[VC];
-            float cm = NEG_BIG;
-#pragma unroll
-            for (int t = 0; t < VC; t++) {
-                s[t] = NEG_BIG;
-                gd[t] = 0.f;
-                if (t < L) {
-                    float ps_ = 0.f, pg_ = 0.f;
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const float4 x = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
-                        const float4 z = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
-                        ps_ = fmaf(qb[4 * g], x.x, ps_);
-                        ps_ = fmaf(qb[4 * g + 1], x.y, ps_);
-                        ps_ = fmaf(qb[4 * g + 2], x.z, ps_);
-                        ps_ = fmaf(qb[4 * g + 3], x.w, ps_);
-                        pg_ = fmaf(gb[4 * g], z.x, pg_);
-                        pg_ = fmaf(gb[4 * g + 1], z.y, pg_);
-                        pg_ = fmaf(gb[4 * g + 2], z.z, pg_);
-                        pg_ = fmaf(gb[4 * g + 3], z.w, pg_);
-                    }
-                    s[t] = xor32_sum(ps_);
-                    gd[t] = xor32_sum(pg_);
-                    cm = fmaxf(cm, s[t]);
-                }
-            }
-            const float mn = fmaxf(m, cm);
-            if (__any(mn > m)) {
-                const float corr = fast_exp2(m - mn);
-                S *= corr;
-                Ag *= corr;
-#pragma unroll
-                for (int v = 0; v < 16; v++) {
-                    Ak[v] *= corr;
-                    Akg[v] *= corr;
-                }
-            }
-            m = mn;
-#pragma unroll
-            for (int t = 0; t < VC; t++) {
-                if (t < L) {
-                    const float p = fast_exp2(s[t] - mn) * w;
-                    const float pg = p * gd[t];
-                    S += p;
-                    Ag += pg;
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        const float4 x = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
-                        Ak[4 * g] = fmaf(p, x.x, Ak[4 * g]);
-                        Ak[4 * g + 1] = fmaf(p, x.y, Ak[4 * g + 1]);
-                        Ak[4 * g + 2] = fmaf(p, x.z, Ak[4 * g + 2]);
-                        Ak[4 * g + 3] = fmaf(p, x.w, Ak[4 * g + 3]);
-                        Akg[4 * g] = fmaf(pg, x.x, Akg[4 * g]);
-                        Akg[4 * g + 1] = fmaf(pg, x.y, Akg[4 * g + 1]);
-                        Akg[4 * g + 2] = fmaf(pg, x.z, Akg[4 * g + 2]);
-                        Akg[4 * g + 3] = fmaf(pg, x.w, Akg[4 * g + 3]);
-                    }
-                }
-            }
-        }
-
-        __syncthreads();
-        if (more) {
-            kt.commit(Ks, lane, !run_is_dense(nrun.len));
-            vt.commit(Vs, lane, !run_is_dense(nrun.len));
-        }
-        __syncthreads();
-        ri = nri;
-        pos = npos;
-        run = nrun;
-    }
-
-    if (mine) {
-        const float inv = 1.0f / S;
-        const float I = Ag * inv;
-        if (half == 0) a.stats[((size_t)bh * a.Ho + ho) * a.Wo + w0 + j] = make_float2(m + fast_log2(S), I);
-        T *dq = static_cast<T *>(a.dq) + pt * ldk + (size_t)h * 32 + 4 * half;
-#pragma unroll
-        for (int g = 0; g < 4; g++)
-            store4(dq + 8 * g, make_float4((Akg[4 * g] - I * Ak[4 * g]) * inv, (Akg[4 * g + 1] - I * Ak[4 * g + 1]) * inv,
-                                           (Akg[4 * g + 2] - I * Ak[4 * g + 2]) * inv, (Akg[4 * g + 3] - I * Ak[4 * g + 3]) * inv));
-    }
-}
-
 // backward dq from saved forward statistics: with lse = log2 sum_j a_j known per query and I = <dy, y>, the softmax is
 // final from the first neighbor on, p_j = exp2(s_j - lse) w_j, and dq = sum_j p_j (g_j - I) k_j needs three matrix
 // products per tile (S^T, G^T, dQ^T += K^T C^T) and no running maximum or rescaling.
@@ -2013,7 +1811,10 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     __shared__ __attribute__((aligned(16))) float Vs[MR * MLK];
 
     S2_MFMA_IDS(a.Wo)
-    const int ho = a.gorder[a.row_first + rowsel];
+    // One latitude per workgroup row, long-run and short-run latitudes interleaved.  (No latitude pairs in this pass: a lane
+    // holding q, dy and dq of two latitudes plus the tile prefetch costs the third resident wavefront per SIMD, which the
+    // matrix-core path of the same kernel needs more than the short rows need the shared LDS reads.)
+    const int ho = a.gorder_mixed[rowsel];
     const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
@@ -2188,9 +1989,14 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     __shared__ __attribute__((aligned(16))) float Gs[MR * MLK];
     __shared__ __attribute__((aligned(16))) float Ls[MR];
     __shared__ __attribute__((aligned(16))) float Is[MR];
+    __shared__ __attribute__((aligned(16))) int Rs[8 * S2_PAIR_MAX_RUNS];
 
     S2_MFMA_IDS(a.Wi)
-    const int hi = a.sorder[a.row_first + rowsel];
+    const int hi = a.sitems[2 * rowsel], pair = a.sitems[2 * rowsel + 1];
+    if (pair >= 0) {
+        dkdv_pair<T>(a, Qs, Gs, Ls, Is, Rs, lane, b, h, w0, nvalid, hi, pair);
+        return;
+    }
     const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
     const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldk + (size_t)h * 32;
     const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * 32;
@@ -2615,27 +2421,27 @@ template <typename T, bool VEC> int launch_p(Which which, const Args &a, int row
     return launch_one<T, 32, VEC>(which, a, row_first, row_count, stream);
 }
 
-// dense kernels: head dims 32, vector-aligned rows, at least 64 columns per virtual latitude
-template <typename T> int launch_dense(Which which, const Args &a0, int row_count, hipStream_t stream)
+// hybrid kernels: head dim 32, vector-aligned rows, at least 64 columns per virtual latitude.  One workgroup row per item
+// of the plan's work list (a long-run latitude, a single short-run latitude or a pair of adjacent short-run latitudes;
+// long-run and short-run units interleaved: matrix-core-heavy and vector-heavy workgroups side by side).  The dq pass
+// exists only in the form that takes the forward's y and lse.
+template <typename T> int launch_dense(Which which, const Args &a0, hipStream_t stream)
 {
-    if (row_count <= 0) return S2ATTN_OK;
     Args a = a0;
     a.row_first = 0;
-    // long-run and short-run latitudes interleaved: matrix-core-heavy and vector-heavy workgroups side by side
-    if (a.gorder_mixed) a.gorder = a.gorder_mixed;
-    if (a.sorder_mixed) a.sorder = a.sorder_mixed;
     void (*kern)(const Args) = nullptr;
     long nblocks = 0;
     if (which == FWD) {
         kern = fwd_mfma_kernel<T>;
-        nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
+        nblocks = (long)a.n_gitems * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
     } else if (which == DQ) {
-        kern = (a.ysaved && a.lse) ? dq_saved_mfma_kernel<T> : dq_mfma_kernel<T>;
-        nblocks = (long)row_count * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
+        kern = dq_saved_mfma_kernel<T>;
+        nblocks = (long)a.Ho * ((a.Wo + MT - 1) / MT) * a.B * a.nh;
     } else {
         kern = dkdv_mfma_kernel<T>;
-        nblocks = (long)row_count * ((a.Wi + MT - 1) / MT) * a.B * a.nh;
+        nblocks = (long)a.n_sitems * ((a.Wi + MT - 1) / MT) * a.B * a.nh;
     }
+    if (nblocks <= 0) return S2ATTN_OK;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
     hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
     const hipError_t e = hipGetLastError();
@@ -2674,7 +2480,7 @@ template <typename T> bool m32_ok(Which which, const Args &a)
 
 bool dense_ok(Which which, const Args &a, bool vec)
 {
-    (void)which;
+    if (which == DQ && !(a.ysaved && a.lse)) return false;
     return vec && a.dk_ == 32 && a.dv_ == 32 && a.Wi >= 64;
 }
 
@@ -2695,7 +2501,7 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
         // head dim 32 on at least 64 columns: the hybrid kernels handle short runs themselves (vector path inside), so
         // they take every latitude; measured ahead of the 16-longitude family there (cfg3 13.5 against 16.4 ms)
         (void)ndense;
-        return launch_dense<T>(which, a, nrows, stream);
+        return launch_dense<T>(which, a, stream);
     }
     if (m32_ok<T>(which, a)) {
         if (a.dk_ <= 16) return launch_m32<16, 1>(which, a, stream);
@@ -2715,17 +2521,43 @@ int launch(Which which, const Args &a, int dtype, bool vec, int ndense, hipStrea
     return launch_t<f16_t>(which, a, vec, ndense, stream);
 }
 
+// The plan must be the blob s2attn_plan_build made for exactly these grid extents.
+int check_plan(const s2attn_plan *plan, const s2attn_shape *sh)
+{
+    if (!plan || !plan->data) return s2attn_fail(S2ATTN_E_INVALID, "plan is null");
+    const int32_t *h = plan->header;
+    if (h[S2ATTN_PH_MAGIC] != S2ATTN_PLAN_MAGIC) return s2attn_fail(S2ATTN_E_INVALID, "plan header does not carry this library's plan format");
+    if (h[S2ATTN_PH_NLAT_IN] != sh->nlat_in || h[S2ATTN_PH_NLON_IN] != sh->nlon_in || h[S2ATTN_PH_NLAT_OUT] != sh->nlat_out || h[S2ATTN_PH_NLON_OUT] != sh->nlon_out)
+        return s2attn_fail(S2ATTN_E_INVALID, "plan was built for grids %dx%d -> %dx%d, the call is for %dx%d -> %dx%d", h[S2ATTN_PH_NLAT_IN], h[S2ATTN_PH_NLON_IN],
+                           h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], sh->nlat_in, sh->nlon_in, sh->nlat_out, sh->nlon_out);
+    const int32_t total = h[S2ATTN_PH_TOTAL];
+    for (int i = S2ATTN_PH_GATHER_OFF; i <= S2ATTN_PH_SCATTER_PAIR_RUNS; i++) {
+        if (i == S2ATTN_PH_GATHER_NITEMS || i == S2ATTN_PH_GATHER_NPAIRS || i == S2ATTN_PH_SCATTER_NITEMS) continue;
+        if (h[i] < S2ATTN_PLAN_HEADER_INTS || h[i] > total) return s2attn_fail(S2ATTN_E_INVALID, "plan header: offset %d of array %d lies outside the plan", h[i], i);
+    }
+    return S2ATTN_OK;
+}
+
 void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const float *quad_w)
 {
+    const int32_t *h = plan->header, *d = plan->data;
     a.quad_w = quad_w;
-    a.goff = plan->gather_off;
-    a.gruns = reinterpret_cast<const Run *>(plan->gather_runs);
-    a.gorder = plan->gather_order;
-    a.soff = plan->scatter_off;
-    a.sruns = reinterpret_cast<const Run *>(plan->scatter_runs);
-    a.sorder = plan->scatter_order;
-    a.gorder_mixed = plan->gather_order_mixed;
-    a.sorder_mixed = plan->scatter_order_mixed;
+    a.goff = d + h[S2ATTN_PH_GATHER_OFF];
+    a.gruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_GATHER_RUNS]);
+    a.gorder = d + h[S2ATTN_PH_GATHER_ORDER];
+    a.gorder_mixed = d + h[S2ATTN_PH_GATHER_ORDER_MIXED];
+    a.soff = d + h[S2ATTN_PH_SCATTER_OFF];
+    a.sruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_SCATTER_RUNS]);
+    a.sorder = d + h[S2ATTN_PH_SCATTER_ORDER];
+    a.sorder_mixed = d + h[S2ATTN_PH_SCATTER_ORDER_MIXED];
+    a.gitems = d + h[S2ATTN_PH_GATHER_ITEMS];
+    a.gpoff = d + h[S2ATTN_PH_GATHER_PAIR_OFF];
+    a.gpruns = reinterpret_cast<const PRun *>(d + h[S2ATTN_PH_GATHER_PAIR_RUNS]);
+    a.n_gitems = h[S2ATTN_PH_GATHER_NITEMS];
+    a.sitems = d + h[S2ATTN_PH_SCATTER_ITEMS];
+    a.spoff = d + h[S2ATTN_PH_SCATTER_PAIR_OFF];
+    a.spruns = reinterpret_cast<const PRun *>(d + h[S2ATTN_PH_SCATTER_PAIR_RUNS]);
+    a.n_sitems = h[S2ATTN_PH_SCATTER_NITEMS];
     a.B = sh->batch;
     a.nh = sh->num_heads;
     const bool up = sh->nlon_out % sh->nlon_in == 0 && sh->nlon_out != sh->nlon_in;
@@ -2755,8 +2587,8 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     int rc = check_shape(shape);
     if (rc != S2ATTN_OK) return rc;
     if (!k || !v || !q || !y || !quad_weights) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
-    if (!plan || !plan->gather_off || !plan->gather_order || (plan->nruns > 0 && !plan->gather_runs))
-        return s2attn_fail(S2ATTN_E_INVALID, "plan is missing its gather arrays");
+    rc = check_plan(plan, shape);
+    if (rc != S2ATTN_OK) return rc;
     Args a = {};
     fill_args(a, plan, shape, quad_weights);
     a.k = k, a.v = v, a.q = q, a.y = y;
@@ -2764,23 +2596,29 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     a.tile_rows = TQ - 1 + TL;
     const size_t al = 4 * (size_t)esize(shape->dtype);
     const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(y, al);
-    return launch(FWD, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
+    return launch(FWD, a, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
 }
 
 namespace {
-// Shapes of the 16-bit and the fp32 16-longitude matrix-core kernels.  Their dq pass consumes the forward's output and normaliser; a backward
+// Shapes of the matrix-core kernel families (16-bit, fp32 16-longitude, hybrid).  Their dq pass consumes the forward's output and normaliser; a backward
 // that is not handed them (s2attn_backward, s2attn_backward_dq) first recomputes both into the tail of the workspace.
 bool h16_shape(const s2attn_shape *sh)
 {
     const int w = sh->nlon_out < sh->nlon_in ? sh->nlon_out : sh->nlon_in; // columns of a virtual latitude
     if (sh->ck != sh->cv || w < HK) return false;
-    if (sh->dtype == S2ATTN_F32) // the fp32 16-longitude family works the same way (head dim 32: only below the hybrid kernels' 64 columns)
-        return m32_width(sh->ck, sh->cv) && !(sh->ck == 32 && w >= 64);
+    if (sh->dtype == S2ATTN_F32) return m32_width(sh->ck, sh->cv); // the fp32 16-longitude family and the hybrid kernels work the same way
     return h16_width(sh->ck, sh->cv);
 }
 int64_t stat_points(const s2attn_shape *sh) { return (int64_t)sh->batch * sh->num_heads * sh->nlat_out * sh->nlon_out; }
 int64_t round16(int64_t n) { return (n + 15) / 16 * 16; }
 } // namespace
+
+extern "C" int64_t s2attn_backward_saved_workspace_bytes(const s2attn_shape *shape)
+{
+    const int rc = check_shape(shape);
+    if (rc != S2ATTN_OK) return rc;
+    return round16(stat_points(shape) * (int64_t)sizeof(float2));
+}
 
 extern "C" int64_t s2attn_backward_workspace_bytes(const s2attn_shape *shape)
 {
@@ -2799,9 +2637,8 @@ int backward_args(Args &a, bool &vec, const void *k, const void *v, const void *
     const int rc = check_shape(shape);
     if (rc != S2ATTN_OK) return rc;
     if (!k || !v || !q || !dy || !quad_weights || !workspace) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
-    if (!plan || !plan->gather_off || !plan->gather_order || !plan->scatter_off || !plan->scatter_order
-        || (plan->nruns > 0 && (!plan->gather_runs || !plan->scatter_runs)))
-        return s2attn_fail(S2ATTN_E_INVALID, "plan is missing arrays");
+    const int rcp = check_plan(plan, shape);
+    if (rcp != S2ATTN_OK) return rcp;
     if (!aligned(workspace, sizeof(float2))) return s2attn_fail(S2ATTN_E_INVALID, "workspace must be 8-byte aligned");
     fill_args(a, plan, shape, quad_weights);
     a.k = k, a.v = v, a.q = q, a.dy = dy;
@@ -2830,11 +2667,11 @@ extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, c
         void *y = ws + round16(n * (int64_t)sizeof(float2)) + round16(n * 4);
         Args f = a;
         f.y = y, f.lse = lse, f.dq = nullptr, f.dy = nullptr;
-        const int rc2 = launch(FWD, f, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
+        const int rc2 = launch(FWD, f, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
         if (rc2 != S2ATTN_OK) return rc2;
         a.ysaved = y, a.lse = lse;
     }
-    return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
+    return launch(DQ, a, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2attn_backward_dq_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
@@ -2852,7 +2689,7 @@ extern "C" int s2attn_backward_dq_saved(const void *k, const void *v, const void
     const size_t al = 4 * (size_t)esize(shape->dtype);
     vec = vec && aligned(dq, al) && aligned(y, al);
     a.tile_rows = TQ - 1 + TL;
-    return launch(DQ, a, shape->dtype, vec, plan->gather_ndense, static_cast<hipStream_t>(stream));
+    return launch(DQ, a, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q, const void *dy, const float *quad_weights,
@@ -2869,7 +2706,7 @@ extern "C" int s2attn_backward_dkdv(const void *k, const void *v, const void *q,
     vec = vec && aligned(dk, al) && aligned(dv, al);
     a.tile_rows = TQ + TL;
     if (a.tile_rows < TQ) a.tile_rows = TQ; // the tile also stages the lane-owned k/v and dk/dv rows
-    return launch(DKDV, a, shape->dtype, vec, plan->scatter_ndense, static_cast<hipStream_t>(stream));
+    return launch(DKDV, a, shape->dtype, vec, plan->header[S2ATTN_PH_SCATTER_NDENSE], static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2attn_backward_saved(const void *k, const void *v, const void *q, const void *dy, const void *y, const float *lse,
@@ -2907,7 +2744,7 @@ extern "C" int s2attn_backward_saved_noalloc(const void *k, const void *v, const
                                              const float *quad_weights, void *dk, void *dv, void *dq, const s2attn_plan *plan,
                                              const s2attn_shape *shape, void *stream)
 {
-    const int64_t need = s2attn_backward_workspace_bytes(shape);
+    const int64_t need = s2attn_backward_saved_workspace_bytes(shape);
     if (need < 0) return (int)need;
     if (need > (int64_t)S2ATTN_NOALLOC_SCRATCH_BYTES)
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "this shape needs %lld bytes of backward workspace, the built-in scratch array holds %lld; use s2attn_backward_saved with a caller-allocated workspace",

@@ -115,14 +115,6 @@ int decompose(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int n
 
 } // namespace
 
-extern "C" int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
-                                     int nlat_out, int nlon_out)
-{
-    int64_t n = 0;
-    const int rc = decompose(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, nullptr, &n);
-    return rc == S2ATTN_OK ? n : (int64_t)rc;
-}
-
 namespace {
 
 // Cost model (SIMD cycles per 32 grid points) deciding which kernel family a latitude goes to.  The matrix-core
@@ -141,17 +133,39 @@ struct RowCost {
 // (steps of 1/8 in log2), keeping the natural order inside a class.  A plain sort by cost interleaves the two
 // hemispheres (mirror latitudes cost the same); with classes, consecutive entries are neighboring latitudes, whose
 // tiles share most of their K/V rows in L2.  Returns the number of long-run latitudes.
-// mixed (may be null): the same two lists merged so that at every point of the launch about the same share of each list's
-// work has been handed out.  The kernels that treat long runs on the matrix cores and short runs on the vector ALU take this
-// order: their matrix-core-heavy and vector-heavy workgroups then sit side by side on a SIMD for the whole launch instead
-// of one kind after the other (measured 6-7 % on 721x1440 grids); the kernels that put every run on the matrix cores
-// lose 8-35 % with it (their long rows must start first) and keep `order`.
+// mixed: the same two lists merged so that at every point of the launch about the same share of each list's work has
+// been handed out (see merge_by_share).
 int cost_class(int64_t c)
 {
     int cls = 0;
     while ((c >> cls) > 15) cls++; // c = m * 2^cls, 8 <= m < 16
     return c <= 0 ? -1 : cls * 8 + (int)((c >> cls) - 8);
 }
+
+// Two work lists (matrix-core-heavy and vector-heavy units, each most work first) merged in proportion to their work.
+// The kernels that treat long runs on the matrix cores and short runs on the vector ALU take this order: both kinds of
+// workgroups then sit side by side on a SIMD for the whole launch instead of one kind after the other (measured 6-7 %
+// on 721x1440 grids).  The long-run list is held back a little (its share of work handed out <= 0.7 of the other's):
+// measured best between 0.5 and 0.8, 1.5-2 % of the step over equal shares.
+template <typename Emit> void merge_by_share(const std::vector<int64_t> &cd_, const std::vector<int64_t> &cv_, Emit emit)
+{
+    double wd = 0, wv = 0;
+    for (int64_t c : cd_) wd += (double)c;
+    for (int64_t c : cv_) wv += (double)c;
+    size_t i = 0, j = 0;
+    double cd = 0, cv = 0;
+    while (i < cd_.size() || j < cv_.size()) {
+        const bool take_dense = j >= cv_.size() || (i < cd_.size() && cd * wv <= 0.7 * cv * wd);
+        if (take_dense) {
+            cd += (double)cd_[i];
+            emit(true, i++);
+        } else {
+            cv += (double)cv_[j];
+            emit(false, j++);
+        }
+    }
+}
+
 int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order, int32_t *mixed)
 {
     const int n = (int)cost.size();
@@ -161,76 +175,222 @@ int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order, int32_t *mi
     std::stable_sort(vec.begin(), vec.end(), [&](int32_t a, int32_t b) { return cost_class(cost[a].vector) > cost_class(cost[b].vector); });
     std::copy(dense.begin(), dense.end(), order);
     std::copy(vec.begin(), vec.end(), order + dense.size());
-    if (!mixed) return (int32_t)dense.size();
-    double wd = 0, wv = 0;
-    for (int32_t r : dense) wd += (double)cost[r].dense;
-    for (int32_t r : vec) wv += (double)cost[r].vector;
-    size_t i = 0, j = 0;
-    double cd = 0, cv = 0;
+    std::vector<int64_t> cd, cv;
+    for (int32_t r : dense) cd.push_back(cost[r].dense);
+    for (int32_t r : vec) cv.push_back(cost[r].vector);
     int32_t *out = mixed;
-    while (i < dense.size() || j < vec.size()) {
-        // the long-run list is held back a little (its share of work handed out <= 0.7 of the other's): measured best
-        // between 0.5 and 0.8, 1.5-2 % of the step over equal shares
-        const bool take_dense = j >= vec.size() || (i < dense.size() && cd * wv <= 0.7 * cv * wd);
-        if (take_dense) {
-            cd += (double)cost[dense[i]].dense;
-            *out++ = dense[i++];
-        } else {
-            cv += (double)cost[vec[j]].vector;
-            *out++ = vec[j++];
-        }
-    }
+    merge_by_share(cd, cv, [&](bool d, size_t k) { *out++ = d ? dense[k] : vec[k]; });
     return (int32_t)dense.size();
 }
 
-} // namespace
+// ---- latitude pairs ------------------------------------------------------------------------------------------------
+// The hybrid kernels (fp32 heads of 32 channels) work two ADJACENT latitudes of the short-run kind in one wavefront: both
+// latitudes' neighborhoods lie in nearly the same bands of the other grid, so one staged band and one LDS read of each
+// of its rows serve two queries (or two keys) per lane.  A pair is formed when, latitude by latitude of the other grid,
+// the two runs fit into one band shorter than S2_LMIN positions; its runs are stored merged:
+//   (lat, ws, len, aux, dA, lenA, dB, lenB)
+// (lat, ws, len, aux) is the union band in the form of a single run of the same grouping; position i of the band
+// (0 <= i < len) belongs to the first latitude iff dA <= i < dA + lenA and to the second iff dB <= i < dB + lenB.
+struct Group {
+    const int32_t *runs; // 4 ints each
+    int n;
+};
 
-extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
-                                 int nlat_out, int nlon_out, int64_t nruns, int32_t *gather_off, int32_t *gather_runs,
-                                 int32_t *gather_order, int32_t *scatter_off, int32_t *scatter_runs, int32_t *scatter_order,
-                                 int32_t *ndense, int32_t *gather_order_mixed, int32_t *scatter_order_mixed)
+// centred representative of a circular start column
+int centred(int ws, int W) { return ws < (W + 1) / 2 ? ws : ws - W; }
+
+bool short_sorted(const Group &g)
 {
-    if (!gather_off || !gather_order || !scatter_off || !scatter_order || !ndense || (nruns > 0 && (!gather_runs || !scatter_runs)))
-        return s2attn_fail(S2ATTN_E_INVALID, "plan output array is null");
+    for (int i = 0; i < g.n; i++) {
+        if (g.runs[4 * i + 2] >= S2_LMIN) return false;
+        if (i > 0 && g.runs[4 * i] <= g.runs[4 * (i - 1)]) return false; // one run per latitude, ascending
+    }
+    return g.n > 0;
+}
 
+// merges the runs of two groups; scatter = the d offsets are measured from the END of the union band (the dk/dv kernels
+// index a band backwards: staged row 0 is the query column that sees the tile's first key through the LAST neighbor).
+bool merge_pair(const Group &A, const Group &B, int W, bool scatter, std::vector<int32_t> *out)
+{
+    if (!short_sorted(A) || !short_sorted(B) || W < 4 * S2_LMIN) return false;
+    std::vector<int32_t> tmp;
+    int i = 0, j = 0;
+    while (i < A.n || j < B.n) {
+        const int32_t *ra = i < A.n ? A.runs + 4 * i : nullptr, *rb = j < B.n ? B.runs + 4 * j : nullptr;
+        const bool useA = ra && (!rb || ra[0] <= rb[0]), useB = rb && (!ra || rb[0] <= ra[0]);
+        const int32_t *any = useA ? ra : rb;
+        int s0 = 0, e1 = 0, sA = 0, lenA = 0, sB = 0, lenB = 0;
+        if (useA) sA = centred(ra[1], W), lenA = ra[2];
+        if (useB) sB = centred(rb[1], W), lenB = rb[2];
+        if (useA && useB) {
+            s0 = std::min(sA, sB), e1 = std::max(sA + lenA, sB + lenB);
+        } else if (useA) {
+            s0 = sA, e1 = sA + lenA, sB = sA;
+        } else {
+            s0 = sB, e1 = sB + lenB, sA = sB;
+        }
+        if (e1 - s0 >= S2_LMIN) return false;
+        const int dA = scatter ? e1 - (sA + lenA) : sA - s0, dB = scatter ? e1 - (sB + lenB) : sB - s0;
+        const int32_t rec[8] = {any[0], ((s0 % W) + W) % W, e1 - s0, any[3], dA, lenA, dB, lenB};
+        tmp.insert(tmp.end(), rec, rec + 8);
+        i += useA, j += useB;
+    }
+    if (tmp.size() > 8 * (size_t)S2_PAIR_MAX_RUNS) return false;
+    out->insert(out->end(), tmp.begin(), tmp.end());
+    return true;
+}
+
+// Work list of one grouping for the hybrid kernels: items (latitude, pair index or -1), long-run latitudes and short-run
+// units (single latitudes or pairs) merged by share of work as in order_rows.
+void build_items(const int32_t *off, const int32_t *runs, int ngroups, int W, bool scatter, const std::vector<RowCost> &cost,
+                 std::vector<int32_t> *items, std::vector<int32_t> *pair_off, std::vector<int32_t> *pair_runs)
+{
+    struct Unit {
+        int32_t lat, pair;
+        int64_t c;
+    };
+    std::vector<Unit> dense, vec;
+    pair_off->assign(1, 0);
+    for (int r = 0; r < ngroups; r++) {
+        if (cost[r].dense < cost[r].vector) {
+            dense.push_back({r, -1, cost[r].dense});
+            continue;
+        }
+        if (r + 1 < ngroups && cost[r + 1].dense >= cost[r + 1].vector) {
+            const Group A = {runs + 4 * (size_t)off[r], off[r + 1] - off[r]}, B = {runs + 4 * (size_t)off[r + 1], off[r + 2] - off[r + 1]};
+            if (merge_pair(A, B, W, scatter, pair_runs)) {
+                vec.push_back({r, (int32_t)pair_off->size() - 1, cost[r].vector + cost[r + 1].vector});
+                pair_off->push_back((int32_t)(pair_runs->size() / 8));
+                r++;
+                continue;
+            }
+        }
+        vec.push_back({r, -1, cost[r].vector});
+    }
+    std::stable_sort(dense.begin(), dense.end(), [&](const Unit &a, const Unit &b) { return cost_class(a.c) > cost_class(b.c); });
+    std::stable_sort(vec.begin(), vec.end(), [&](const Unit &a, const Unit &b) { return cost_class(a.c) > cost_class(b.c); });
+    std::vector<int64_t> cd, cv;
+    for (const Unit &u : dense) cd.push_back(u.c);
+    for (const Unit &u : vec) cv.push_back(u.c);
+    merge_by_share(cd, cv, [&](bool d, size_t k) {
+        const Unit &u = d ? dense[k] : vec[k];
+        items->push_back(u.lat);
+        items->push_back(u.pair);
+    });
+}
+
+// appends an array to the blob at a 16-byte boundary, returns its offset in ints
+int32_t append(std::vector<int32_t> &blob, const int32_t *data, size_t n)
+{
+    while (blob.size() % 4) blob.push_back(0);
+    const size_t at = blob.size();
+    blob.insert(blob.end(), data, data + n);
+    return (int32_t)at;
+}
+
+int build_blob(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in, int nlat_out, int nlon_out,
+               std::vector<int32_t> &blob)
+{
     std::vector<HostRun> runs;
     int64_t n = 0;
     const int rc = decompose(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, &runs, &n);
     if (rc != S2ATTN_OK) return rc;
-    if (n != nruns) return s2attn_fail(S2ATTN_E_INVALID, "nruns = %lld does not match the CSR (%lld runs)", (long long)nruns, (long long)n);
 
     const bool up = nlon_out % nlon_in == 0 && nlon_out != nlon_in;
     const int psk = up ? 1 : nlon_in / nlon_out, psq = up ? nlon_out / nlon_in : 1;
     const int nvin = nlat_in * psk, nvout = nlat_out * psq; // virtual latitudes
+    const int W = up ? nlon_in : nlon_out;
 
     // both groupings by stable counting sort (entries keep the CSR's order inside a group)
     std::vector<RowCost> gcost(nvout), scost(nvin);
-    std::fill(gather_off, gather_off + nvout + 1, 0);
-    std::fill(scatter_off, scatter_off + nvin + 1, 0);
+    std::vector<int32_t> goff(nvout + 1, 0), soff(nvin + 1, 0), gruns(4 * (size_t)n), sruns(4 * (size_t)n);
     for (int64_t i = 0; i < n; i++) {
-        gather_off[runs[i].ho + 1]++;
-        scatter_off[runs[i].hi + 1]++;
+        goff[runs[i].ho + 1]++;
+        soff[runs[i].hi + 1]++;
     }
-    for (int r = 0; r < nvout; r++) gather_off[r + 1] += gather_off[r];
-    for (int r = 0; r < nvin; r++) scatter_off[r + 1] += scatter_off[r];
-    std::vector<int32_t> gcur(gather_off, gather_off + nvout), scur(scatter_off, scatter_off + nvin);
+    for (int r = 0; r < nvout; r++) goff[r + 1] += goff[r];
+    for (int r = 0; r < nvin; r++) soff[r + 1] += soff[r];
+    std::vector<int32_t> gcur(goff.begin(), goff.end() - 1), scur(soff.begin(), soff.end() - 1);
     for (int64_t i = 0; i < n; i++) {
         const HostRun &r = runs[i];
         const int32_t g = gcur[r.ho]++, sidx = scur[r.hi]++;
-        gather_runs[4 * g + 0] = r.hi;
-        gather_runs[4 * g + 1] = r.ws;
-        gather_runs[4 * g + 2] = r.len;
-        gather_runs[4 * g + 3] = r.hi / psk; // real input latitude: quadrature weight index, row address
-        scatter_runs[4 * sidx + 0] = r.ho;
-        scatter_runs[4 * sidx + 1] = r.ws;
-        scatter_runs[4 * sidx + 2] = r.len;
-        scatter_runs[4 * sidx + 3] = r.ho / psq; // real output latitude: row address
+        gruns[4 * g + 0] = r.hi;
+        gruns[4 * g + 1] = r.ws;
+        gruns[4 * g + 2] = r.len;
+        gruns[4 * g + 3] = r.hi / psk; // real input latitude: quadrature weight index, row address
+        sruns[4 * sidx + 0] = r.ho;
+        sruns[4 * sidx + 1] = r.ws;
+        sruns[4 * sidx + 2] = r.len;
+        sruns[4 * sidx + 3] = r.ho / psq; // real output latitude: row address
         gcost[r.ho].add(r.len);
         scost[r.hi].add(r.len);
     }
+    std::vector<int32_t> gorder(nvout), gmixed(nvout), sorder(nvin), smixed(nvin);
+    const int32_t gnd = order_rows(gcost, gorder.data(), gmixed.data());
+    const int32_t snd = order_rows(scost, sorder.data(), smixed.data());
+    std::vector<int32_t> gitems, gpoff, gpruns, sitems, spoff, spruns;
+    build_items(goff.data(), gruns.data(), nvout, W, false, gcost, &gitems, &gpoff, &gpruns);
+    build_items(soff.data(), sruns.data(), nvin, W, true, scost, &sitems, &spoff, &spruns);
 
-    ndense[0] = order_rows(gcost, gather_order, gather_order_mixed);
-    ndense[1] = order_rows(scost, scatter_order, scatter_order_mixed);
+    blob.assign(S2ATTN_PLAN_HEADER_INTS, 0);
+    int32_t h[S2ATTN_PLAN_HEADER_INTS] = {};
+    h[S2ATTN_PH_MAGIC] = S2ATTN_PLAN_MAGIC;
+    h[S2ATTN_PH_NVOUT] = nvout, h[S2ATTN_PH_NVIN] = nvin, h[S2ATTN_PH_NRUNS] = (int32_t)n;
+    h[S2ATTN_PH_GATHER_NDENSE] = gnd, h[S2ATTN_PH_SCATTER_NDENSE] = snd;
+    h[S2ATTN_PH_NLAT_IN] = nlat_in, h[S2ATTN_PH_NLON_IN] = nlon_in, h[S2ATTN_PH_NLAT_OUT] = nlat_out, h[S2ATTN_PH_NLON_OUT] = nlon_out;
+    h[S2ATTN_PH_GATHER_OFF] = append(blob, goff.data(), goff.size());
+    h[S2ATTN_PH_GATHER_RUNS] = append(blob, gruns.data(), gruns.size());
+    h[S2ATTN_PH_GATHER_ORDER] = append(blob, gorder.data(), gorder.size());
+    h[S2ATTN_PH_GATHER_ORDER_MIXED] = append(blob, gmixed.data(), gmixed.size());
+    h[S2ATTN_PH_SCATTER_OFF] = append(blob, soff.data(), soff.size());
+    h[S2ATTN_PH_SCATTER_RUNS] = append(blob, sruns.data(), sruns.size());
+    h[S2ATTN_PH_SCATTER_ORDER] = append(blob, sorder.data(), sorder.size());
+    h[S2ATTN_PH_SCATTER_ORDER_MIXED] = append(blob, smixed.data(), smixed.size());
+    h[S2ATTN_PH_GATHER_NITEMS] = (int32_t)(gitems.size() / 2);
+    h[S2ATTN_PH_GATHER_ITEMS] = append(blob, gitems.data(), gitems.size());
+    h[S2ATTN_PH_GATHER_PAIR_OFF] = append(blob, gpoff.data(), gpoff.size());
+    h[S2ATTN_PH_GATHER_PAIR_RUNS] = append(blob, gpruns.data(), gpruns.size());
+    h[S2ATTN_PH_GATHER_NPAIRS] = (int32_t)gpoff.size() - 1;
+    h[S2ATTN_PH_SCATTER_NITEMS] = (int32_t)(sitems.size() / 2);
+    h[S2ATTN_PH_SCATTER_ITEMS] = append(blob, sitems.data(), sitems.size());
+    h[S2ATTN_PH_SCATTER_PAIR_OFF] = append(blob, spoff.data(), spoff.size());
+    h[S2ATTN_PH_SCATTER_PAIR_RUNS] = append(blob, spruns.data(), spruns.size());
+    h[S2ATTN_PH_SCATTER_NPAIRS] = (int32_t)spoff.size() - 1;
+    while (blob.size() % 4) blob.push_back(0);
+    if (blob.size() > 0x7fffffffULL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the plan needs %zu ints, more than its 32-bit offsets index", blob.size());
+    h[S2ATTN_PH_TOTAL] = (int32_t)blob.size();
+    std::copy(h, h + S2ATTN_PLAN_HEADER_INTS, blob.begin());
+    return S2ATTN_OK;
+}
+
+} // namespace
+
+extern "C" int64_t s2attn_plan_count(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                                     int nlat_out, int nlon_out)
+{
+    int64_t n = 0;
+    const int rc = decompose(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, nullptr, &n);
+    return rc == S2ATTN_OK ? n : (int64_t)rc;
+}
+
+extern "C" int64_t s2attn_plan_size(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                                    int nlat_out, int nlon_out)
+{
+    std::vector<int32_t> blob;
+    const int rc = build_blob(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, blob);
+    return rc == S2ATTN_OK ? (int64_t)blob.size() : (int64_t)rc;
+}
+
+extern "C" int s2attn_plan_build(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int nlat_in, int nlon_in,
+                                 int nlat_out, int nlon_out, int32_t *blob_out, int64_t blob_ints)
+{
+    if (!blob_out) return s2attn_fail(S2ATTN_E_INVALID, "plan output buffer is null");
+    std::vector<int32_t> blob;
+    const int rc = build_blob(col_idx, row_off, nnz, nlat_in, nlon_in, nlat_out, nlon_out, blob);
+    if (rc != S2ATTN_OK) return rc;
+    if ((int64_t)blob.size() != blob_ints)
+        return s2attn_fail(S2ATTN_E_INVALID, "the plan of this CSR has %zu ints, the buffer %lld (size it with s2attn_plan_size)", blob.size(), (long long)blob_ints);
+    std::copy(blob.begin(), blob.end(), blob_out);
     return S2ATTN_OK;
 }
 

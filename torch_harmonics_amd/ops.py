@@ -2,11 +2,10 @@
 torch.library operators over the C ABI of libs2attn.so.
 
 Operator set and signatures follow the reference:
-  s2attn::forward / s2attn::backward            attention_kernels::forward / backward
-                                                (attention_interface.cpp:114-119)
-  s2attn::permute_to_nhwc / permute_to_nchw     attention_kernels::permute_to_nhwc / nchw
-                                                (attention_interface.cpp:85-86, fake and autograd
-                                                rules as in attention/_layout.py:76-103)
+  attention_kernels::forward / backward         the reference's own operator names and schemas (attention_interface.cpp:
+  attention_kernels::permute_to_nhwc / _nchw    85-119), registered for the CUDA dispatch key by the C++ binding
+                                                csrc/s2attn_torch.cpp; fake and autograd rules here, as in
+                                                attention_optimized.py:230-322 and attention/_layout.py:76-103
   s2attn::_neighborhood_s2_attention_optimized  the autograd-carrying op
                                                 (attention_optimized.py:230-322)
 Argument order is (k, v, q, ...), outputs of backward are (dk, dv, dq), as there.
@@ -17,13 +16,13 @@ longitude counts as in the reference.  Tensors must live on a ROCm device: there
 """
 
 import ctypes
-from typing import Tuple
+from typing import List, Optional, Tuple
 
 import torch
 
 from . import _lib
 from ._attention_utils import _setup_context_attention_backward
-from .plan import get_plan, get_row_order, get_transposed_csr
+from .plan import get_row_order, get_transposed_csr
 
 _DTYPE_CODE = {torch.float32: _lib.S2ATTN_F32, torch.bfloat16: _lib.S2ATTN_BF16, torch.float16: _lib.S2ATTN_F16}
 
@@ -39,251 +38,52 @@ def _require_gpu(t: torch.Tensor, name: str, device: torch.device = None) -> Non
         raise RuntimeError(f"{name} is on {t.device} but the other operands are on {device}")
 
 
-def _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
-    """Same conditions the reference entry points enforce (attention_cuda_fwd.cu:553-570, attention_cuda_bwd.cu:874-893)."""
-    downsample = nlon_in % nlon_out == 0
-    upsample = nlon_out % nlon_in == 0
-    if not (downsample or upsample):
-        raise RuntimeError(f"either nlon_in ({nlon_in}) must be an integer multiple of nlon_out ({nlon_out}), or vice versa")
-    if num_heads < 1:
-        raise RuntimeError(f"num_heads must be positive, got {num_heads}")
-    for name, t in (("kx", kx), ("vx", vx), ("qy", qy)) + ((("dy", dy),) if dy is not None else ()):
-        if t.dim() != 4:
-            raise RuntimeError(f"{name} must be a 4-dimensional (B, nlat, nlon, heads*channels) tensor, got {t.dim()} dimensions")
-        if not t.is_contiguous():
-            raise RuntimeError(f"{name} must be contiguous")
-    if qy.shape[3] % num_heads != 0:
-        raise RuntimeError(f"q/k channel count ({qy.shape[3]}) must be divisible by num_heads ({num_heads})")
-    if vx.shape[3] % num_heads != 0:
-        raise RuntimeError(f"v channel count ({vx.shape[3]}) must be divisible by num_heads ({num_heads})")
-    if kx.dtype != qy.dtype:
-        raise RuntimeError(f"k dtype ({kx.dtype}) must match q dtype ({qy.dtype})")
-    if vx.dtype != qy.dtype:
-        raise RuntimeError(f"v dtype ({vx.dtype}) must match q dtype ({qy.dtype})")
-    if dy is not None and dy.dtype != qy.dtype:
-        raise RuntimeError(f"dy dtype ({dy.dtype}) must match q dtype ({qy.dtype})")
-    if kx.shape[3] != qy.shape[3]:
-        raise RuntimeError(f"k and q must have the same channel count, got {kx.shape[3]} and {qy.shape[3]}")
-    if kx.shape[:3] != vx.shape[:3] or kx.shape[0] != qy.shape[0]:
-        raise RuntimeError("k and v must share (B, nlat_in, nlon_in) and q must share B")
-    if kx.shape[2] != nlon_in or qy.shape[1] != nlat_out or qy.shape[2] != nlon_out:
-        raise RuntimeError(f"tensor extents do not match nlon_in={nlon_in}, nlat_out={nlat_out}, nlon_out={nlon_out}")
-    if dy is not None and (dy.shape[:3] != qy.shape[:3] or dy.shape[3] != vx.shape[3]):
-        raise RuntimeError("dy must have the shape of the forward output")
-    if quad_weights.numel() != kx.shape[1]:
-        raise RuntimeError(f"quad_weights must have nlat_in = {kx.shape[1]} entries, got {quad_weights.numel()}")
-    if col_idx.dtype != torch.int64 or row_off.dtype != torch.int64:
-        raise RuntimeError("col_idx and row_off must be int64")
-    if qy.dtype not in _DTYPE_CODE and qy.dtype != torch.float64:
-        raise RuntimeError(f"unsupported dtype {qy.dtype}")
+# ---- raw operators: registered by the C++ binding (csrc/s2attn_torch.cpp) under the reference's names -------------------------
+#   attention_kernels::forward / backward / permute_to_nhwc / permute_to_nchw      (attention_interface.cpp:85-119)
+#   s2attn_kernels::forward_lse / backward_saved   the same pair with y and the softmax normaliser handed to the backward
+# Argument checks, output allocation, the plan cache and the launch live there; what Python adds, as in the reference
+# (attention_optimized.py:230-322, _layout.py:76-103), are the fake kernels and the autograd rules.
+_lib.load_torch_ops()
+
+forward = torch.ops.attention_kernels.forward
+backward = torch.ops.attention_kernels.backward
+permute_to_nhwc = torch.ops.attention_kernels.permute_to_nhwc
+permute_to_nchw = torch.ops.attention_kernels.permute_to_nchw
+forward_lse = torch.ops.s2attn_kernels.forward_lse
+backward_saved = torch.ops.s2attn_kernels.backward_saved
 
 
-def _shape_struct(kx, vx, qy, num_heads) -> _lib.ShapeStruct:
-    B, Hi, Wi, CK = kx.shape
-    _, Ho, Wo, _ = qy.shape
-    return _lib.ShapeStruct(B, num_heads, Hi, Wi, Ho, Wo, CK // num_heads, vx.shape[3] // num_heads, _DTYPE_CODE[qy.dtype])
-
-
-def _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, with_lse):
-    _validate(kx, vx, qy, None, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-    for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
-        _require_gpu(t, name, kx.device)
-    if qy.dtype == torch.float64:  # stored as fp64, computed in fp32 like the reference (attention_cuda_utils.cuh:185-190)
-        y, lse = _forward_impl(kx.float(), vx.float(), qy.float(), quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, with_lse)
-        return y.double(), lse
-    y = torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
-    lse = torch.empty((kx.shape[0], num_heads, nlat_out, nlon_out) if with_lse else (0,), dtype=torch.float32, device=kx.device)
-    if y.numel() == 0:
-        return y, lse
-    plan = get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out)
-    shape = _shape_struct(kx, vx, qy, num_heads)
-    qw = quad_weights.to(dtype=torch.float32).contiguous()
-    with torch.cuda.device(kx.device):
-        rc = _lib.load().s2attn_forward_lse(
-            kx.data_ptr(),
-            vx.data_ptr(),
-            qy.data_ptr(),
-            qw.data_ptr(),
-            y.data_ptr(),
-            lse.data_ptr() if with_lse else None,
-            ctypes.byref(plan.struct),
-            ctypes.byref(shape),
-            _stream_ptr(kx.device),
-        )
-    _lib.check(rc, "s2attn_forward_lse")
-    return y, lse
-
-
-@torch.library.custom_op("s2attn::forward", mutates_args=())
-def forward(
-    kx: torch.Tensor,
-    vx: torch.Tensor,
-    qy: torch.Tensor,
-    quad_weights: torch.Tensor,
-    col_idx: torch.Tensor,
-    row_off: torch.Tensor,
-    num_heads: int,
-    nlon_in: int,
-    nlat_out: int,
-    nlon_out: int,
-) -> torch.Tensor:
-    return _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, False)[0]
-
-
-@forward.register_fake
+@torch.library.register_fake("attention_kernels::forward")
 def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
     return torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
 
 
-@torch.library.custom_op("s2attn::forward_lse", mutates_args=())
-def forward_lse(
-    kx: torch.Tensor,
-    vx: torch.Tensor,
-    qy: torch.Tensor,
-    quad_weights: torch.Tensor,
-    col_idx: torch.Tensor,
-    row_off: torch.Tensor,
-    num_heads: int,
-    nlon_in: int,
-    nlat_out: int,
-    nlon_out: int,
-) -> Tuple[torch.Tensor, torch.Tensor]:
-    """forward plus the fp32 log2-domain softmax normaliser [B, num_heads, nlat_out, nlon_out] that backward_saved takes."""
-    return _forward_impl(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, True)
-
-
-@forward_lse.register_fake
-def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
+@torch.library.register_fake("s2attn_kernels::forward_lse")
+def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, plan=None, plan_header=None):
     y = torch.empty((kx.shape[0], nlat_out, nlon_out, vx.shape[3]), dtype=kx.dtype, device=kx.device)
     return y, torch.empty((kx.shape[0], num_heads, nlat_out, nlon_out), dtype=torch.float32, device=kx.device)
 
 
-def _backward_impl(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
-    _validate(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-    for name, t in (("kx", kx), ("vx", vx), ("qy", qy), ("dy", dy), ("quad_weights", quad_weights), ("col_idx", col_idx), ("row_off", row_off)):
-        _require_gpu(t, name, kx.device)
-    saved = y is not None
-    if saved:
-        _require_gpu(y, "y", kx.device)
-        _require_gpu(lse, "lse", kx.device)
-        if y.shape != dy.shape or y.dtype != dy.dtype or not y.is_contiguous():
-            raise RuntimeError("y must be the contiguous forward output (shape and dtype of dy)")
-        if lse.shape != (kx.shape[0], num_heads, nlat_out, nlon_out) or lse.dtype != torch.float32 or not lse.is_contiguous():
-            raise RuntimeError("lse must be the contiguous fp32 (B, num_heads, nlat_out, nlon_out) tensor returned by forward_lse")
-    if qy.dtype == torch.float64:
-        dk, dv, dq = _backward_impl(
-            kx.float(), vx.float(), qy.float(), dy.float(), y.float() if saved else None, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out
-        )
-        return dk.double(), dv.double(), dq.double()
-    dk, dv, dq = torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
-    if qy.numel() == 0 or kx.numel() == 0:
-        return dk.zero_(), dv.zero_(), dq.zero_()
-    plan = get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out)
-    shape = _shape_struct(kx, vx, qy, num_heads)
-    lib = _lib.load()
-    nbytes = lib.s2attn_backward_workspace_bytes(ctypes.byref(shape))
-    _lib.check(nbytes, "s2attn_backward_workspace_bytes")
-    workspace = torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=kx.device)
-    qw = quad_weights.to(dtype=torch.float32).contiguous()
-    head = (kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr())
-    tail = (qw.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), workspace.data_ptr(), ctypes.byref(plan.struct), ctypes.byref(shape), _stream_ptr(kx.device))
-    with torch.cuda.device(kx.device):
-        if saved:
-            rc = lib.s2attn_backward_saved(*head, y.data_ptr(), lse.data_ptr(), *tail)
-        else:
-            rc = lib.s2attn_backward(*head, *tail)
-    _lib.check(rc, "s2attn_backward_saved" if saved else "s2attn_backward")
-    return dk, dv, dq
-
-
-@torch.library.custom_op("s2attn::backward", mutates_args=())
-def backward(
-    kx: torch.Tensor,
-    vx: torch.Tensor,
-    qy: torch.Tensor,
-    dy: torch.Tensor,
-    quad_weights: torch.Tensor,
-    col_idx: torch.Tensor,
-    row_off: torch.Tensor,
-    num_heads: int,
-    nlon_in: int,
-    nlat_out: int,
-    nlon_out: int,
-) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    return _backward_impl(kx, vx, qy, dy, None, None, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-
-
-@backward.register_fake
+@torch.library.register_fake("attention_kernels::backward")
 def _(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
     return torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
 
 
-@torch.library.custom_op("s2attn::backward_saved", mutates_args=())
-def backward_saved(
-    kx: torch.Tensor,
-    vx: torch.Tensor,
-    qy: torch.Tensor,
-    dy: torch.Tensor,
-    y: torch.Tensor,
-    lse: torch.Tensor,
-    quad_weights: torch.Tensor,
-    col_idx: torch.Tensor,
-    row_off: torch.Tensor,
-    num_heads: int,
-    nlon_in: int,
-    nlat_out: int,
-    nlon_out: int,
-) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
-    """backward with the (y, lse) pair of forward_lse, so that the softmax statistics are not recomputed."""
-    return _backward_impl(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out)
-
-
-@backward_saved.register_fake
-def _(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
+@torch.library.register_fake("s2attn_kernels::backward_saved")
+def _(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, plan=None, plan_header=None):
     return torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
 
 
 # ---- layout ops ------------------------------------------------------------------------
 
 
-def _permute(x: torch.Tensor, to_nhwc: bool) -> torch.Tensor:
-    if x.dim() != 4:
-        raise RuntimeError(f"expected a 4-dimensional tensor, got {x.dim()} dimensions")
-    if not x.is_contiguous():
-        raise RuntimeError("layout conversion expects a contiguous tensor")
-    _require_gpu(x, "x")
-    d0, d1, d2, d3 = x.shape
-    out_shape = (d0, d2, d3, d1) if to_nhwc else (d0, d3, d1, d2)
-    out = torch.empty(out_shape, dtype=x.dtype, device=x.device)
-    if x.numel() == 0:
-        return out
-    if x.element_size() not in (2, 4, 8):
-        raise RuntimeError(f"layout conversion supports 2-, 4- and 8-byte elements, got {x.dtype}")
-    lib = _lib.load()
-    fn = lib.s2attn_permute_to_nhwc if to_nhwc else lib.s2attn_permute_to_nchw
-    with torch.cuda.device(x.device):
-        rc = fn(x.data_ptr(), out.data_ptr(), d0, d1, d2, d3, x.element_size(), _stream_ptr(x.device))
-    _lib.check(rc, "s2attn_permute")
-    return out
-
-
-@torch.library.custom_op("s2attn::permute_to_nhwc", mutates_args=())
-def permute_to_nhwc(x: torch.Tensor) -> torch.Tensor:
-    return _permute(x, True)
-
-
-@permute_to_nhwc.register_fake
+@torch.library.register_fake("attention_kernels::permute_to_nhwc")
 def _(x):
     B, C, H, W = x.shape
     return x.new_empty((B, H, W, C))
 
 
-@torch.library.custom_op("s2attn::permute_to_nchw", mutates_args=())
-def permute_to_nchw(x: torch.Tensor) -> torch.Tensor:
-    return _permute(x, False)
-
-
-@permute_to_nchw.register_fake
+@torch.library.register_fake("attention_kernels::permute_to_nchw")
 def _(x):
     B, H, W, C = x.shape
     return x.new_empty((B, C, H, W))
@@ -294,8 +94,8 @@ def _no_context(ctx, inputs, output):
 
 
 # the two conversions are inverses of each other, so each one's gradient is the other one
-permute_to_nhwc.register_autograd(lambda ctx, g: permute_to_nchw(g.contiguous()), setup_context=_no_context)
-permute_to_nchw.register_autograd(lambda ctx, g: permute_to_nhwc(g.contiguous()), setup_context=_no_context)
+torch.library.register_autograd("attention_kernels::permute_to_nhwc", lambda ctx, g: permute_to_nchw(g.contiguous()), setup_context=_no_context)
+torch.library.register_autograd("attention_kernels::permute_to_nchw", lambda ctx, g: permute_to_nhwc(g.contiguous()), setup_context=_no_context)
 
 
 # ---- the autograd-carrying attention op ---------------------------------------------------
@@ -348,36 +148,41 @@ def _neighborhood_s2_attention_saved(
     nlon_in: int,
     nlat_out: int,
     nlon_out: int,
+    plan: Optional[torch.Tensor] = None,
+    plan_header: Optional[List[int]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    return forward_lse(kw.contiguous(), vw.contiguous(), qw.contiguous(), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out)
+    return forward_lse(kw.contiguous(), vw.contiguous(), qw.contiguous(), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header)
 
 
 @_neighborhood_s2_attention_saved.register_fake
-def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
+def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan=None, plan_header=None):
     y = torch.empty((kw.shape[0], nlat_out, nlon_out, vw.shape[3]), dtype=kw.dtype, device=kw.device)
     return y, torch.empty((kw.shape[0], nh, nlat_out, nlon_out), dtype=torch.float32, device=kw.device)
 
 
 def _setup_context_saved(ctx, inputs, output):
-    _setup_context_attention_backward(ctx, inputs, output)
+    _setup_context_attention_backward(ctx, inputs[:10], output)
     ctx.y, ctx.lse = output[0].detach(), output[1].detach()
+    ctx.plan, ctx.plan_header = inputs[10], inputs[11]
     ctx.mark_non_differentiable(output[1])
 
 
 def _neighborhood_s2_attention_bwd_saved(ctx, grad_output, grad_lse):
     col_idx, row_off, quad_weights, kw, vw, qw = ctx.saved_tensors
     dkw, dvw, dqw = backward_saved(
-        kw.contiguous(), vw.contiguous(), qw.contiguous(), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in, ctx.nlat_out, ctx.nlon_out
-    )
-    return dkw, dvw, dqw, None, None, None, None, None, None, None
+        kw.contiguous(), vw.contiguous(), qw.contiguous(), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in, ctx.nlat_out, ctx.nlon_out,
+        ctx.plan, ctx.plan_header,
+    )  # fmt: skip
+    return dkw, dvw, dqw, None, None, None, None, None, None, None, None, None
 
 
 _neighborhood_s2_attention_saved.register_autograd(_neighborhood_s2_attention_bwd_saved, setup_context=_setup_context_saved)
 
 
-def neighborhood_s2_attention(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
-    """Differentiable attention on NHWC heads-packed tensors; what NeighborhoodAttentionS2.forward calls."""
-    return _neighborhood_s2_attention_saved(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out)[0]
+def neighborhood_s2_attention(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan=None, plan_header=None):
+    """Differentiable attention on NHWC heads-packed tensors; what NeighborhoodAttentionS2.forward calls.  plan, plan_header:
+    the psi's plan built ahead of time (the module builds it in its constructor), so that no call copies psi to the host."""
+    return _neighborhood_s2_attention_saved(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header)[0]
 
 
 # Autocast: k, v, q are brought to the active autocast dtype and the op re-entered with autocast off;
@@ -394,10 +199,12 @@ def _make_autocast_impl(device_type: str):
 
 def _make_autocast_impl_saved(device_type: str):
     @torch.library.impl("s2attn::_neighborhood_s2_attention_saved", f"Autocast{device_type.upper()}")
-    def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
+    def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan=None, plan_header=None):
         cast_dtype = torch.get_autocast_dtype(device_type)
         with torch.amp.autocast(device_type, enabled=False):
-            return _neighborhood_s2_attention_saved(kw.to(cast_dtype), vw.to(cast_dtype), qw.to(cast_dtype), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out)
+            return _neighborhood_s2_attention_saved(
+                kw.to(cast_dtype), vw.to(cast_dtype), qw.to(cast_dtype), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header
+            )
 
     return _
 

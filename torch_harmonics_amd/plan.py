@@ -1,6 +1,7 @@
 """
 Neighborhood plans: the run-length form of psi that the kernels consume, built once per
-(col_idx, row_off) pair by the C++ builder in libs2attn.so and cached.
+(col_idx, row_off) pair by the C++ builder in libs2attn.so (one position-independent int32
+array, see include/s2attn.h) and cached.
 
 The reference re-sorts the CSR rows by length on the device on every call
 (attention_cuda_utils.cu:74-113).  Here the conversion happens on the host the first time
@@ -28,40 +29,51 @@ def _version(t: torch.Tensor) -> int:
 
 
 class Plan:
-    """Six int32 arrays plus the two interleaved launch orders on one device, and the ctypes view the library takes."""
+    """The plan blob on one device (one int32 tensor), its header on the host, and the ctypes view the library takes."""
 
-    def __init__(self, arrays, nruns, ndense, keepalive, mixed):
-        self.gather_off, self.gather_runs, self.gather_order, self.scatter_off, self.scatter_runs, self.scatter_order = arrays
-        self.gather_order_mixed, self.scatter_order_mixed = mixed
-        self.nruns = nruns
-        self.gather_ndense, self.scatter_ndense = ndense
+    def __init__(self, blob: torch.Tensor, header, keepalive=None):
+        self.blob = blob
+        self.header = tuple(int(x) for x in header)
         self._keepalive = keepalive
-        self.struct = _lib.PlanStruct(
-            self.gather_off.data_ptr(),
-            self.gather_runs.data_ptr(),
-            self.gather_order.data_ptr(),
-            self.scatter_off.data_ptr(),
-            self.scatter_runs.data_ptr(),
-            self.scatter_order.data_ptr(),
-            nruns,
-            self.gather_ndense,
-            self.scatter_ndense,
-            self.gather_order_mixed.data_ptr(),
-            self.scatter_order_mixed.data_ptr(),
-        )
+        self.struct = _lib.PlanStruct.make(blob.data_ptr(), self.header)
+
+    def _array(self, off_field: str, n: int, width: int = 1) -> torch.Tensor:
+        off = self.header[_lib.PH[off_field]]
+        a = self.blob[off : off + n * width]
+        return a.view(n, width) if width > 1 else a
+
+    # views into the blob (see include/s2attn.h for their meaning)
+    @property
+    def nruns(self):
+        return self.header[_lib.PH["NRUNS"]]
+
+    def arrays(self):
+        """(gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order) as views of the blob."""
+        h, PH = self.header, _lib.PH
+        nvout, nvin, nruns = h[PH["NVOUT"]], h[PH["NVIN"]], h[PH["NRUNS"]]
+        return [
+            self._array("GATHER_OFF", nvout + 1), self._array("GATHER_RUNS", nruns, 4), self._array("GATHER_ORDER", nvout),
+            self._array("SCATTER_OFF", nvin + 1), self._array("SCATTER_RUNS", nruns, 4), self._array("SCATTER_ORDER", nvin),
+        ]  # fmt: skip
+
+    def mixed_orders(self):
+        h, PH = self.header, _lib.PH
+        return self._array("GATHER_ORDER_MIXED", h[PH["NVOUT"]]), self._array("SCATTER_ORDER_MIXED", h[PH["NVIN"]])
+
+    def items(self, side: str):
+        """Work list of the hybrid kernels for side "GATHER" or "SCATTER": (items [n, 2] = (latitude, pair or -1),
+        pair_off [npairs + 1], pair_runs [*, 8] = (lat, ws, len, aux, dA, lenA, dB, lenB))."""
+        h, PH = self.header, _lib.PH
+        n, npairs = h[PH[side + "_NITEMS"]], h[PH[side + "_NPAIRS"]]
+        poff = self._array(side + "_PAIR_OFF", npairs + 1)
+        return self._array(side + "_ITEMS", n, 2), poff, self._array(side + "_PAIR_RUNS", int(poff[-1]) if self.blob.device.type == "cpu" else 0, 8)
+
+    def to(self, device) -> "Plan":
+        return Plan(self.blob.to(device), self.header, self._keepalive)
 
 
-def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int, with_mixed: bool = False):
-    """
-    Runs the library's host builder on CPU copies of the CSR.  Returns
-    ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns, (gather_ndense, scatter_ndense))
-    as CPU int32 tensors; gather_runs has shape (nruns, 4) = (virtual input latitude, ws, len, real input latitude),
-    grouped by virtual output latitude; scatter_runs (virtual output latitude, ws, len, real output latitude), grouped by
-    virtual input latitude.  Virtual latitude = real latitude * ratio + column class on the finer of the two grids (see
-    include/s2attn.h); the first *_ndense entries of each order are the latitudes with long runs.  with_mixed: a fourth
-    element (gather_order_mixed, scatter_order_mixed), the same latitudes with long-run and short-run ones interleaved in
-    proportion to their work (the launch order of the kernels that split their work between matrix cores and vector ALU).
-    """
+def build_host_blob(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int) -> Plan:
+    """Runs the library's host builder on CPU copies of the CSR and returns the plan with its blob in host memory."""
     lib = _lib.load()
     ci = col_idx.detach().to(device="cpu", dtype=torch.int64).contiguous()
     ro = row_off.detach().to(device="cpu", dtype=torch.int64).contiguous()
@@ -69,54 +81,70 @@ def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, 
     nrow = nlat_in if up else nlat_out
     if ro.numel() != nrow + 1:
         raise RuntimeError(f"row_off must have {'nlat_in' if up else 'nlat_out'} + 1 = {nrow + 1} entries, got {ro.numel()}")
-    nnz = ci.numel()
-    nvin = nlat_in * (1 if up else max(nlon_in // max(nlon_out, 1), 1))
-    nvout = nlat_out * (nlon_out // nlon_in if up else 1)
-    nruns = lib.s2attn_plan_count(ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out)
-    _lib.check(nruns, "s2attn_plan_count")
-    arrays = [
-        torch.zeros(nvout + 1, dtype=torch.int32),
-        torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
-        torch.zeros(nvout, dtype=torch.int32),
-        torch.zeros(nvin + 1, dtype=torch.int32),
-        torch.zeros((max(nruns, 1), 4), dtype=torch.int32),
-        torch.zeros(nvin, dtype=torch.int32),
-    ]
-    ndense = torch.zeros(2, dtype=torch.int32)
-    mixed = (torch.zeros(nvout, dtype=torch.int32), torch.zeros(nvin, dtype=torch.int32))
-    rc = lib.s2attn_plan_build(
-        ci.data_ptr(), ro.data_ptr(), nnz, nlat_in, nlon_in, nlat_out, nlon_out, nruns, *[a.data_ptr() for a in arrays], ndense.data_ptr(),
-        mixed[0].data_ptr() if with_mixed else None, mixed[1].data_ptr() if with_mixed else None,
-    )  # fmt: skip
-    _lib.check(rc, "s2attn_plan_build")
-    if with_mixed:
-        return arrays, int(nruns), (int(ndense[0]), int(ndense[1])), mixed
-    return arrays, int(nruns), (int(ndense[0]), int(ndense[1]))
+    args = (ci.data_ptr(), ro.data_ptr(), ci.numel(), nlat_in, nlon_in, nlat_out, nlon_out)
+    n = lib.s2attn_plan_size(*args)
+    _lib.check(n, "s2attn_plan_size")
+    blob = torch.zeros(n, dtype=torch.int32)
+    _lib.check(lib.s2attn_plan_build(*args, blob.data_ptr(), n), "s2attn_plan_build")
+    return Plan(blob, blob[: _lib.PLAN_HEADER_INTS].tolist())
+
+
+def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int, with_mixed: bool = False):
+    """
+    The plan's basic arrays as CPU int32 tensors (views of the blob):
+    ([gather_off, gather_runs, gather_order, scatter_off, scatter_runs, scatter_order], nruns, (gather_ndense, scatter_ndense));
+    gather_runs has shape (nruns, 4) = (virtual input latitude, ws, len, real input latitude),
+    grouped by virtual output latitude; scatter_runs (virtual output latitude, ws, len, real output latitude), grouped by
+    virtual input latitude.  Virtual latitude = real latitude * ratio + column class on the finer of the two grids (see
+    include/s2attn.h); the first *_ndense entries of each order are the latitudes with long runs.  with_mixed: a fourth
+    element (gather_order_mixed, scatter_order_mixed), the same latitudes with long-run and short-run ones interleaved in
+    proportion to their work.
+    """
+    plan = build_host_blob(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    h, PH = plan.header, _lib.PH
+    out = (plan.arrays(), plan.nruns, (h[PH["GATHER_NDENSE"]], h[PH["SCATTER_NDENSE"]]))
+    return out + (plan.mixed_orders(),) if with_mixed else out
+
+
+def _plan_key(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out):
+    return (col_idx.data_ptr(), row_off.data_ptr(), col_idx.numel(), row_off.numel(), _version(col_idx), _version(row_off), str(col_idx.device),
+            nlat_in, nlon_in, nlat_out, nlon_out)  # fmt: skip
 
 
 def get_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int) -> Plan:
-    """Device plan for this psi, from the cache when the same tensors were seen before."""
-    key = (
-        col_idx.data_ptr(),
-        row_off.data_ptr(),
-        col_idx.numel(),
-        row_off.numel(),
-        _version(col_idx),
-        _version(row_off),
-        str(col_idx.device),
-        nlat_in,
-        nlon_in,
-        nlat_out,
-        nlon_out,
-    )
+    """Device plan for this psi, from the cache when the same tensors were seen before; else built from a host copy of the CSR
+    (one device-to-host copy, the first time a psi is seen)."""
+    key = _plan_key(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
     with _lock:
         plan = _cache.get(key)
         if plan is not None:
             _cache.move_to_end(key)
             return plan
-    arrays, nruns, ndense, mixed = build_host_plan(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out, with_mixed=True)
-    dev = col_idx.device
-    plan = Plan([a.to(dev) for a in arrays], nruns, ndense, (col_idx, row_off), [m.to(dev) for m in mixed])
+    host = build_host_blob(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    plan = Plan(host.blob.to(col_idx.device), host.header, (col_idx, row_off))
+    with _lock:
+        _cache[key] = plan
+        while len(_cache) > _MAX_ENTRIES:
+            _cache.popitem(last=False)
+    return plan
+
+
+def plan_from_blob(blob: torch.Tensor, header, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int) -> Plan:
+    """Plan around a blob that already lives on the right device (the module builds it in its constructor and keeps it as a
+    buffer, so no forward ever copies the CSR back to the host).  Cached per blob storage."""
+    key = ("blob", blob.data_ptr(), blob.numel(), _version(blob), str(blob.device))
+    with _lock:
+        plan = _cache.get(key)
+        if plan is not None:
+            _cache.move_to_end(key)
+            return plan
+    PH = _lib.PH
+    header = tuple(int(x) for x in header)
+    if len(header) != _lib.PLAN_HEADER_INTS or header[PH["MAGIC"]] != _lib.PLAN_MAGIC or header[PH["TOTAL"]] != blob.numel() or blob.dtype != torch.int32:
+        raise RuntimeError("plan header does not describe this plan tensor")
+    if (header[PH["NLAT_IN"]], header[PH["NLON_IN"]], header[PH["NLAT_OUT"]], header[PH["NLON_OUT"]]) != (nlat_in, nlon_in, nlat_out, nlon_out):
+        raise RuntimeError("plan was built for other grid extents than this call's")
+    plan = Plan(blob.contiguous(), header, blob)
     with _lock:
         _cache[key] = plan
         while len(_cache) > _MAX_ENTRIES:
