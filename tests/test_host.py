@@ -554,3 +554,32 @@ def test_weight_gradient_split_reduction(n):
     gen = torch.Generator().manual_seed(n)
     g, x = torch.randn(n, 6, generator=gen, dtype=torch.float64), torch.randn(n, 5, generator=gen, dtype=torch.float64)
     torch.testing.assert_close(_weight_grad(g, x), g.t() @ x, rtol=1e-12, atol=1e-9)
+
+
+def test_reference_operator_names_and_schemas_are_registered():
+    """The C++ binding defines the reference's operators verbatim (attention_interface.cpp:85-86, 114-119) and implements them
+    for the CUDA dispatch key (what ROCm tensors dispatch to); Python adds the fake kernels."""
+    want = {
+        "permute_to_nhwc": "attention_kernels::permute_to_nhwc(Tensor x) -> Tensor",
+        "permute_to_nchw": "attention_kernels::permute_to_nchw(Tensor x) -> Tensor",
+        "forward": "attention_kernels::forward(Tensor kx, Tensor vx, Tensor qy, Tensor quad_weights, Tensor col_idx, Tensor row_off, int "
+        "num_heads, int nlon_in, int nlat_out, int nlon_out) -> Tensor",
+        "backward": "attention_kernels::backward(Tensor kx, Tensor vx, Tensor qy, Tensor dy, Tensor quad_weights, Tensor col_idx, Tensor "
+        "row_off, int num_heads, int nlon_in, int nlat_out, int nlon_out) -> (Tensor, Tensor, Tensor)",
+    }
+    for name, schema in want.items():
+        op = getattr(torch.ops.attention_kernels, name).default
+        assert str(op._schema) == schema
+        assert torch.Tag.pt2_compliant_tag in op.tags
+        assert torch._C._dispatch_has_kernel_for_dispatch_key(f"attention_kernels::{name}", "CUDA")
+        assert torch._C._dispatch_has_kernel_for_dispatch_key(f"attention_kernels::{name}", "Meta")
+    assert ops.forward is torch.ops.attention_kernels.forward and ops.backward is torch.ops.attention_kernels.backward
+    assert os.path.exists(_lib.TORCH_LIB_PATH)
+    # fake kernels: shapes and dtypes without touching a device
+    with torch._subclasses.fake_tensor.FakeTensorMode():
+        k, v, q = torch.empty(2, 12, 24, 8), torch.empty(2, 12, 24, 4), torch.empty(2, 6, 12, 8)
+        w, ci, ro = torch.empty(12), torch.empty(50, dtype=torch.int64), torch.empty(7, dtype=torch.int64)
+        y = torch.ops.attention_kernels.forward(k, v, q, w, ci, ro, 2, 24, 6, 12)
+        assert y.shape == (2, 6, 12, 4)
+        dk, dv, dq = torch.ops.attention_kernels.backward(k, v, q, y, w, ci, ro, 2, 24, 6, 12)
+        assert dk.shape == k.shape and dv.shape == v.shape and dq.shape == q.shape
