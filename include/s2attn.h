@@ -144,6 +144,14 @@ typedef struct s2attn_shape {
     int ck; /* per-head channels of q and k */
     int cv; /* per-head channels of v and y */
     int dtype;
+    /* Point strides: elements between two consecutive grid points of a tensor.  0 means packed (num_heads*ck or
+     * num_heads*cv, the reference's contract).  A larger value lets a tensor be a column block of a wider row-major buffer:
+     * q | k | v written by ONE fused projection GEMM and read in place, dq | dk | dv written into one buffer so that the
+     * input gradient is one GEMM (the reference runs three projections, attention.py:530-532).  Latitude and batch strides
+     * follow from it (nlon * ld, nlat * nlon * ld).  Strides must be multiples of 4 elements.  Only the kernels for fp32
+     * heads of 32 channels on at least 64 longitudes take unpacked tensors; other shapes return S2ATTN_E_UNSUPPORTED.
+     * ld_y applies to y (forward output, and the saved output handed to the backward), ld_dy to the upstream gradient. */
+    int ld_k, ld_v, ld_q, ld_y, ld_dy, ld_dk, ld_dv, ld_dq;
 } s2attn_shape;
 
 /*

@@ -149,3 +149,41 @@ def test_non_finite_key_reaches_its_neighbors_and_at_most_their_tiles(d, W):
     dist = torch.minimum((lon - wi0) % W, (wi0 - lon) % W)
     assert not extra[:, dist > 64 + maxlen].any(), "a query further than a tile and a run from the point is untouched"
     assert torch.equal(dirty[0, :, :, :d][~bad.to(DEV)], clean[0, :, :, :d][~bad.to(DEV)])
+
+
+@pytest.mark.parametrize("share", ["qkv", "kv"])
+def test_column_blocks_of_a_fused_projection_are_read_and_written_in_place(share):
+    """q | k | v as column blocks of one (B, nlat, nlon, 3C) buffer (or k | v of a 2C one): same y, lse, dq, dk, dv, bit for bit,
+    as on contiguous copies, and the gradients come back as the column blocks of ONE new buffer."""
+    from torch_harmonics_amd import ops
+
+    B, nh, d, H, W = 2, 2, 32, 12, 96
+    C = nh * d
+    col, roff = ogeo.neighborhood_csr((H, W), (H, W), "equiangular", "equiangular", 0.6)
+    w = ogeo.attention_quad_weights(H, W, "equiangular")
+    gen = torch.Generator(device=DEV).manual_seed(11)
+    geo = (w.to(DEV), col.to(DEV), roff.to(DEV), nh, W, H, W)
+    if share == "qkv":
+        buf = torch.randn(B, H, W, 3 * C, device=DEV, generator=gen)
+        q, k, v = buf.split([C, C, C], dim=-1)
+    else:
+        buf = torch.randn(B, H, W, 2 * C, device=DEV, generator=gen)
+        k, v = buf.split([C, C], dim=-1)
+        q = torch.randn(B, H, W, C, device=DEV, generator=gen)
+    q = q / math.sqrt(d) if share == "kv" else q
+    dy = torch.randn(B, H, W, C, device=DEV, generator=gen)
+    assert not k.is_contiguous()
+    y, lse = ops.forward_lse(k, v, q, *geo)
+    dk, dv, dq = ops.backward_saved(k, v, q, dy, y, lse, *geo)
+    yc, lsec = ops.forward_lse(k.contiguous(), v.contiguous(), q.contiguous(), *geo)
+    dkc, dvc, dqc = ops.backward_saved(k.contiguous(), v.contiguous(), q.contiguous(), dy, yc, lsec, *geo)
+    torch.cuda.synchronize()
+    assert torch.equal(y, yc) and torch.equal(lse, lsec)
+    assert torch.equal(dk, dkc) and torch.equal(dv, dvc) and torch.equal(dq, dqc)
+    assert dk.untyped_storage().data_ptr() == dv.untyped_storage().data_ptr() and dk.stride(2) == buf.shape[3]
+    assert (dq.untyped_storage().data_ptr() == dk.untyped_storage().data_ptr()) == (share == "qkv")
+    # shapes whose kernels do not take column blocks refuse them (the module then projects into separate tensors)
+    small = torch.randn(1, H, W, 3 * 16, device=DEV, generator=gen)
+    qs, ks, vs = small.split([16, 16, 16], dim=-1)
+    with pytest.raises(RuntimeError, match="point stride"):
+        ops.forward_lse(ks, vs, qs, geo[0], geo[1], geo[2], 1, W, H, W)

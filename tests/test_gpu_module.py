@@ -56,6 +56,10 @@ MODULE_CASES = [
     (4, 4, 4, 2, (6, 12), (6, 12), "equiangular", "equiangular", True),
     (4, 8, 4, 4, (12, 24), (6, 12), "equiangular", "equiangular", True),
     (2, 64, 64, 4, (24, 48), (24, 48), "equiangular", "equiangular", False),
+    # heads of 32 channels on at least 64 longitudes: q | k | v projected by one fused GEMM and read in place
+    (2, 64, 64, 2, (12, 96), (12, 96), "equiangular", "equiangular", False),
+    (1, 32, 64, 1, (16, 128), (16, 128), "legendre-gauss", "legendre-gauss", False),
+    (2, 64, 64, 2, (24, 192), (12, 96), "equiangular", "equiangular", False),
     # up-sampling rows (nlon_out a multiple of nlon_in): psi keyed by input latitude, default radius from the input grid
     (4, 4, 4, 1, (6, 12), (12, 24), "equiangular", "equiangular", False),
     (4, 8, 4, 4, (6, 12), (12, 24), "equiangular", "equiangular", False),
@@ -99,18 +103,21 @@ def test_module_output_and_all_gradients(case):
         assert_close("d " + name, prm.grad, params[name].grad, rtol=1e-4, atol=1e-4)
 
 
+@pytest.mark.parametrize("fused", [False, True], ids=["separate", "fused_kv"])
 @pytest.mark.parametrize("frozen", [(), ("k_weights", "v_bias"), ("input",)], ids=["all", "frozen_params", "frozen_input"])
-def test_shared_key_value_input_gradients(frozen):
+def test_shared_key_value_input_gradients(frozen, fused):
     """key is value (one tensor feeding two projections): its gradient is the sum of both projections' input gradients, with
-    any subset of the parameters or the input itself frozen."""
+    any subset of the parameters or the input itself frozen.  fused: heads of 32 channels on 64+ longitudes, where k | v come
+    out of one GEMM as column blocks of one buffer."""
     from torch_harmonics_amd import NeighborhoodAttentionS2
 
     torch.manual_seed(SEED)
-    m = NeighborhoodAttentionS2(8, (12, 24), (6, 12), num_heads=2).to(DEV)
+    C, ins, outs = (64, (12, 128), (6, 64)) if fused else (8, (12, 24), (6, 12))
+    m = NeighborhoodAttentionS2(C, ins, outs, num_heads=2).to(DEV)
     for name in frozen:
         if name != "input":
             getattr(m, name).requires_grad_(False)
-    xq, xkv, gout = torch.randn(2, 8, 6, 12), torch.randn(2, 8, 12, 24), torch.randn(2, 8, 6, 12)
+    xq, xkv, gout = torch.randn(2, C, *outs), torch.randn(2, C, *ins), torch.randn(2, C, *outs)
     dq_ = xq.clone().to(DEV).requires_grad_(True)
     dkv = xkv.clone().to(DEV).requires_grad_("input" not in frozen)
     m(dq_, dkv, dkv).backward(gout.to(DEV))

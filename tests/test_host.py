@@ -583,3 +583,43 @@ def test_reference_operator_names_and_schemas_are_registered():
         assert y.shape == (2, 6, 12, 4)
         dk, dv, dq = torch.ops.attention_kernels.backward(k, v, q, y, w, ci, ro, 2, 24, 6, 12)
         assert dk.shape == k.shape and dv.shape == v.shape and dq.shape == q.shape
+
+
+def test_point_strides_are_validated_on_the_host():
+    """A tensor may be a column block of a wider buffer (point stride > packed row); strides must cover the packed row and be
+    multiples of 4 elements."""
+    lib = _lib.load()
+    ok = _lib.ShapeStruct(1, 8, 721, 1440, 721, 1440, 32, 32, _lib.S2ATTN_F32, 768, 768, 768, 0, 0, 768, 768, 768)
+    assert lib.s2attn_backward_saved_workspace_bytes(ctypes.byref(ok)) == 8 * 721 * 1440 * 8
+    short = _lib.ShapeStruct(1, 8, 721, 1440, 721, 1440, 32, 32, _lib.S2ATTN_F32, 128)  # ld_k below num_heads * ck = 256
+    assert lib.s2attn_backward_saved_workspace_bytes(ctypes.byref(short)) == -1 and b"point stride" in lib.s2attn_last_error()
+    odd = _lib.ShapeStruct(1, 8, 721, 1440, 721, 1440, 32, 32, _lib.S2ATTN_F32, 0, 258)
+    assert lib.s2attn_backward_saved_workspace_bytes(ctypes.byref(odd)) == -1
+    assert ops.takes_column_blocks(torch.float32, 32, 32, 1440, 1440) and not ops.takes_column_blocks(torch.float32, 64, 64, 720, 720)
+    assert not ops.takes_column_blocks(torch.bfloat16, 32, 32, 1440, 1440) and not ops.takes_column_blocks(torch.float32, 32, 32, 48, 48)
+
+
+def test_fused_projection_function_matches_separate_linears():
+    """_FusedLinear1x1 on the CPU (pure torch): outputs, input gradient, weight and bias gradients equal three F.linear,
+    both when the gradients arrive as column blocks of one buffer and when they do not."""
+    from torch_harmonics_amd.attention import _column_blocks_of_one_buffer, _FusedLinear1x1
+
+    gen = torch.Generator().manual_seed(3)
+    x = torch.randn(2, 3, 5, 6, generator=gen, dtype=torch.float64, requires_grad=True)
+    ws = [torch.randn(n, 6, generator=gen, dtype=torch.float64, requires_grad=True) for n in (4, 4, 8)]
+    bs = [torch.randn(n, generator=gen, dtype=torch.float64, requires_grad=True) for n in (4, 4, 8)]
+    outs = _FusedLinear1x1.apply(x, ws[0], bs[0], ws[1], bs[1], ws[2], bs[2])
+    ref = [torch.nn.functional.linear(x, w, b) for w, b in zip(ws, bs)]
+    assert all(torch.allclose(a, b) for a, b in zip(outs, ref)) and outs[0].stride(2) == 16
+    gbuf = torch.randn(2, 3, 5, 16, generator=gen, dtype=torch.float64)
+    blocks = gbuf.split([4, 4, 8], dim=-1)
+    assert _column_blocks_of_one_buffer(blocks, [4, 4, 8]) is not None and _column_blocks_of_one_buffer([b.contiguous() for b in blocks], [4, 4, 8]) is None
+    for grads in (blocks, [b.contiguous() for b in blocks]):
+        for t in [x] + ws + bs:
+            t.grad = None
+        torch.autograd.backward(_FusedLinear1x1.apply(x, ws[0], bs[0], ws[1], bs[1], ws[2], bs[2]), grads)
+        got = [t.grad.clone() for t in [x] + ws + bs]
+        for t in [x] + ws + bs:
+            t.grad = None
+        torch.autograd.backward([torch.nn.functional.linear(x, w, b) for w, b in zip(ws, bs)], grads)
+        assert all(torch.allclose(a, t.grad) for a, t in zip(got, [x] + ws + bs))

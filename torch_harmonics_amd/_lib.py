@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 TORCH_LIB_PATH = os.path.join(_HERE, "_C.so")  # libtorch registration of the operators (csrc/s2attn_torch.cpp)
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 10
+ABI_VERSION = 11
 NOALLOC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 _vp = ctypes.c_void_p
@@ -58,7 +58,9 @@ class ShapeStruct(ctypes.Structure):
         ("ck", _int),
         ("cv", _int),
         ("dtype", _int),
-    ]
+        # point strides in elements, 0 = packed (see include/s2attn.h)
+        ("ld_k", _int), ("ld_v", _int), ("ld_q", _int), ("ld_y", _int), ("ld_dy", _int), ("ld_dk", _int), ("ld_dv", _int), ("ld_dq", _int),
+    ]  # fmt: skip
 
 
 class RingShapeStruct(ctypes.Structure):

@@ -17,7 +17,7 @@ import torch.nn.functional as F
 from ._attention_utils import _check_dtypes_match, _check_extent, _check_ndim
 from ._layout import to_nchw, to_nhwc
 from .neighborhood import precompute_neighborhood_s2
-from .ops import neighborhood_s2_attention
+from .ops import neighborhood_s2_attention, takes_column_blocks
 from .plan import build_host_blob
 from .quadrature import precompute_latitudes
 
@@ -105,6 +105,70 @@ class _SharedInputLinear1x1(torch.autograd.Function):
             out += [gw, gb]
         if gx is not None:
             gx = gx.reshape(x.shape).to(x.dtype)
+        return (gx, *out)
+
+
+def _column_blocks_of_one_buffer(grads, widths):
+    """The 2-D (N, sum(widths)) buffer whose consecutive column blocks the given gradients are, or None."""
+    g0 = grads[0]
+    total = sum(widths)
+    if g0 is None or g0.dim() != 4 or g0.stride(3) != 1 or g0.stride(2) != total:
+        return None
+    off = g0.storage_offset()
+    for g, w in zip(grads, widths):
+        if g is None or g.shape[3] != w or g.shape[:3] != g0.shape[:3] or g.stride() != g0.stride() or g.dtype != g0.dtype:
+            return None
+        if g.untyped_storage().data_ptr() != g0.untyped_storage().data_ptr() or g.storage_offset() != off:
+            return None
+        off += w
+    n = g0.shape[0] * g0.shape[1] * g0.shape[2]
+    if g0.stride(1) != g0.shape[2] * total or g0.stride(0) != g0.shape[1] * g0.shape[2] * total:
+        return None
+    return torch.as_strided(g0, (n, total), (total, 1), g0.storage_offset())
+
+
+class _FusedLinear1x1(torch.autograd.Function):
+    """Several projections of ONE input as ONE GEMM with the concatenated weight: the outputs are the column blocks of one
+    (..., sum of widths) buffer, which the attention kernels read in place.  When the gradients come back as column blocks
+    of one buffer as well (the attention backward writes them that way), the input gradient, the weight gradients and the
+    bias gradients are one GEMM, one split-K GEMM and one reduction over that buffer; otherwise they are concatenated first.
+    (The reference runs three F.linear, attention.py:530-532.)"""
+
+    @staticmethod
+    def forward(ctx, x, *params):  # params = (w0, b0, w1, b1, ...), biases all present or all None
+        weights, biases = params[0::2], params[1::2]
+        wcat = torch.cat(weights, 0)
+        bcat = None if biases[0] is None else torch.cat(biases, 0)
+        ctx.save_for_backward(x, wcat)
+        ctx.widths = [w.shape[0] for w in weights]
+        ctx.has_bias = bcat is not None
+        buf = F.linear(x, wcat, bcat)
+        return tuple(buf.split(ctx.widths, dim=-1))
+
+    @staticmethod
+    def backward(ctx, *grads):
+        x, wcat = ctx.saved_tensors
+        x2 = x.reshape(-1, x.shape[-1])
+        if any(g is None for g in grads):
+            like = next(g for g in grads if g is not None)
+            grads = tuple(g if g is not None else like.new_zeros(like.shape[:-1] + (w,)) for g, w in zip(grads, ctx.widths))
+        g2 = _column_blocks_of_one_buffer(grads, ctx.widths)
+        if g2 is None:
+            g2 = torch.cat([g.reshape(-1, g.shape[-1]) for g in grads], 1)
+        gx = gwcat = gbcat = None
+        if ctx.needs_input_grad[0]:
+            gx = (g2 @ wcat.to(g2.dtype)).reshape(x.shape).to(x.dtype)
+        if any(ctx.needs_input_grad[1::2]):
+            gwcat = _weight_grad(g2, x2.to(g2.dtype)).to(wcat.dtype)
+        if ctx.has_bias and any(ctx.needs_input_grad[2::2]):
+            gbcat = g2.sum(0)
+        out = []
+        ofs = 0
+        for i, w in enumerate(ctx.widths):
+            gw = gwcat[ofs : ofs + w] if gwcat is not None and ctx.needs_input_grad[1 + 2 * i] else None
+            gb = gbcat[ofs : ofs + w] if gbcat is not None and ctx.needs_input_grad[2 + 2 * i] else None
+            out += [gw, gb]
+            ofs += w
         return (gx, *out)
 
 
@@ -285,13 +349,23 @@ class NeighborhoodAttentionS2(nn.Module):
         if not normed:
             wq, bq = wq * self.scale, None if bq is None else bq * self.scale
         wk, wv = self.k_weights.view(self.k_weights.shape[0], -1), self.v_weights.view(self.v_weights.shape[0], -1)
-        # projections that share their input share one backward for the input gradient
+        # Projections that share their input: one fused GEMM whose output the attention kernels read in place (q | k | v as
+        # column blocks of one buffer) where the kernels of this shape take such tensors; else one F.linear each with a shared
+        # backward that accumulates the input gradient inside the GEMMs.
+        fused = (
+            not normed
+            and not torch.is_autocast_enabled()
+            and takes_column_blocks(query.dtype, self.k_channels // self.num_heads, self.out_channels // self.num_heads, self.nlon_in, self.nlon_out)
+            and self.k_channels % 4 == 0
+            and self.out_channels % 4 == 0
+        )
+        shared = _FusedLinear1x1 if fused else _SharedInputLinear1x1
         if key_is_query and value_is_query:
-            query, key, value = _SharedInputLinear1x1.apply(query, wq, bq, wk, self.k_bias, wv, self.v_bias)
+            query, key, value = shared.apply(query, wq, bq, wk, self.k_bias, wv, self.v_bias)
         else:
             query = _Linear1x1.apply(query, wq, bq)
             if value_is_key:
-                key, value = _SharedInputLinear1x1.apply(key, wk, self.k_bias, wv, self.v_bias)
+                key, value = shared.apply(key, wk, self.k_bias, wv, self.v_bias)
             else:
                 key = _Linear1x1.apply(key, wk, self.k_bias)
                 value = _Linear1x1.apply(value, wv, self.v_bias)

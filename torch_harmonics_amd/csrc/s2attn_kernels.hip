@@ -58,7 +58,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 10; }
+extern "C" int s2attn_abi_version(void) { return 11; }
 #endif
 
 namespace s2 {
@@ -285,6 +285,10 @@ struct Args {
     const int *gitems, *sitems, *gpoff, *spoff;
     const PRun *gpruns, *spruns;
     int n_gitems, n_sitems;
+    // elements between two consecutive grid points of each tensor: num_heads * channels when packed, more when the tensor is a
+    // column block of a wider buffer (q | k | v of one fused projection); only the hybrid kernels take unpacked tensors
+    unsigned ldk, ldv, ldq, ldy, ldg, lddk, lddv, lddq;
+    int unpacked; // any of them differs from the packed value
     int B, nh, Hi, Wi, Ho, Wo, dk_, dv_;
     int kps; // nlon_in / nlon_out when the input grid is the finer one, else 1; see key_point()
     int qps; // nlon_out / nlon_in when the output grid is the finer one, else 1; see query_point()
@@ -1628,7 +1632,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
         fwd_pair<T>(a, Ks, Vs, Rs, lane, b, h, w0, nvalid, ho, pair);
         return;
     }
-    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const unsigned ldk = a.ldk, ldv = a.ldv; // elements between two grid points, per tensor (packed heads, or a row of a fused buffer)
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
     const bool mine = j < nvalid;
@@ -1636,7 +1640,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
 
     float qb[16];
     {
-        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 4 * half;
+        const T *qrow = static_cast<const T *>(a.q) + pt * a.ldq + (size_t)h * 32 + 4 * half;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const float4 x = load4(qrow + 8 * g);
@@ -1796,7 +1800,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     if (mine) {
         if (a.lse && half == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + j] = m + fast_log2(S);
         const float inv = 1.0f / S;
-        T *y = static_cast<T *>(a.y) + pt * ldv + (size_t)h * 32 + 4 * half;
+        T *y = static_cast<T *>(a.y) + pt * a.ldy + (size_t)h * 32 + 4 * half;
 #pragma unroll
         for (int g = 0; g < 4; g++) store4(y + 8 * g, make_float4(acc[4 * g] * inv, acc[4 * g + 1] * inv, acc[4 * g + 2] * inv, acc[4 * g + 3] * inv));
     }
@@ -1815,7 +1819,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     // holding q, dy and dq of two latitudes plus the tile prefetch costs the third resident wavefront per SIMD, which the
     // matrix-core path of the same kernel needs more than the short rows need the shared LDS reads.)
     const int ho = a.gorder_mixed[rowsel];
-    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const unsigned ldk = a.ldk, ldv = a.ldv;
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
     const bool mine = j < nvalid;
@@ -1825,9 +1829,9 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     float qb[16], gb[16];
     float I = 0.f;
     {
-        const T *qrow = static_cast<const T *>(a.q) + pt * ldk + (size_t)h * 32 + 4 * half;
-        const T *grow = static_cast<const T *>(a.dy) + pt * ldv + (size_t)h * 32 + 4 * half;
-        const T *yrow = static_cast<const T *>(a.ysaved) + pt * ldv + (size_t)h * 32 + 4 * half;
+        const T *qrow = static_cast<const T *>(a.q) + pt * a.ldq + (size_t)h * 32 + 4 * half;
+        const T *grow = static_cast<const T *>(a.dy) + pt * a.ldg + (size_t)h * 32 + 4 * half;
+        const T *yrow = static_cast<const T *>(a.ysaved) + pt * a.ldy + (size_t)h * 32 + 4 * half;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const float4 x = load4(qrow + 8 * g);
@@ -1971,7 +1975,7 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     // which the compiler only uses while nothing in the kernel can have written memory, into vector loads with waits)
     if (mine && half == 0) a.stats[sidx] = make_float2(lse, I);
     if (mine) {
-        T *dq = static_cast<T *>(a.dq) + pt * ldk + (size_t)h * 32 + 4 * half;
+        T *dq = static_cast<T *>(a.dq) + pt * a.lddq + (size_t)h * 32 + 4 * half;
 #pragma unroll
         for (int g = 0; g < 4; g++) store4(dq + 8 * g, make_float4(dqt[4 * g], dqt[4 * g + 1], dqt[4 * g + 2], dqt[4 * g + 3]));
     }
@@ -1997,17 +2001,17 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
         dkdv_pair<T>(a, Qs, Gs, Ls, Is, Rs, lane, b, h, w0, nvalid, hi, pair);
         return;
     }
-    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
-    const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldk + (size_t)h * 32;
-    const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * 32;
+    const unsigned ldq = a.ldq, ldg = a.ldg;
+    const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldq + (size_t)h * 32;
+    const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldg + (size_t)h * 32;
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = j < nvalid;
     const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? j : 0)) * a.kps;
 
     float kb[16], vb[16];
     {
-        const T *krow = static_cast<const T *>(a.k) + pt * ldk + (size_t)h * 32 + 4 * half;
-        const T *vrow = static_cast<const T *>(a.v) + pt * ldv + (size_t)h * 32 + 4 * half;
+        const T *krow = static_cast<const T *>(a.k) + pt * a.ldk + (size_t)h * 32 + 4 * half;
+        const T *vrow = static_cast<const T *>(a.v) + pt * a.ldv + (size_t)h * 32 + 4 * half;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             const float4 x = load4(krow + 8 * g);
@@ -2034,8 +2038,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
         const bool fifth = !run_is_dense(rn.len);
-        qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldk, ldk * a.qps, c0, a.Wo, lane, fifth);
-        gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldv, ldv * a.qps, c0, a.Wo, lane, fifth);
+        qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldq, ldq * a.qps, c0, a.Wo, lane, fifth);
+        gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldg, ldg * a.qps, c0, a.Wo, lane, fifth);
         int col = c0 + lane; // lanes 0..39 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
         if (lane < MR) st = stats[(size_t)rn.lat * a.Wo + col];
@@ -2166,8 +2170,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     }
 
     if (mine) {
-        T *dk = static_cast<T *>(a.dk) + pt * ldk + (size_t)h * 32 + 4 * half;
-        T *dv = static_cast<T *>(a.dv) + pt * ldv + (size_t)h * 32 + 4 * half;
+        T *dk = static_cast<T *>(a.dk) + pt * a.lddk + (size_t)h * 32 + 4 * half;
+        T *dv = static_cast<T *>(a.dv) + pt * a.lddv + (size_t)h * 32 + 4 * half;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
             store4(dk + 8 * g, make_float4(dkt[4 * g], dkt[4 * g + 1], dkt[4 * g + 2], dkt[4 * g + 3]));
@@ -2322,10 +2326,20 @@ int check_shape(const s2attn_shape *sh)
         return s2attn_fail(S2ATTN_E_INVALID, "nlon_in (%d) must be an integer multiple of nlon_out (%d), or the other way round", sh->nlon_in, sh->nlon_out);
     if (sh->dtype != S2ATTN_F32 && sh->dtype != S2ATTN_BF16 && sh->dtype != S2ATTN_F16)
         return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", sh->dtype);
+    {
+        const int pk = sh->num_heads * sh->ck, pv = sh->num_heads * sh->cv;
+        const int lds[8] = {sh->ld_k, sh->ld_q, sh->ld_dk, sh->ld_dq, sh->ld_v, sh->ld_y, sh->ld_dy, sh->ld_dv};
+        for (int i = 0; i < 8; i++)
+            if (lds[i] != 0 && (lds[i] < (i < 4 ? pk : pv) || lds[i] % 4 != 0))
+                return s2attn_fail(S2ATTN_E_INVALID, "point stride %d is smaller than the packed row (%d) or not a multiple of 4", lds[i], i < 4 ? pk : pv);
+    }
     if (sh->ck > 512 || sh->cv > 512)
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "per-head channels above 512 are not instantiated (ck=%d, cv=%d)", sh->ck, sh->cv);
     // the kernels form offsets inside one latitude of one batch entry in 32 bits
     const long long wmax = sh->nlon_in > sh->nlon_out ? sh->nlon_in : sh->nlon_out, cmax = sh->ck > sh->cv ? sh->ck : sh->cv;
+    long long ldmax = 0;
+    for (int ld : {sh->ld_k, sh->ld_q, sh->ld_dk, sh->ld_dq, sh->ld_v, sh->ld_y, sh->ld_dy, sh->ld_dv}) ldmax = ld > ldmax ? ld : ldmax;
+    if (wmax * ldmax * 4 >= (1LL << 31)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "one latitude row of a strided tensor (%lld points x %lld elements) exceeds 2 GiB", wmax, ldmax);
     if (wmax * sh->num_heads * cmax * 4 >= (1LL << 31))
         return s2attn_fail(S2ATTN_E_UNSUPPORTED, "one latitude row of a tensor (%lld points x %d heads x %lld channels) exceeds 2 GiB", wmax, sh->num_heads, cmax);
     return S2ATTN_OK;
@@ -2488,6 +2502,12 @@ template <typename T> int launch_t(Which which, const Args &a, bool vec, int nde
 {
     const int nrows = which == DKDV ? a.Hi : a.Ho;
     int first = 0;
+    if (a.unpacked) { // column blocks of a wider buffer: only the hybrid kernels address every tensor by its own point stride
+        if (!dense_ok(which, a, vec))
+            return s2attn_fail(S2ATTN_E_UNSUPPORTED, "tensors with a point stride need the hybrid kernels: ck = cv = 32, 16-byte aligned, at least 64 longitudes%s",
+                               which == DQ ? ", backward from saved statistics" : "");
+        return launch_dense<T>(which, a, stream);
+    }
     if (h16_ok<T>(which, a)) {
         if (a.dk_ == 32) return launch_h16<T, 32, false>(which, a, stream);
         if (a.dk_ == 64) return launch_h16<T, 64, false>(which, a, stream);
@@ -2568,7 +2588,13 @@ void fill_args(Args &a, const s2attn_plan *plan, const s2attn_shape *sh, const f
     a.Wi = a.Wo = up ? sh->nlon_in : sh->nlon_out; // columns of a virtual latitude
     a.dk_ = sh->ck;
     a.dv_ = sh->cv;
+    const unsigned pk = (unsigned)sh->num_heads * sh->ck, pv = (unsigned)sh->num_heads * sh->cv;
+    a.ldk = sh->ld_k ? sh->ld_k : pk, a.ldq = sh->ld_q ? sh->ld_q : pk, a.lddk = sh->ld_dk ? sh->ld_dk : pk, a.lddq = sh->ld_dq ? sh->ld_dq : pk;
+    a.ldv = sh->ld_v ? sh->ld_v : pv, a.ldy = sh->ld_y ? sh->ld_y : pv, a.ldg = sh->ld_dy ? sh->ld_dy : pv, a.lddv = sh->ld_dv ? sh->ld_dv : pv;
+    a.unpacked = a.ldk != pk || a.ldq != pk || a.lddk != pk || a.lddq != pk || a.ldv != pv || a.ldy != pv || a.ldg != pv || a.lddv != pv;
 }
+
+
 
 } // namespace
 
@@ -2667,6 +2693,8 @@ extern "C" int s2attn_backward_dq(const void *k, const void *v, const void *q, c
         void *y = ws + round16(n * (int64_t)sizeof(float2)) + round16(n * 4);
         Args f = a;
         f.y = y, f.lse = lse, f.dq = nullptr, f.dy = nullptr;
+        f.ldy = (unsigned)shape->num_heads * shape->cv; // the recomputed output in the workspace is packed
+        a.ldy = f.ldy;
         const int rc2 = launch(FWD, f, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
         if (rc2 != S2ATTN_OK) return rc2;
         a.ysaved = y, a.lse = lse;

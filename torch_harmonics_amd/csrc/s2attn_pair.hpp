@@ -85,7 +85,7 @@ template <typename T>
 __device__ inline void fwd_pair(const Args &a, float *Ks, float *Vs, int *Rs, int lane, int b, int h, int w0, int nvalid, int hoA, int pidx)
 {
     const int j = lane & 31, half = lane >> 5, bh = b * a.nh + h, hoB = hoA + 1;
-    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
+    const unsigned ldk = a.ldk, ldv = a.ldv;
     const T *kx = static_cast<const T *>(a.k) + (size_t)b * a.Hi * a.Wi * ldk + (size_t)h * 32;
     const T *vx = static_cast<const T *>(a.v) + (size_t)b * a.Hi * a.Wi * ldv + (size_t)h * 32;
     const bool mine = j < nvalid;
@@ -93,8 +93,8 @@ __device__ inline void fwd_pair(const Args &a, float *Ks, float *Vs, int *Rs, in
     const size_t ptA = (size_t)query_point(a, b, hoA, hoA / a.qps) + col, ptB = (size_t)query_point(a, b, hoB, hoB / a.qps) + col;
 
     float qA[16], qB[16], accA[16], accB[16];
-    load_half_row(qA, static_cast<const T *>(a.q) + ptA * ldk + (size_t)h * 32 + 4 * half, LOG2E);
-    load_half_row(qB, static_cast<const T *>(a.q) + ptB * ldk + (size_t)h * 32 + 4 * half, LOG2E);
+    load_half_row(qA, static_cast<const T *>(a.q) + ptA * a.ldq + (size_t)h * 32 + 4 * half, LOG2E);
+    load_half_row(qB, static_cast<const T *>(a.q) + ptB * a.ldq + (size_t)h * 32 + 4 * half, LOG2E);
 #pragma unroll
     for (int v = 0; v < 16; v++) accA[v] = 0.f, accB[v] = 0.f;
     float mA = NEG_BIG, SA = 0.f, mB = NEG_BIG, SB = 0.f;
@@ -184,8 +184,8 @@ __device__ inline void fwd_pair(const Args &a, float *Ks, float *Vs, int *Rs, in
             a.lse[((size_t)bh * a.Ho + hoA) * a.Wo + w0 + j] = mA + fast_log2(SA);
             a.lse[((size_t)bh * a.Ho + hoB) * a.Wo + w0 + j] = mB + fast_log2(SB);
         }
-        store_half_row(static_cast<T *>(a.y) + ptA * ldv + (size_t)h * 32 + 4 * half, accA, 1.0f / SA);
-        store_half_row(static_cast<T *>(a.y) + ptB * ldv + (size_t)h * 32 + 4 * half, accB, 1.0f / SB);
+        store_half_row(static_cast<T *>(a.y) + ptA * a.ldy + (size_t)h * 32 + 4 * half, accA, 1.0f / SA);
+        store_half_row(static_cast<T *>(a.y) + ptB * a.ldy + (size_t)h * 32 + 4 * half, accB, 1.0f / SB);
     }
 }
 
@@ -194,9 +194,9 @@ template <typename T>
 __device__ inline void dkdv_pair(const Args &a, float *Qs, float *Gs, float *Ls, float *Is, int *Rs, int lane, int b, int h, int w0, int nvalid, int hiA, int pidx)
 {
     const int j = lane & 31, half = lane >> 5, bh = b * a.nh + h, hiB = hiA + 1;
-    const unsigned ldk = a.nh * 32, ldv = a.nh * 32;
-    const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldk + (size_t)h * 32;
-    const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldv + (size_t)h * 32;
+    const unsigned ldq = a.ldq, ldg = a.ldg;
+    const T *qy = static_cast<const T *>(a.q) + (size_t)b * a.Ho * a.Wo * ldq + (size_t)h * 32;
+    const T *gy = static_cast<const T *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldg + (size_t)h * 32;
     const float2 *stats = a.stats + (size_t)bh * a.Ho * a.Wo;
     const bool mine = j < nvalid;
     const size_t col = (size_t)(w0 + (mine ? j : 0)) * a.kps;
@@ -205,10 +205,10 @@ __device__ inline void dkdv_pair(const Args &a, float *Qs, float *Gs, float *Ls,
     float kA[16], kB[16], vA[16], vB[16], dkA[16], dkB[16], dvA[16], dvB[16];
     {
         const size_t ofs = (size_t)h * 32 + 4 * half;
-        load_half_row(kA, static_cast<const T *>(a.k) + ptA * ldk + ofs, LOG2E);
-        load_half_row(kB, static_cast<const T *>(a.k) + ptB * ldk + ofs, LOG2E);
-        load_half_row(vA, static_cast<const T *>(a.v) + ptA * ldv + ofs, 1.0f);
-        load_half_row(vB, static_cast<const T *>(a.v) + ptB * ldv + ofs, 1.0f);
+        load_half_row(kA, static_cast<const T *>(a.k) + ptA * a.ldk + ofs, LOG2E);
+        load_half_row(kB, static_cast<const T *>(a.k) + ptB * a.ldk + ofs, LOG2E);
+        load_half_row(vA, static_cast<const T *>(a.v) + ptA * a.ldv + ofs, 1.0f);
+        load_half_row(vB, static_cast<const T *>(a.v) + ptB * a.ldv + ofs, 1.0f);
     }
 #pragma unroll
     for (int v = 0; v < 16; v++) dkA[v] = 0.f, dkB[v] = 0.f, dvA[v] = 0.f, dvB[v] = 0.f;
@@ -224,8 +224,8 @@ __device__ inline void dkdv_pair(const Args &a, float *Qs, float *Gs, float *Ls,
     auto fetch = [&](const PRun &rn, int p) {
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
-        qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.aux) * ldk, ldk * a.qps, c0, a.Wo, lane, true);
-        gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.aux) * ldv, ldv * a.qps, c0, a.Wo, lane, true);
+        qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.aux) * ldq, ldq * a.qps, c0, a.Wo, lane, true);
+        gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.aux) * ldg, ldg * a.qps, c0, a.Wo, lane, true);
         int cs = c0 + lane; // lanes 0..39 fetch the statistics of the staged rows
         cs -= (cs >= a.Wo) ? a.Wo : 0;
         if (lane < MR) st = stats[(size_t)rn.lat * a.Wo + cs];
@@ -291,9 +291,9 @@ __device__ inline void dkdv_pair(const Args &a, float *Qs, float *Gs, float *Ls,
 
     if (mine) {
         const size_t ofs = (size_t)h * 32 + 4 * half;
-        store_half_row(static_cast<T *>(a.dk) + ptA * ldk + ofs, dkA, 1.0f);
-        store_half_row(static_cast<T *>(a.dk) + ptB * ldk + ofs, dkB, 1.0f);
-        store_half_row(static_cast<T *>(a.dv) + ptA * ldv + ofs, dvA, 1.0f);
-        store_half_row(static_cast<T *>(a.dv) + ptB * ldv + ofs, dvB, 1.0f);
+        store_half_row(static_cast<T *>(a.dk) + ptA * a.lddk + ofs, dkA, 1.0f);
+        store_half_row(static_cast<T *>(a.dk) + ptB * a.lddk + ofs, dkB, 1.0f);
+        store_half_row(static_cast<T *>(a.dv) + ptA * a.lddv + ofs, dvA, 1.0f);
+        store_half_row(static_cast<T *>(a.dv) + ptB * a.lddv + ofs, dvB, 1.0f);
     }
 }

@@ -49,6 +49,20 @@ void require_gpu(const Tensor &t, const char *name, const c10::Device &dev)
     TORCH_CHECK(t.device() == dev, name, " is on ", t.device(), " but the other operands are on ", dev);
 }
 
+// Activations are contiguous NHWC (the reference's contract) or a COLUMN BLOCK of a contiguous row-major buffer: unit
+// channel stride, one point stride ld >= channels for the longitude axis, latitude and batch strides that follow from it.
+// That is what a slice buf[..., c0:c1] of a fused q | k | v projection is; the library reads it in place.
+// Returns 0 for a packed tensor, else ld; raises for anything else.
+int64_t point_stride(const Tensor &t, const char *name)
+{
+    if (t.is_contiguous()) return 0;
+    const int64_t ld = t.stride(2);
+    const bool ok = t.stride(3) == 1 && ld >= t.size(3) && ld % 4 == 0 && t.stride(1) == t.size(2) * ld && t.stride(0) == t.size(1) * t.size(2) * ld
+                    && t.storage_offset() % 4 == 0;
+    TORCH_CHECK(ok, name, " must be contiguous, or a column block of a contiguous (B, nlat, nlon, width) buffer with width and offset multiples of 4");
+    return ld;
+}
+
 // Same conditions the reference entry points enforce (attention_cuda_fwd.cu:553-570, attention_cuda_bwd.cu:874-893).
 void validate(const Tensor &kx, const Tensor &vx, const Tensor &qy, const Tensor *dy, const Tensor &quad_weights, const Tensor &col_idx,
               const Tensor &row_off, int64_t num_heads, int64_t nlon_in, int64_t nlat_out, int64_t nlon_out)
@@ -61,7 +75,7 @@ void validate(const Tensor &kx, const Tensor &vx, const Tensor &qy, const Tensor
     for (int i = 0; i < 4; i++) {
         if (!ts[i]) continue;
         TORCH_CHECK(ts[i]->dim() == 4, names[i], " must be a 4-dimensional (B, nlat, nlon, heads*channels) tensor, got ", ts[i]->dim(), " dimensions");
-        TORCH_CHECK(ts[i]->is_contiguous(), names[i], " must be contiguous");
+        (void)point_stride(*ts[i], names[i]);
     }
     TORCH_CHECK(qy.size(3) % num_heads == 0, "q/k channel count (", qy.size(3), ") must be divisible by num_heads (", num_heads, ")");
     TORCH_CHECK(vx.size(3) % num_heads == 0, "v channel count (", vx.size(3), ") must be divisible by num_heads (", num_heads, ")");
@@ -160,7 +174,8 @@ s2attn_plan plan_for(const Tensor &col_idx, const Tensor &row_off, int64_t nlat_
 
 s2attn_shape shape_of(const Tensor &kx, const Tensor &vx, const Tensor &qy, int64_t num_heads)
 {
-    s2attn_shape sh;
+    s2attn_shape sh = {};
+    sh.ld_k = (int)point_stride(kx, "kx"), sh.ld_v = (int)point_stride(vx, "vx"), sh.ld_q = (int)point_stride(qy, "qy");
     sh.batch = (int)kx.size(0), sh.num_heads = (int)num_heads;
     sh.nlat_in = (int)kx.size(1), sh.nlon_in = (int)kx.size(2), sh.nlat_out = (int)qy.size(1), sh.nlon_out = (int)qy.size(2);
     sh.ck = (int)(kx.size(3) / num_heads), sh.cv = (int)(vx.size(3) / num_heads);
@@ -217,8 +232,8 @@ std::tuple<Tensor, Tensor, Tensor> backward_impl(const Tensor &kx, const Tensor 
     const bool saved = y != nullptr;
     if (saved) {
         require_gpu(*y, "y", kx.device()), require_gpu(*lse, "lse", kx.device());
-        TORCH_CHECK(y->sizes() == dy.sizes() && y->scalar_type() == dy.scalar_type() && y->is_contiguous(),
-                    "y must be the contiguous forward output (shape and dtype of dy)");
+        TORCH_CHECK(y->sizes() == dy.sizes() && y->scalar_type() == dy.scalar_type(), "y must be the forward output (shape and dtype of dy)");
+        (void)point_stride(*y, "y");
         TORCH_CHECK(lse->dim() == 4 && lse->size(0) == kx.size(0) && lse->size(1) == num_heads && lse->size(2) == nlat_out && lse->size(3) == nlon_out
                         && lse->scalar_type() == at::kFloat && lse->is_contiguous(),
                     "lse must be the contiguous fp32 (B, num_heads, nlat_out, nlon_out) tensor returned by forward_lse");
@@ -229,10 +244,28 @@ std::tuple<Tensor, Tensor, Tensor> backward_impl(const Tensor &kx, const Tensor 
                                row_off, num_heads, nlon_in, nlat_out, nlon_out, plan_blob, plan_header);
         return {std::get<0>(r).to(at::kDouble), std::get<1>(r).to(at::kDouble), std::get<2>(r).to(at::kDouble)};
     }
-    Tensor dk = at::empty_like(kx), dv = at::empty_like(vx), dq = at::empty_like(qy);
+    // Gradients mirror the layout of their tensors: k | v (| q) that are column blocks of ONE buffer get their gradients as the
+    // same column blocks of ONE new buffer, so that the caller's input gradient is a single GEMM over it.
+    Tensor dk, dv, dq;
+    const int64_t ldk = point_stride(kx, "kx"), ldv = point_stride(vx, "vx"), ldq = point_stride(qy, "qy");
+    const bool kv_fused = ldk > 0 && ldk == ldv && kx.storage().is_alias_of(vx.storage()) && kx.storage_offset() / ldk == vx.storage_offset() / ldk;
+    const bool all_fused = kv_fused && ldq == ldk && qy.storage().is_alias_of(kx.storage()) && qy.sizes().slice(0, 3) == kx.sizes().slice(0, 3)
+                           && qy.storage_offset() / ldk == kx.storage_offset() / ldk;
+    if (kv_fused) {
+        Tensor buf = at::empty({kx.size(0), kx.size(1), kx.size(2), ldk}, kx.options());
+        const int64_t used = kx.size(3) + vx.size(3) + (all_fused ? qy.size(3) : 0);
+        if (used != ldk) buf.zero_(); // columns of the buffer that belong to none of the three
+        dk = buf.narrow(3, kx.storage_offset() % ldk, kx.size(3));
+        dv = buf.narrow(3, vx.storage_offset() % ldk, vx.size(3));
+        dq = all_fused ? buf.narrow(3, qy.storage_offset() % ldk, qy.size(3)) : at::empty(qy.sizes(), qy.options());
+    } else {
+        dk = at::empty(kx.sizes(), kx.options()), dv = at::empty(vx.sizes(), vx.options()), dq = at::empty(qy.sizes(), qy.options());
+    }
     if (qy.numel() == 0 || kx.numel() == 0) return {dk.zero_(), dv.zero_(), dq.zero_()};
     const s2attn_plan plan = plan_for(col_idx, row_off, kx.size(1), nlon_in, nlat_out, nlon_out, plan_blob, plan_header);
-    const s2attn_shape sh = shape_of(kx, vx, qy, num_heads);
+    s2attn_shape sh = shape_of(kx, vx, qy, num_heads);
+    sh.ld_dy = (int)point_stride(dy, "dy"), sh.ld_y = saved ? (int)point_stride(*y, "y") : 0;
+    sh.ld_dk = (int)point_stride(dk, "dk"), sh.ld_dv = (int)point_stride(dv, "dv"), sh.ld_dq = (int)point_stride(dq, "dq");
     // the backward that is handed y and lse needs the two statistics per point only; the other one also recomputes y and lse
     const int64_t nbytes = saved ? s2attn_backward_saved_workspace_bytes(&sh) : s2attn_backward_workspace_bytes(&sh);
     check_rc(nbytes, "s2attn_backward_workspace_bytes");

@@ -133,6 +133,16 @@ def _neighborhood_s2_attention_bwd_optimized(ctx, grad_output):
 _neighborhood_s2_attention_optimized.register_autograd(_neighborhood_s2_attention_bwd_optimized, setup_context=_setup_context_attention_backward)
 
 
+def _packed_or_block(t: torch.Tensor) -> torch.Tensor:
+    """t itself when it is contiguous or a column block of a contiguous (B, nlat, nlon, width) buffer (a slice of a fused
+    q | k | v projection, which the kernels read in place), else a contiguous copy."""
+    if t.is_contiguous():
+        return t
+    if t.dim() == 4 and t.stride(3) == 1 and t.stride(2) % 4 == 0 and t.stride(1) == t.shape[2] * t.stride(2) and t.stride(0) == t.shape[1] * t.stride(1) and t.storage_offset() % 4 == 0:
+        return t
+    return t.contiguous()
+
+
 # Same op, but the forward also hands its output and softmax normaliser to the backward (the reference recomputes both,
 # attention_cuda_bwd.cu:856-956).  Two outputs, so it cannot carry the reference's one-tensor signature; the module
 # calls it through neighborhood_s2_attention below.
@@ -151,7 +161,7 @@ def _neighborhood_s2_attention_saved(
     plan: Optional[torch.Tensor] = None,
     plan_header: Optional[List[int]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    return forward_lse(kw.contiguous(), vw.contiguous(), qw.contiguous(), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header)
+    return forward_lse(_packed_or_block(kw), _packed_or_block(vw), _packed_or_block(qw), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header)
 
 
 @_neighborhood_s2_attention_saved.register_fake
@@ -170,8 +180,8 @@ def _setup_context_saved(ctx, inputs, output):
 def _neighborhood_s2_attention_bwd_saved(ctx, grad_output, grad_lse):
     col_idx, row_off, quad_weights, kw, vw, qw = ctx.saved_tensors
     dkw, dvw, dqw = backward_saved(
-        kw.contiguous(), vw.contiguous(), qw.contiguous(), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in, ctx.nlat_out, ctx.nlon_out,
-        ctx.plan, ctx.plan_header,
+        _packed_or_block(kw), _packed_or_block(vw), _packed_or_block(qw), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in,
+        ctx.nlat_out, ctx.nlon_out, ctx.plan, ctx.plan_header,
     )  # fmt: skip
     return dkw, dvw, dqw, None, None, None, None, None, None, None, None, None
 
@@ -551,3 +561,9 @@ def backward_ring_step_upsample_pass2(
 @backward_ring_step_upsample_pass2.register_fake
 def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_norm_buf, dkx, dvx, quad_weights, col_idx, row_off, nlon_in, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out):
     return None
+
+
+def takes_column_blocks(dtype: torch.dtype, ck: int, cv: int, nlon_in: int, nlon_out: int) -> bool:
+    """True for the shapes whose kernels read q, k, v in place out of a wider buffer and write dq, dk, dv into one
+    (fp32 heads of 32 channels on at least 64 longitudes per virtual latitude: the hybrid kernels)."""
+    return dtype == torch.float32 and ck == 32 and cv == 32 and min(nlon_in, nlon_out) >= 64
