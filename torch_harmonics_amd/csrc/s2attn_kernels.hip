@@ -1757,15 +1757,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
                         x[g] = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
                         z[g] = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
                     }
-                    float part = 0.f;
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        part = fmaf(qb[4 * g], x[g].x, part);
-                        part = fmaf(qb[4 * g + 1], x[g].y, part);
-                        part = fmaf(qb[4 * g + 2], x[g].z, part);
-                        part = fmaf(qb[4 * g + 3], x[g].w, part);
-                    }
-                    const float sv = xor32_sum(part);
+                    const float sv = xor32_sum(dot16(qb, x));
                     if (__any(sv > m + RESCALE_THR)) {
                         const float mn = sv > m + RESCALE_THR ? sv : m, corr = fast_exp2(m - mn);
                         S *= corr;
@@ -1931,23 +1923,11 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
 #pragma unroll
             for (int t = 0; t < VC; t++) {
                 if (t < L) {
-                    float4 xk[4];
-                    float ps_ = 0.f, pg_ = 0.f;
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        xk[g] = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
-                        const float4 z = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
-                        ps_ = fmaf(qb[4 * g], xk[g].x, ps_);
-                        ps_ = fmaf(qb[4 * g + 1], xk[g].y, ps_);
-                        ps_ = fmaf(qb[4 * g + 2], xk[g].z, ps_);
-                        ps_ = fmaf(qb[4 * g + 3], xk[g].w, ps_);
-                        pg_ = fmaf(gb[4 * g], z.x, pg_);
-                        pg_ = fmaf(gb[4 * g + 1], z.y, pg_);
-                        pg_ = fmaf(gb[4 * g + 2], z.z, pg_);
-                        pg_ = fmaf(gb[4 * g + 3], z.w, pg_);
-                    }
-                    const float sv = xor32_sum(ps_);
-                    const float gv = xor32_sum(pg_);
+                    float4 xk[4], zv[4];
+                    read_row(xk, kq + t * MLK);
+                    read_row(zv, vq + t * MLK);
+                    const float sv = xor32_sum(dot16(qb, xk));
+                    const float gv = xor32_sum(dot16(gb, zv));
                     const float coef = fast_exp2(sv - lse) * w * (gv - I);
 #pragma unroll
                     for (int g = 0; g < 4; g++) {
@@ -2128,22 +2108,10 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
             for (int i = 0; i < VC; i++) {
                 if (i < L) {
                     float4 xq[4], xg[4];
-                    float ps_ = 0.f, pg_ = 0.f;
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        xq[g] = *reinterpret_cast<const float4 *>(qq + i * MLK + 8 * g);
-                        xg[g] = *reinterpret_cast<const float4 *>(gq + i * MLK + 8 * g);
-                        ps_ = fmaf(kb[4 * g], xq[g].x, ps_);
-                        ps_ = fmaf(kb[4 * g + 1], xq[g].y, ps_);
-                        ps_ = fmaf(kb[4 * g + 2], xq[g].z, ps_);
-                        ps_ = fmaf(kb[4 * g + 3], xq[g].w, ps_);
-                        pg_ = fmaf(vb[4 * g], xg[g].x, pg_);
-                        pg_ = fmaf(vb[4 * g + 1], xg[g].y, pg_);
-                        pg_ = fmaf(vb[4 * g + 2], xg[g].z, pg_);
-                        pg_ = fmaf(vb[4 * g + 3], xg[g].w, pg_);
-                    }
-                    const float s = xor32_sum(ps_);
-                    const float gd = xor32_sum(pg_);
+                    read_row(xq, qq + i * MLK);
+                    read_row(xg, gq + i * MLK);
+                    const float s = xor32_sum(dot16(kb, xq));
+                    const float gd = xor32_sum(dot16(vb, xg));
                     const float p = fast_exp2(s - Ls[j + i]) * w;
                     const float coef = p * (gd - Is[j + i]);
 #pragma unroll

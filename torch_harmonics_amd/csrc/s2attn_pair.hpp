@@ -35,17 +35,19 @@ __device__ inline PRun load_prun(const int *Rs, int k)
     return r;
 }
 
+// Four independent chains of four FMAs, then a tree add: a single chain of 16 dependent FMAs leaves a wavefront waiting on
+// its own previous instruction most of the time (few wavefronts are resident to fill the gaps).
 __device__ inline float dot16(const float (&q)[16], const float4 (&x)[4])
 {
-    float p = 0.f;
+    float p[4];
 #pragma unroll
     for (int g = 0; g < 4; g++) {
-        p = fmaf(q[4 * g], x[g].x, p);
-        p = fmaf(q[4 * g + 1], x[g].y, p);
-        p = fmaf(q[4 * g + 2], x[g].z, p);
-        p = fmaf(q[4 * g + 3], x[g].w, p);
+        p[g] = q[4 * g] * x[g].x;
+        p[g] = fmaf(q[4 * g + 1], x[g].y, p[g]);
+        p[g] = fmaf(q[4 * g + 2], x[g].z, p[g]);
+        p[g] = fmaf(q[4 * g + 3], x[g].w, p[g]);
     }
-    return p;
+    return (p[0] + p[1]) + (p[2] + p[3]);
 }
 
 __device__ inline void axpy16(float (&acc)[16], float c, const float4 (&x)[4])
