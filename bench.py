@@ -283,7 +283,7 @@ def cpu_baseline(cfg, mod, k, v, q, dy):
     t1 = time.perf_counter()
     oracle.backward_f32(ks, vs, qs, gs, w, col_s, ro_s, nh_s, fast=True)
     t2 = time.perf_counter()
-    return {
+    out = {
         "value": pairs / (t2 - t0),
         "unit": "pairs/s",
         "cores": cores,
@@ -293,6 +293,17 @@ def cpu_baseline(cfg, mod, k, v, q, dy):
         "fwd_ms": 1e3 * (t1 - t0),
         "bwd_ms": 1e3 * (t2 - t1),
     }
+    # The forward alone has no scratch and is feasible in full: all heads, all latitudes of the workload (the reference backward
+    # would need 2 * B * heads * nlat_out * nlon_out * max_row_len floats, 383 GB at 721x1440 with 8 heads).
+    full_pairs = cfg["B"] * cfg["nh"] * Wo * int(col.numel())
+    if full_pairs <= 4e9:
+        kf, vf, qf = k.float().cpu().contiguous(), v.float().cpu().contiguous(), q.float().cpu().contiguous()
+        t0 = time.perf_counter()
+        oracle.forward_f32(kf, vf, qf, w, col, ro, cfg["nh"], fast=True)
+        t1 = time.perf_counter()
+        out["full_forward_ms"] = 1e3 * (t1 - t0)
+        out["full_forward_pairs_per_s"] = full_pairs / (t1 - t0)
+    return out
 
 
 def main():

@@ -252,13 +252,21 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void fwd
         // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
         const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
         float mx = -INFINITY;
+        if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask (most steps of a long run)
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const unsigned t = (unsigned)(tb + 16 * kb + v);
-                sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
-                mx = fmaxf(mx, sc[kb][v]);
+                for (int v = 0; v < 4; v++) mx = fmaxf(mx, sc[kb][v]);
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned t = (unsigned)(tb + 16 * kb + v);
+                    sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
+                    mx = fmaxf(mx, sc[kb][v]);
+                }
             }
         }
         mx = h16_quarter_max(mx);
@@ -406,13 +414,21 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
             }
         }
         const int tb = pos + 4 * qd - c;
+        if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const unsigned t = (unsigned)(tb + 16 * kb + v);
-                const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
-                gc[kb][v] = p * (gc[kb][v] - I);
+                for (int v = 0; v < 4; v++) gc[kb][v] = fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) * (gc[kb][v] - I);
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned t = (unsigned)(tb + 16 * kb + v);
+                    const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
+                    gc[kb][v] = p * (gc[kb][v] - I);
+                }
             }
         }
         const uint4 dop = make_uint4(M::pack2(gc[0][0], gc[0][1]), M::pack2(gc[0][2], gc[0][3]), M::pack2(gc[1][0], gc[1][1]), M::pack2(gc[1][2], gc[1][3]));
@@ -546,6 +562,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dkd
             }
         }
         const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
+        const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
             const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 16 * qb + 4 * qd);
@@ -554,8 +571,8 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dkd
             const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const unsigned t = (unsigned)(tb + 16 * qb + v);
-                const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v])) : 0.f;
+                float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v]));
+                if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
                 sc[qb][v] = p;
                 gc[qb][v] = p * (gc[qb][v] - iv[v]);
             }

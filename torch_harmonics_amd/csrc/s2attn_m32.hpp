@@ -234,13 +234,21 @@ template <int D, int NS> __global__ __launch_bounds__(64 * NS) void fwd_m32_kern
         // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
         const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
         float mx = -INFINITY;
+        if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask (most steps of a long run)
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const unsigned t = (unsigned)(tb + 16 * kb + v);
-                sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
-                mx = fmaxf(mx, sc[kb][v]);
+                for (int v = 0; v < 4; v++) mx = fmaxf(mx, sc[kb][v]);
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned t = (unsigned)(tb + 16 * kb + v);
+                    sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
+                    mx = fmaxf(mx, sc[kb][v]);
+                }
             }
         }
         mx = h16_quarter_max(mx);
@@ -378,13 +386,21 @@ template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dq_m32_kerne
         m32_scores<D, PITCH>(gc, Vs, c, qd, gop);
         m32_exchange<NS>(xs, wv, lane, sc, &gc);
         const int tb = pos + 4 * qd - c;
+        if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask
 #pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
+            for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const unsigned t = (unsigned)(tb + 16 * kb + v);
-                const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
-                gc[kb][v] = p * (gc[kb][v] - I);
+                for (int v = 0; v < 4; v++) gc[kb][v] = fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) * (gc[kb][v] - I);
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned t = (unsigned)(tb + 16 * kb + v);
+                    const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
+                    gc[kb][v] = p * (gc[kb][v] - I);
+                }
             }
         }
         m32_accumulate<D, PITCH>(acc, Ks, c, qd, gc);
@@ -501,6 +517,7 @@ template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dkdv_m32_ker
         m32_scores<D, PITCH>(gc, Gs, c, qd, vop);
         m32_exchange<NS>(xs, wv, lane, sc, &gc);
         const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
+        const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
             const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 16 * qb + 4 * qd);
@@ -509,8 +526,8 @@ template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dkdv_m32_ker
             const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const unsigned t = (unsigned)(tb + 16 * qb + v);
-                const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v])) : 0.f;
+                float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v]));
+                if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
                 sc[qb][v] = p;
                 gc[qb][v] = p * (gc[qb][v] - iv[v]);
             }
