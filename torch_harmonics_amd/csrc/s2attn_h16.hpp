@@ -4,11 +4,16 @@
 // Shape domain: ck == cv = dr, a multiple of 8 with dr <= D (the tile is D channels wide, D a multiple of 32; channels
 // from dr on are staged as zeros and never stored), at least 32 columns per virtual latitude, 16-byte aligned rows.
 //
-// One wavefront owns HQ = 16 consecutive longitudes of one latitude for one (batch, head) and walks every run of that
-// latitude in steps of HK = 32 band positions (len + 15 positions per run; position u belongs to the neighborhood of
-// column c iff 0 <= u - c < len).  Lane l = (c = l % 16, qd = l / 16).  Facts about the instruction used below:
-//   A operand: lane supplies A[i = c][k = 8 qd + e], e < 8;   B operand: lane supplies B[k = 8 qd + e][j = c];
-//   D: register v of the lane holds D[i = 4 qd + v][j = c].
+// A workgroup of NW = 4 wavefronts owns 64 consecutive longitudes of one latitude for one (batch, head); wavefront w owns
+// HQ = 16 of them and walks every run of that latitude in steps of HK = 32 band positions (len + 15 positions per run;
+// position u belongs to the neighborhood of column c iff 0 <= u - c < len).  The four walks read one staged band: band
+// row x of a run is the grid point "first longitude of the workgroup + run start + x", wavefront w is at rows
+// 16 w + pos .. + 32 in a step, so a run starts with 80 staged rows and every further step adds 32 for the whole
+// workgroup (each wavefront alone would stage 32 per step: loads through the vector L1 (64 B/clk per CU) and LDS writes
+// (about 75 B/clk per CU measured, against 215 B/clk for 16-byte LDS reads) are what these kernels run out of first).
+// The band lives in LDS as a ring of BR = 128 rows: the 32 rows of the next step never overlap the 80 rows in use, so a
+// step inside a run needs one barrier; the first step of the next run replaces rows in use and needs two.
+// Lane l = (c = l % 16, qd = l / 16).  Facts about the instruction used below:
 // Scores are produced transposed (S^T[position][column]) so that a lane holds 8 positions of ITS column per step:
 // (block kb < 2, v < 4) <-> position 16 kb + 4 qd + v.  Packed to 16 bit in the order e = 4 kb + v these eight values
 // are, unchanged, the B operand of the second product, whose k slot (qd, e) therefore means position 16 kb + 4 qd + v.
@@ -27,8 +32,12 @@ typedef short s16x4_t __attribute__((ext_vector_type(4)));
 typedef float f4v __attribute__((ext_vector_type(4)));
 typedef unsigned u4v __attribute__((ext_vector_type(4)));
 
-constexpr int HQ = 16; // grid points per wavefront
-constexpr int HK = 32; // band positions per step
+constexpr int HQ = 16;                    // grid points per wavefront
+constexpr int HK = 32;                    // band positions per step
+constexpr int NW = 4;                     // wavefronts per workgroup
+constexpr int WQ = HQ * NW;               // grid points per workgroup
+constexpr int FRESH = HK + HQ * (NW - 1); // band rows the first step of a run needs
+constexpr int BR = 128;                   // rows of the LDS ring (a power of two, a multiple of 16, at least FRESH + HK)
 constexpr int HG = 16; // latitudes (in launch order) whose tiles of one longitude range are issued back to back: they run at
                        // the same time on one XCD and fetch the same K/V (Q/dY) rows, so all but the first hit in its L2
 
@@ -62,7 +71,7 @@ template <> struct H16<f16_t> {
     }
 };
 
-// 32 consecutive longitudes (c0.., wrapping once at W) of one latitude/head as a [32][row] LDS tile: rows of CPR_
+// (Staging of the fp32 family, s2attn_m32.hpp, one band per wavefront.)  32 consecutive longitudes (c0.., wrapping once at W) of one latitude/head as a [32][row] LDS tile: rows of CPR_
 // 16-byte pieces, PITCH_ bytes apart.  fetch() keeps the tile in registers (one 16-byte load per lane per iteration) so
 // that the loads of the next step fly while the current one is consumed; commit() writes it to LDS.
 template <int CPR_, int PITCH_> struct BandTile {
@@ -105,26 +114,81 @@ template <int CPR_, int PITCH_> struct BandTile {
     }
 };
 
-// 16-bit tile of D channels.  Row pitch measured with SQ_LDS_BANK_CONFLICT: pitches of 32 or 96 bytes modulo 128 are free
-// of bank conflicts for all three access patterns (16-byte row pieces by lanes (c, qd), transposing 8-byte reads, 16-byte
+// The staged band of two tensors that share their addressing (k and v, or q and dy): rows of CPR 16-byte pieces, PITCH
+// bytes apart, row x of the run at ring row x % BR.  fetch() loads rows x0 .. x0 + n of the run into registers, one
+// 16-byte piece per thread per iteration and tensor (the loads fly while the current step is consumed); commit() writes
+// them to LDS.  Row pitch measured with SQ_LDS_BANK_CONFLICT: pitches of 32 or 96 bytes modulo 128 are free of bank
+// conflicts for all three access patterns (16-byte row pieces by lanes (c, qd), transposing 8-byte reads, 16-byte
 // writes); 2 D + 16 costs both reads 2x.
-template <int D> struct HTile : BandTile<D / 8, 2 * D + 32> {};
+template <int D> struct WgBand {
+    static constexpr int CPR = D / 8;                   // 16-byte pieces per row
+    static constexpr int PITCH = 2 * D + 32;            // bytes
+    static constexpr int RPI = 64 * NW / CPR;           // rows per iteration of the workgroup
+    static constexpr int NIT = (FRESH + RPI - 1) / RPI; // iterations for the first step of a run
+    static constexpr int BYTES = BR * PITCH;            // one tensor's ring
+    u4v ra[NIT], rb[NIT];
 
-// A operand "channels 16 cb + c, positions (kb, v) of this lane's quarter" from a [position][channel] tile
-template <int PITCH> __device__ inline uint4 h16_read_transposed(const char *tile, int cb, int c, int qd)
+    // cbase: longitude of band row 0 on the circle of W columns (0 <= cbase < W); ldc: bytes between two columns.
+    // N (FRESH or HK) is the number of rows; iterations and row tests that N rules out are not compiled.
+    template <int N, bool PAD> __device__ inline void fetch(const char *pa, const char *pb, int tid, int cbase, int x0, int W, unsigned ldc, bool piece_ok)
+    {
+        const int r0 = tid / CPR;
+        const unsigned pc = 16u * (tid % CPR);
+        int cs = (cbase + x0) % W;
+#pragma unroll
+        for (int it = 0; it < (N + RPI - 1) / RPI; it++) {
+            if (PAD) { // a thread may own a piece beyond the end of the row (a head narrower than the tile): it stages zeros
+                ra[it] = u4v{0u, 0u, 0u, 0u};
+                rb[it] = u4v{0u, 0u, 0u, 0u};
+            }
+            if (((it + 1) * RPI <= N || it * RPI + r0 < N) && (!PAD || piece_ok)) {
+                unsigned col = (unsigned)(cs + r0); // r0 < RPI <= 64 <= 2 W
+                col = min(col, col - (unsigned)W);  // col - W wraps to a huge value when col < W
+                if (RPI > 32) col = min(col, col - (unsigned)W);
+                const unsigned off = col * ldc + pc;
+                ra[it] = *reinterpret_cast<const u4v *>(pa + off);
+                rb[it] = *reinterpret_cast<const u4v *>(pb + off);
+            }
+            cs += RPI;
+            while (cs >= W) cs -= W;
+        }
+    }
+    template <int N> __device__ inline void commit(char *A, char *B, int tid, int x0) const
+    {
+        const int r0 = tid / CPR, pc = 16 * (tid % CPR);
+#pragma unroll
+        for (int it = 0; it < (N + RPI - 1) / RPI; it++) {
+            if ((it + 1) * RPI <= N || it * RPI + r0 < N) {
+                const int o = ((x0 + it * RPI + r0) & (BR - 1)) * PITCH + pc;
+                *reinterpret_cast<u4v *>(A + o) = ra[it];
+                *reinterpret_cast<u4v *>(B + o) = rb[it];
+            }
+        }
+    }
+};
+
+// start of the 16 ring rows that hold band rows x .. x + 16 (x a multiple of 16)
+template <int PITCH> __device__ inline const char *band_block(const char *ring, int x)
+{
+    return ring + (x & (BR - 1)) * PITCH;
+}
+
+// A operand "channels 16 cb + c, positions (kb, v) of this lane's quarter" from the two 16-row blocks of a step
+// ([position][channel] rows)
+template <int PITCH> __device__ inline uint4 h16_read_transposed(const char *blk0, const char *blk1, int cb, int c, int qd)
 {
     typedef s16x4_t __attribute__((address_space(3))) * lds_ptr;
-    const char *p0 = tile + (4 * qd + (c >> 2)) * PITCH + 32 * cb + 8 * (c & 3);
-    const s16x4_t r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0));
-    const s16x4_t r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(p0 + 16 * PITCH));
+    const int o = (4 * qd + (c >> 2)) * PITCH + 32 * cb + 8 * (c & 3);
+    const s16x4_t r0 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(blk0 + o));
+    const s16x4_t r1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_ptr)(blk1 + o));
     const uint2 u0 = __builtin_bit_cast(uint2, r0), u1 = __builtin_bit_cast(uint2, r1);
     return make_uint4(u0.x, u0.y, u1.x, u1.y);
 }
 
-// A operand "row 16 kb + c, channels 32 s + 8 qd .. + 8" (plain 16-byte read)
-template <int PITCH> __device__ inline uint4 h16_read_row(const char *tile, int kb, int s, int c, int qd)
+// A operand "row c of the block, channels 32 s + 8 qd .. + 8" (plain 16-byte read)
+template <int PITCH> __device__ inline uint4 h16_read_row(const char *blk, int s, int c, int qd)
 {
-    return *reinterpret_cast<const uint4 *>(tile + (16 * kb + c) * PITCH + 64 * s + 16 * qd);
+    return *reinterpret_cast<const uint4 *>(blk + c * PITCH + 64 * s + 16 * qd);
 }
 
 // one 16-byte piece of a grid point's vector, zeros when the head ends before it
@@ -160,10 +224,11 @@ __device__ inline void xcd_split(int id, int BH, int per_bh, int &bh, int &rest)
 }
 
 #define S2_H16_IDS(W_TILED, NROWS)                                            \
-    const int lane = threadIdx.x;                                             \
+    const int tid = threadIdx.x;                                              \
+    const int lane = tid & 63, wave = tid >> 6;                               \
     const int c = lane & 15, qd = lane >> 4;                                  \
     const int BH = a.B * a.nh;                                                \
-    const int ntile = ((W_TILED) + HQ - 1) / HQ;                              \
+    const int ntile = ((W_TILED) + WQ - 1) / WQ;                              \
     int bh, id_;                                                              \
     xcd_split(blockIdx.x, BH, ntile *(NROWS), bh, id_);                       \
     const int grp_ = id_ / (HG * ntile);                                      \
@@ -172,17 +237,67 @@ __device__ inline void xcd_split(int id, int BH, int per_bh, int &bh, int &rest)
     const int wt = id_ / grows_;                                              \
     const int rowsel = grp_ * HG + id_ % grows_;                              \
     const int b = bh / a.nh, h = bh % a.nh;                                   \
-    const int w0 = wt * HQ;                                                   \
-    const int nvalid = min(HQ, (W_TILED)-w0);
+    const int wg0 = wt * WQ;                          /* first longitude of the workgroup */ \
+    const bool active = wg0 + HQ * wave < (W_TILED); /* a wavefront past the end of the row only helps staging */ \
+    const int w0 = active ? wg0 + HQ * wave : 0;                              \
+    const int nvalid = active ? min(HQ, (W_TILED)-w0) : 0;
 
 // ---- forward ---------------------------------------------------------------------------------------------------
-template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void fwd_h16_kernel(const Args a)
+// Dynamic LDS of the three kernels: the rings of the two staged tensors (the dk/dv pass keeps two floats per band row in
+// the padding of the first ring's rows: with 64 channels the two rings are exactly a quarter of a CU's LDS).
+template <int D> constexpr int h16_lds_bytes() { return 2 * WgBand<D>::BYTES; }
+
+// Uniform reads of the plan and the weights inside the walk.  A load through the constant address space is always a
+// scalar load; through a plain pointer it becomes a vector load with a full wait as soon as the loop holds a workgroup
+// barrier, whose fence the compiler has to assume orders a write to the same memory.  Neither array is written by a kernel.
+template <typename V> __device__ inline V uniform_load(const V *p)
 {
-    typedef HTile<D> Tile;
+    typedef const V __attribute__((address_space(4))) * cptr;
+    return *(cptr)(p);
+}
+__device__ inline Run uniform_load(const Run *p)
+{
+    typedef int i4v __attribute__((ext_vector_type(4)));
+    const i4v r = uniform_load(reinterpret_cast<const i4v *>(p));
+    return Run{r[0], r[1], r[2], r[3]};
+}
+
+// One step of the walk over the runs of a latitude, the same for every wavefront of the workgroup: where the walk
+// stands after this step, and what has to be staged for it.
+struct H16Walk {
+    int ri, rend, pos;
+    Run run;
+    int nri, npos;
+    Run nrun;
+    bool more, fresh;
+    __device__ inline void plan(const Run *runs)
+    {
+        nri = ri;
+        npos = pos + HK;
+        nrun = run;
+        if (npos >= run.len + HQ - 1) {
+            nri++;
+            npos = 0;
+            if (nri < rend) nrun = uniform_load(runs + nri);
+        }
+        more = nri < rend;
+        fresh = npos == 0;
+    }
+    __device__ inline void advance()
+    {
+        ri = nri;
+        pos = npos;
+        run = nrun;
+    }
+};
+
+template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) void fwd_h16_kernel(const Args a)
+{
+    typedef WgBand<D> Tile;
     typedef H16<T> M;
     constexpr int PITCH = Tile::PITCH, NS = D / 32, NCB = D / 16;
-    __shared__ __attribute__((aligned(16))) char Ks[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) char Vs[HK * PITCH];
+    extern __shared__ __attribute__((aligned(16))) char h16_lds[];
+    char *Ks = h16_lds, *Vs = h16_lds + Tile::BYTES;
 
     S2_H16_IDS(a.Wo, a.Ho)
     const int ho = a.gorder[a.row_first + rowsel];
@@ -204,103 +319,98 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void fwd
     for (int cb = 0; cb < NCB; cb++) acc[cb] = f4v{0.f, 0.f, 0.f, 0.f};
     float m = NEG_BIG, S = 0.f;
 
-    int ri = a.goff[ho];
-    const int rend = a.goff[ho + 1];
-    int pos = 0;
-    Run run = {0, 0, 0, 0};
-    Tile kt, vt;
+    H16Walk wk;
+    wk.ri = a.goff[ho];
+    wk.rend = a.goff[ho + 1];
+    wk.pos = 0;
+    wk.run = Run{0, 0, 0, 0};
+    Tile bd;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
-    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
-    const bool piece_ok = 8 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int p) {
-        const int c0 = (rn.ws + w0 + p) % a.Wi;
-        unsigned off[Tile::NIT];
-        Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
+    const bool piece_ok = 8 * (tid % Tile::CPR) < dr; // this thread's 16-byte piece of a staged row exists
+    auto fetch = [&](const Run &rn, int x0) {
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        kt.fetch_if(kx + lat_off, off, piece_ok);
-        vt.fetch_if(vx + lat_off, off, piece_ok);
+        if (x0 == 0)
+            bd.template fetch<FRESH, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, 0, a.Wi, ldbk, piece_ok);
+        else
+            bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, x0, a.Wi, ldbk, piece_ok);
     };
-    if (ri < rend) {
-        run = a.gruns[ri];
-        fetch(run, 0);
-        kt.commit(Ks, lane);
-        vt.commit(Vs, lane);
+    if (wk.ri < wk.rend) {
+        wk.run = a.gruns[wk.ri];
+        fetch(wk.run, 0);
+        bd.template commit<FRESH>(Ks, Vs, tid, 0);
     }
     __syncthreads();
     settle(qop);
 
-    while (ri < rend) {
-        const float lw = fast_log2(a.quad_w[run.pad]);
-        const int len = run.len;
-        int nri = ri, npos = pos + HK;
-        Run nrun = run;
-        if (npos >= len + HQ - 1) {
-            nri++;
-            npos = 0;
-            if (nri < rend) nrun = a.gruns[nri];
-        }
-        const bool more = nri < rend;
-        if (more) fetch(nrun, npos);
-
-        f4v sc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            sc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < NS; s++) sc[kb] = M::mfma(h16_read_row<PITCH>(Ks, kb, s, c, qd), qop[s], sc[kb]);
-        }
-        // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
-        const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
-        float mx = -INFINITY;
-        if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask (most steps of a long run)
+    while (wk.ri < wk.rend) {
+        wk.plan(a.gruns);
+        if (wk.more) fetch(wk.nrun, wk.fresh ? 0 : FRESH - HK + wk.npos);
+        if (active) {
+            const float lw = fast_log2(uniform_load(a.quad_w + wk.run.pad));
+            const int len = wk.run.len, pos = wk.pos;
+            const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
+            const char *kblk[2] = {band_block<PITCH>(Ks, xw), band_block<PITCH>(Ks, xw + 16)};
+            const char *vblk[2] = {band_block<PITCH>(Vs, xw), band_block<PITCH>(Vs, xw + 16)};
+            f4v sc[2];
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
+                sc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int v = 0; v < 4; v++) mx = fmaxf(mx, sc[kb][v]);
+                for (int s = 0; s < NS; s++) sc[kb] = M::mfma(h16_read_row<PITCH>(kblk[kb], s, c, qd), qop[s], sc[kb]);
             }
-        } else {
+            // band mask, running maximum (of score * log2 e + log2 w, common to the four lanes of a column), probabilities
+            const int tb = pos + 4 * qd - c; // neighbor index of element (kb, v): tb + 16 kb + v
+            float mx = -INFINITY;
+            if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask (most steps of a long run)
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) mx = fmaxf(mx, sc[kb][v]);
+                }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const unsigned t = (unsigned)(tb + 16 * kb + v);
+                        sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
+                        mx = fmaxf(mx, sc[kb][v]);
+                    }
+                }
+            }
+            mx = h16_quarter_max(mx);
+            const float mn = fmaxf(m, fmaf(mx, LOG2E, lw)); // m starts finite, so mn is finite
+            if (__any(mn > m)) {
+                const float corr = fast_exp2(m - mn);
+                S *= corr;
+#pragma unroll
+                for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
+            }
+            m = mn;
+            const float sh = lw - mn;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const unsigned t = (unsigned)(tb + 16 * kb + v);
-                    sc[kb][v] = (t < (unsigned)len) ? sc[kb][v] : -INFINITY;
-                    mx = fmaxf(mx, sc[kb][v]);
+                    const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // masked: exp2(-inf) = 0
+                    sc[kb][v] = p;
+                    S += p; // this lane's share; the four lanes of a column are added up at the end
                 }
             }
+            const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[cb] = M::mfma(h16_read_transposed<PITCH>(vblk[0], vblk[1], cb, c, qd), pop, acc[cb]);
         }
-        mx = h16_quarter_max(mx);
-        const float mn = fmaxf(m, fmaf(mx, LOG2E, lw)); // m starts finite, so mn is finite
-        if (__any(mn > m)) {
-            const float corr = fast_exp2(m - mn);
-            S *= corr;
-#pragma unroll
-            for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
-        }
-        m = mn;
-        const float sh = lw - mn;
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // masked: exp2(-inf) = 0
-                sc[kb][v] = p;
-                S += p; // this lane's share; the four lanes of a column are added up at the end
+        if (wk.more) {
+            if (wk.fresh) {
+                __syncthreads(); // the next run's rows replace rows the slowest wavefront may still be reading
+                bd.template commit<FRESH>(Ks, Vs, tid, 0);
+            } else {
+                bd.template commit<HK>(Ks, Vs, tid, FRESH - HK + wk.npos);
             }
         }
-        const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
-#pragma unroll
-        for (int cb = 0; cb < NCB; cb++) acc[cb] = M::mfma(h16_read_transposed<PITCH>(Vs, cb, c, qd), pop, acc[cb]);
-
         __syncthreads();
-        if (more) {
-            kt.commit(Ks, lane);
-            vt.commit(Vs, lane);
-        }
-        __syncthreads();
-        ri = nri;
-        pos = npos;
-        run = nrun;
+        wk.advance();
     }
 
     S = h16_quarter_sum(S);
@@ -317,13 +427,13 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void fwd
 
 // ---- backward, dq pass (needs the forward's y and lse) -------------------------------------------------------------
 // Three products per step:  S^T = K Q^T,  G^T = V dY^T,  dQ^T += K^T dS^T  with dS = P o (G - I),  I = <dy, y>.
-template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_h16_kernel(const Args a)
+template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) void dq_h16_kernel(const Args a)
 {
-    typedef HTile<D> Tile;
+    typedef WgBand<D> Tile;
     typedef H16<T> M;
     constexpr int PITCH = Tile::PITCH, NS = D / 32, NCB = D / 16;
-    __shared__ __attribute__((aligned(16))) char Ks[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) char Vs[HK * PITCH];
+    extern __shared__ __attribute__((aligned(16))) char h16_lds[];
+    char *Ks = h16_lds, *Vs = h16_lds + Tile::BYTES;
 
     S2_H16_IDS(a.Wo, a.Ho)
     const int ho = a.gorder[a.row_first + rowsel];
@@ -361,27 +471,25 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
 #pragma unroll
     for (int cb = 0; cb < NCB; cb++) acc[cb] = f4v{0.f, 0.f, 0.f, 0.f};
 
-    int ri = a.goff[ho];
-    const int rend = a.goff[ho + 1];
-    int pos = 0;
-    Run run = {0, 0, 0, 0};
-    Tile kt, vt;
+    H16Walk wk;
+    wk.ri = a.goff[ho];
+    wk.rend = a.goff[ho + 1];
+    wk.pos = 0;
+    wk.run = Run{0, 0, 0, 0};
+    Tile bd;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
-    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbk + 16u * (lane % Tile::CPR);
-    const bool piece_ok = 8 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int p) {
-        const int c0 = (rn.ws + w0 + p) % a.Wi;
-        unsigned off[Tile::NIT];
-        Tile::offsets(off, lane_off, lane, c0, a.Wi, ldbk);
+    const bool piece_ok = 8 * (tid % Tile::CPR) < dr; // this thread's 16-byte piece of a staged row exists
+    auto fetch = [&](const Run &rn, int x0) {
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        kt.fetch_if(kx + lat_off, off, piece_ok);
-        vt.fetch_if(vx + lat_off, off, piece_ok);
+        if (x0 == 0)
+            bd.template fetch<FRESH, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, 0, a.Wi, ldbk, piece_ok);
+        else
+            bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, x0, a.Wi, ldbk, piece_ok);
     };
-    if (ri < rend) {
-        run = a.gruns[ri];
-        fetch(run, 0);
-        kt.commit(Ks, lane);
-        vt.commit(Vs, lane);
+    if (wk.ri < wk.rend) {
+        wk.run = a.gruns[wk.ri];
+        fetch(wk.run, 0);
+        bd.template commit<FRESH>(Ks, Vs, tid, 0);
     }
     __syncthreads();
     settle(qop);
@@ -389,61 +497,58 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
     float lse_ = lse;
     settle(lse_);
 
-    while (ri < rend) {
-        const float lwl = fast_log2(a.quad_w[run.pad]) - lse_;
-        const int len = run.len;
-        int nri = ri, npos = pos + HK;
-        Run nrun = run;
-        if (npos >= len + HQ - 1) {
-            nri++;
-            npos = 0;
-            if (nri < rend) nrun = a.gruns[nri];
-        }
-        const bool more = nri < rend;
-        if (more) fetch(nrun, npos);
-
-        f4v sc[2], gc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; kb++) {
-            sc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
-            gc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-            for (int s = 0; s < NS; s++) {
-                sc[kb] = M::mfma(h16_read_row<PITCH>(Ks, kb, s, c, qd), qop[s], sc[kb]);
-                gc[kb] = M::mfma(h16_read_row<PITCH>(Vs, kb, s, c, qd), gop[s], gc[kb]);
-            }
-        }
-        const int tb = pos + 4 * qd - c;
-        if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask
+    while (wk.ri < wk.rend) {
+        wk.plan(a.gruns);
+        if (wk.more) fetch(wk.nrun, wk.fresh ? 0 : FRESH - HK + wk.npos);
+        if (active) {
+            const float lwl = fast_log2(uniform_load(a.quad_w + wk.run.pad)) - lse_;
+            const int len = wk.run.len, pos = wk.pos;
+            const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
+            const char *kblk[2] = {band_block<PITCH>(Ks, xw), band_block<PITCH>(Ks, xw + 16)};
+            const char *vblk[2] = {band_block<PITCH>(Vs, xw), band_block<PITCH>(Vs, xw + 16)};
+            f4v sc[2], gc[2];
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
+                sc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
+                gc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int v = 0; v < 4; v++) gc[kb][v] = fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) * (gc[kb][v] - I);
-            }
-        } else {
-#pragma unroll
-            for (int kb = 0; kb < 2; kb++) {
-#pragma unroll
-                for (int v = 0; v < 4; v++) {
-                    const unsigned t = (unsigned)(tb + 16 * kb + v);
-                    const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
-                    gc[kb][v] = p * (gc[kb][v] - I);
+                for (int s = 0; s < NS; s++) {
+                    sc[kb] = M::mfma(h16_read_row<PITCH>(kblk[kb], s, c, qd), qop[s], sc[kb]);
+                    gc[kb] = M::mfma(h16_read_row<PITCH>(vblk[kb], s, c, qd), gop[s], gc[kb]);
                 }
             }
-        }
-        const uint4 dop = make_uint4(M::pack2(gc[0][0], gc[0][1]), M::pack2(gc[0][2], gc[0][3]), M::pack2(gc[1][0], gc[1][1]), M::pack2(gc[1][2], gc[1][3]));
+            const int tb = pos + 4 * qd - c;
+            if (pos >= HQ - 1 && pos + HK <= len) { // every element of the step is a neighbor: no band mask
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++) acc[cb] = M::mfma(h16_read_transposed<PITCH>(Ks, cb, c, qd), dop, acc[cb]);
-
-        __syncthreads();
-        if (more) {
-            kt.commit(Ks, lane);
-            vt.commit(Vs, lane);
+                for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) gc[kb][v] = fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) * (gc[kb][v] - I);
+                }
+            } else {
+#pragma unroll
+                for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                    for (int v = 0; v < 4; v++) {
+                        const unsigned t = (unsigned)(tb + 16 * kb + v);
+                        const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
+                        gc[kb][v] = p * (gc[kb][v] - I);
+                    }
+                }
+            }
+            const uint4 dop = make_uint4(M::pack2(gc[0][0], gc[0][1]), M::pack2(gc[0][2], gc[0][3]), M::pack2(gc[1][0], gc[1][1]), M::pack2(gc[1][2], gc[1][3]));
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[cb] = M::mfma(h16_read_transposed<PITCH>(kblk[0], kblk[1], cb, c, qd), dop, acc[cb]);
+        }
+        if (wk.more) {
+            if (wk.fresh) {
+                __syncthreads(); // the next run's rows replace rows the slowest wavefront may still be reading
+                bd.template commit<FRESH>(Ks, Vs, tid, 0);
+            } else {
+                bd.template commit<HK>(Ks, Vs, tid, FRESH - HK + wk.npos);
+            }
         }
         __syncthreads();
-        ri = nri;
-        pos = npos;
-        run = nrun;
+        wk.advance();
     }
 
     // (stored after the walk: a global store ahead of the loop would turn the loop's scalar loads of runs and weights,
@@ -462,15 +567,14 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dq_
 // The wavefront owns 16 INPUT longitudes (column c = key) and walks the runs grouped by input latitude; staged rows
 // are queries.  Staged row r of a run (first row = longitude w0 - ws - len + 1) sees key c iff 0 <= r - c < len.
 // Four products per step:  S = Q K^T,  G = dY V^T  (rows = queries, columns = keys),  dV^T += dY^T P,  dK^T += Q^T dS.
-template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dkdv_h16_kernel(const Args a)
+template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) void dkdv_h16_kernel(const Args a)
 {
-    typedef HTile<D> Tile;
+    typedef WgBand<D> Tile;
     typedef H16<T> M;
     constexpr int PITCH = Tile::PITCH, NS = D / 32, NCB = D / 16;
-    __shared__ __attribute__((aligned(16))) char Qs[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) char Gs[HK * PITCH];
-    __shared__ __attribute__((aligned(16))) float Ls[HK];
-    __shared__ __attribute__((aligned(16))) float Is[HK];
+    extern __shared__ __attribute__((aligned(16))) char h16_lds[];
+    char *Qs = h16_lds, *Gs = h16_lds + Tile::BYTES;
+    constexpr int STAT = 2 * D; // byte offset, in a row of Qs, of (lse, I = <dy, y>) of the staged query
 
     S2_H16_IDS(a.Wi, a.Hi)
     const int hi = a.sorder[a.row_first + rowsel];
@@ -500,97 +604,92 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64) void dkd
     }
     const float lw = fast_log2(a.quad_w[hi / a.kps]);
 
-    int ri = a.soff[hi];
-    const int rend = a.soff[hi + 1];
-    int pos = 0;
-    Run run = {0, 0, 0, 0};
-    Tile qt, gt;
+    H16Walk wk;
+    wk.ri = a.soff[hi];
+    wk.rend = a.soff[hi + 1];
+    wk.pos = 0;
+    wk.run = Run{0, 0, 0, 0};
+    Tile bd;
     float2 st = make_float2(0.f, 0.f);
     const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
-    const unsigned lane_off = (unsigned)(lane / Tile::CPR) * ldbq + 16u * (lane % Tile::CPR);
-    const bool piece_ok = 8 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int p) {
-        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
-        c0 += (c0 < 0) ? a.Wo : 0;
-        unsigned off[Tile::NIT];
-        Tile::offsets(off, lane_off, lane, c0, a.Wo, ldbq);
+    const bool piece_ok = 8 * (tid % Tile::CPR) < dr; // this thread's 16-byte piece of a staged row exists
+    auto fetch = [&](const Run &rn, int x0) {
+        int cbase = (wg0 - rn.ws - rn.len + 1) % a.Wo; // longitude of band row 0
+        cbase += (cbase < 0) ? a.Wo : 0;
         const size_t lat_off = (size_t)query_row(a, rn.lat, rn.pad) * ldb;
-        qt.fetch_if(qy + lat_off, off, piece_ok);
-        gt.fetch_if(gy + lat_off, off, piece_ok);
-        int col = c0 + lane; // lanes 0..31 fetch the statistics of the staged rows
-        col -= (col >= a.Wo) ? a.Wo : 0;
-        if (lane < HK) st = stats[(size_t)rn.lat * a.Wo + col];
-    };
-    auto commit = [&]() {
-        qt.commit(Qs, lane);
-        gt.commit(Gs, lane);
-        if (lane < HK) {
-            Ls[lane] = st.x;
-            Is[lane] = st.y;
+        if (x0 == 0)
+            bd.template fetch<FRESH, PAD>(qy + lat_off, gy + lat_off, tid, cbase, 0, a.Wo, ldbq, piece_ok);
+        else
+            bd.template fetch<HK, PAD>(qy + lat_off, gy + lat_off, tid, cbase, x0, a.Wo, ldbq, piece_ok);
+        if (tid < (x0 == 0 ? FRESH : HK)) { // the first threads fetch the statistics of the staged rows
+            int col = (cbase + x0) % a.Wo + tid;
+            while (col >= a.Wo) col -= a.Wo;
+            st = stats[(size_t)rn.lat * a.Wo + col];
         }
     };
-    if (ri < rend) {
-        run = a.sruns[ri];
-        fetch(run, 0);
-        commit();
+    auto commit = [&](int x0) {
+        if (x0 == 0)
+            bd.template commit<FRESH>(Qs, Gs, tid, 0);
+        else
+            bd.template commit<HK>(Qs, Gs, tid, x0);
+        if (tid < (x0 == 0 ? FRESH : HK)) *reinterpret_cast<float2 *>(Qs + ((x0 + tid) & (BR - 1)) * PITCH + STAT) = st;
+    };
+    if (wk.ri < wk.rend) {
+        wk.run = a.sruns[wk.ri];
+        fetch(wk.run, 0);
+        commit(0);
     }
     __syncthreads();
     settle(kop);
     settle(vop);
 
-    while (ri < rend) {
-        const int len = run.len;
-        int nri = ri, npos = pos + HK;
-        Run nrun = run;
-        if (npos >= len + HQ - 1) {
-            nri++;
-            npos = 0;
-            if (nri < rend) nrun = a.sruns[nri];
-        }
-        const bool more = nri < rend;
-        if (more) fetch(nrun, npos);
-
-        f4v sc[2], gc[2];
+    while (wk.ri < wk.rend) {
+        wk.plan(a.sruns);
+        if (wk.more) fetch(wk.nrun, wk.fresh ? 0 : FRESH - HK + wk.npos);
+        if (active) {
+            const int len = wk.run.len, pos = wk.pos;
+            const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
+            const char *qblk[2] = {band_block<PITCH>(Qs, xw), band_block<PITCH>(Qs, xw + 16)};
+            const char *gblk[2] = {band_block<PITCH>(Gs, xw), band_block<PITCH>(Gs, xw + 16)};
+            f4v sc[2], gc[2];
 #pragma unroll
-        for (int qb = 0; qb < 2; qb++) {
-            sc[qb] = f4v{0.f, 0.f, 0.f, 0.f};
-            gc[qb] = f4v{0.f, 0.f, 0.f, 0.f};
+            for (int qb = 0; qb < 2; qb++) {
+                sc[qb] = f4v{0.f, 0.f, 0.f, 0.f};
+                gc[qb] = f4v{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int s = 0; s < NS; s++) {
-                sc[qb] = M::mfma(h16_read_row<PITCH>(Qs, qb, s, c, qd), kop[s], sc[qb]);
-                gc[qb] = M::mfma(h16_read_row<PITCH>(Gs, qb, s, c, qd), vop[s], gc[qb]);
+                for (int s = 0; s < NS; s++) {
+                    sc[qb] = M::mfma(h16_read_row<PITCH>(qblk[qb], s, c, qd), kop[s], sc[qb]);
+                    gc[qb] = M::mfma(h16_read_row<PITCH>(gblk[qb], s, c, qd), vop[s], gc[qb]);
+                }
+            }
+            const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
+            const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
+#pragma unroll
+            for (int qb = 0; qb < 2; qb++) {
+                const char *sp = qblk[qb] + 4 * qd * PITCH + STAT;
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const float2 li = *reinterpret_cast<const float2 *>(sp + v * PITCH);
+                    float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - li.x));
+                    if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
+                    sc[qb][v] = p;
+                    gc[qb][v] = p * (gc[qb][v] - li.y);
+                }
+            }
+            const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
+            const uint4 dop = make_uint4(M::pack2(gc[0][0], gc[0][1]), M::pack2(gc[0][2], gc[0][3]), M::pack2(gc[1][0], gc[1][1]), M::pack2(gc[1][2], gc[1][3]));
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) {
+                dvt[cb] = M::mfma(h16_read_transposed<PITCH>(gblk[0], gblk[1], cb, c, qd), pop, dvt[cb]);
+                dkt[cb] = M::mfma(h16_read_transposed<PITCH>(qblk[0], qblk[1], cb, c, qd), dop, dkt[cb]);
             }
         }
-        const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
-        const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
-#pragma unroll
-        for (int qb = 0; qb < 2; qb++) {
-            const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 16 * qb + 4 * qd);
-            const float4 i4 = *reinterpret_cast<const float4 *>(Is + 16 * qb + 4 * qd);
-            const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
-            const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
-#pragma unroll
-            for (int v = 0; v < 4; v++) {
-                float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v]));
-                if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
-                sc[qb][v] = p;
-                gc[qb][v] = p * (gc[qb][v] - iv[v]);
-            }
+        if (wk.more) {
+            if (wk.fresh) __syncthreads(); // the next run's rows replace rows the slowest wavefront may still be reading
+            commit(wk.fresh ? 0 : FRESH - HK + wk.npos);
         }
-        const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
-        const uint4 dop = make_uint4(M::pack2(gc[0][0], gc[0][1]), M::pack2(gc[0][2], gc[0][3]), M::pack2(gc[1][0], gc[1][1]), M::pack2(gc[1][2], gc[1][3]));
-#pragma unroll
-        for (int cb = 0; cb < NCB; cb++) {
-            dvt[cb] = M::mfma(h16_read_transposed<PITCH>(Gs, cb, c, qd), pop, dvt[cb]);
-            dkt[cb] = M::mfma(h16_read_transposed<PITCH>(Qs, cb, c, qd), dop, dkt[cb]);
-        }
-
         __syncthreads();
-        if (more) commit();
-        __syncthreads();
-        ri = nri;
-        pos = npos;
-        run = nrun;
+        wk.advance();
     }
 
     if (mine) {

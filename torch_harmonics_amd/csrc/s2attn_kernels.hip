@@ -2199,18 +2199,23 @@ template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a
         a.row_first = 0;
         void (*kern)(const Args) = nullptr;
         long nblocks = 0;
+        const int lds = h16_lds_bytes<D>();
         if (which == FWD) {
             kern = fwd_h16_kernel<T, D, PAD>;
-            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+            nblocks = (long)a.Ho * ((a.Wo + WQ - 1) / WQ) * a.B * a.nh;
         } else if (which == DQ) {
             kern = dq_h16_kernel<T, D, PAD>;
-            nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+            nblocks = (long)a.Ho * ((a.Wo + WQ - 1) / WQ) * a.B * a.nh;
         } else {
             kern = dkdv_h16_kernel<T, D, PAD>;
-            nblocks = (long)a.Hi * ((a.Wi + HQ - 1) / HQ) * a.B * a.nh;
+            nblocks = (long)a.Hi * ((a.Wi + WQ - 1) / WQ) * a.B * a.nh;
         }
         if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+        if (lds > 48 * 1024) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, lds);
+            if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+        }
+        hipLaunchKernelGGL(kern, dim3((unsigned)nblocks), dim3(64 * NW), lds, stream, a);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
         return S2ATTN_OK;
