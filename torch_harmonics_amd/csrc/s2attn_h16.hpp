@@ -128,13 +128,12 @@ template <int D> struct WgBand {
     static constexpr int BYTES = BR * PITCH;            // one tensor's ring
     u4v ra[NIT], rb[NIT];
 
-    // cbase: longitude of band row 0 on the circle of W columns (0 <= cbase < W); ldc: bytes between two columns.
+    // cs: longitude of the first of the N rows on the circle of W columns (0 <= cs < W); ldc: bytes between two columns.
     // N (FRESH or HK) is the number of rows; iterations and row tests that N rules out are not compiled.
-    template <int N, bool PAD> __device__ inline void fetch(const char *pa, const char *pb, int tid, int cbase, int x0, int W, unsigned ldc, bool piece_ok)
+    template <int N, bool PAD> __device__ inline void fetch(const char *pa, const char *pb, int tid, int cs, int W, unsigned ldc, bool piece_ok)
     {
         const int r0 = tid / CPR;
         const unsigned pc = 16u * (tid % CPR);
-        int cs = (cbase + x0) % W;
 #pragma unroll
         for (int it = 0; it < (N + RPI - 1) / RPI; it++) {
             if (PAD) { // a thread may own a piece beyond the end of the row (a head narrower than the tile): it stages zeros
@@ -270,6 +269,15 @@ struct H16Walk {
     int nri, npos;
     Run nrun;
     bool more, fresh;
+    int cnext; // longitude of the first band row, of the run staged last, that is not staged yet
+    // first longitude to stage for the next step: c0 = longitude of band row 0 if that step starts a run (0 <= c0 < 2 W)
+    __device__ inline int stage(bool fresh_, int c0, int W)
+    {
+        int cs = fresh_ ? c0 : cnext;
+        while (cs >= W) cs -= W;
+        cnext = cs + (fresh_ ? FRESH : HK);
+        return cs;
+    }
     __device__ inline void plan(const Run *runs)
     {
         nri = ri;
@@ -327,16 +335,17 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     Tile bd;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
     const bool piece_ok = 8 * (tid % Tile::CPR) < dr; // this thread's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int x0) {
+    auto fetch = [&](const Run &rn, bool fresh) {
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        if (x0 == 0)
-            bd.template fetch<FRESH, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, 0, a.Wi, ldbk, piece_ok);
+        const int cs = wk.stage(fresh, rn.ws + wg0, a.Wi);
+        if (fresh)
+            bd.template fetch<FRESH, PAD>(kx + lat_off, vx + lat_off, tid, cs, a.Wi, ldbk, piece_ok);
         else
-            bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, x0, a.Wi, ldbk, piece_ok);
+            bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, cs, a.Wi, ldbk, piece_ok);
     };
     if (wk.ri < wk.rend) {
         wk.run = a.gruns[wk.ri];
-        fetch(wk.run, 0);
+        fetch(wk.run, true);
         bd.template commit<FRESH>(Ks, Vs, tid, 0);
     }
     __syncthreads();
@@ -344,7 +353,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 
     while (wk.ri < wk.rend) {
         wk.plan(a.gruns);
-        if (wk.more) fetch(wk.nrun, wk.fresh ? 0 : FRESH - HK + wk.npos);
+        if (wk.more) fetch(wk.nrun, wk.fresh);
         if (active) {
             const float lw = fast_log2(uniform_load(a.quad_w + wk.run.pad));
             const int len = wk.run.len, pos = wk.pos;
@@ -378,16 +387,19 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
                     }
                 }
             }
-            mx = h16_quarter_max(mx);
-            const float mn = fmaxf(m, fmaf(mx, LOG2E, lw)); // m starts finite, so mn is finite
-            if (__any(mn > m)) {
+            // The running maximum is only the reference point of the exponentials: it moves when a column's maximum has
+            // grown by more than RESCALE_THR (probabilities stay below 2^RESCALE_THR), which after a row's first steps is
+            // rare; until then the step needs no exchange between the four lanes of a column and no rescaling.
+            if (__any(fmaf(mx, LOG2E, lw) > m + RESCALE_THR)) {
+                const float cm = fmaf(h16_quarter_max(mx), LOG2E, lw);
+                const float mn = (cm > m + RESCALE_THR) ? cm : m; // m starts finite, so mn is finite
                 const float corr = fast_exp2(m - mn);
                 S *= corr;
 #pragma unroll
                 for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
+                m = mn;
             }
-            m = mn;
-            const float sh = lw - mn;
+            const float sh = lw - m;
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
@@ -479,16 +491,17 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     Tile bd;
     const unsigned ldbk = ldb * a.kps; // bytes between two columns of a virtual input latitude
     const bool piece_ok = 8 * (tid % Tile::CPR) < dr; // this thread's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int x0) {
+    auto fetch = [&](const Run &rn, bool fresh) {
         const size_t lat_off = (size_t)key_row(a, rn.lat, rn.pad) * ldb;
-        if (x0 == 0)
-            bd.template fetch<FRESH, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, 0, a.Wi, ldbk, piece_ok);
+        const int cs = wk.stage(fresh, rn.ws + wg0, a.Wi);
+        if (fresh)
+            bd.template fetch<FRESH, PAD>(kx + lat_off, vx + lat_off, tid, cs, a.Wi, ldbk, piece_ok);
         else
-            bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, (rn.ws + wg0) % a.Wi, x0, a.Wi, ldbk, piece_ok);
+            bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, cs, a.Wi, ldbk, piece_ok);
     };
     if (wk.ri < wk.rend) {
         wk.run = a.gruns[wk.ri];
-        fetch(wk.run, 0);
+        fetch(wk.run, true);
         bd.template commit<FRESH>(Ks, Vs, tid, 0);
     }
     __syncthreads();
@@ -499,7 +512,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 
     while (wk.ri < wk.rend) {
         wk.plan(a.gruns);
-        if (wk.more) fetch(wk.nrun, wk.fresh ? 0 : FRESH - HK + wk.npos);
+        if (wk.more) fetch(wk.nrun, wk.fresh);
         if (active) {
             const float lwl = fast_log2(uniform_load(a.quad_w + wk.run.pad)) - lse_;
             const int len = wk.run.len, pos = wk.pos;
@@ -613,16 +626,20 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     float2 st = make_float2(0.f, 0.f);
     const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
     const bool piece_ok = 8 * (tid % Tile::CPR) < dr; // this thread's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int x0) {
-        int cbase = (wg0 - rn.ws - rn.len + 1) % a.Wo; // longitude of band row 0
-        cbase += (cbase < 0) ? a.Wo : 0;
+    auto fetch = [&](const Run &rn, bool fresh) {
+        int c0 = 0;
+        if (fresh) { // longitude of band row 0, in [0, 2 W)
+            c0 = wg0 - rn.ws - rn.len + 1 + a.Wo;
+            while (c0 < 0) c0 += a.Wo;
+        }
+        const int cs = wk.stage(fresh, c0, a.Wo);
         const size_t lat_off = (size_t)query_row(a, rn.lat, rn.pad) * ldb;
-        if (x0 == 0)
-            bd.template fetch<FRESH, PAD>(qy + lat_off, gy + lat_off, tid, cbase, 0, a.Wo, ldbq, piece_ok);
+        if (fresh)
+            bd.template fetch<FRESH, PAD>(qy + lat_off, gy + lat_off, tid, cs, a.Wo, ldbq, piece_ok);
         else
-            bd.template fetch<HK, PAD>(qy + lat_off, gy + lat_off, tid, cbase, x0, a.Wo, ldbq, piece_ok);
-        if (tid < (x0 == 0 ? FRESH : HK)) { // the first threads fetch the statistics of the staged rows
-            int col = (cbase + x0) % a.Wo + tid;
+            bd.template fetch<HK, PAD>(qy + lat_off, gy + lat_off, tid, cs, a.Wo, ldbq, piece_ok);
+        if (tid < (fresh ? FRESH : HK)) { // the first threads fetch the statistics of the staged rows
+            int col = cs + tid;
             while (col >= a.Wo) col -= a.Wo;
             st = stats[(size_t)rn.lat * a.Wo + col];
         }
@@ -636,7 +653,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     };
     if (wk.ri < wk.rend) {
         wk.run = a.sruns[wk.ri];
-        fetch(wk.run, 0);
+        fetch(wk.run, true);
         commit(0);
     }
     __syncthreads();
@@ -645,7 +662,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 
     while (wk.ri < wk.rend) {
         wk.plan(a.sruns);
-        if (wk.more) fetch(wk.nrun, wk.fresh ? 0 : FRESH - HK + wk.npos);
+        if (wk.more) fetch(wk.nrun, wk.fresh);
         if (active) {
             const int len = wk.run.len, pos = wk.pos;
             const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
