@@ -266,8 +266,10 @@ __device__ inline Run uniform_load(const Run *p)
 struct H16Walk {
     int ri, rend, pos;
     Run run;
+    float w; // quadrature weight of the run's input latitude (gather side), read together with the run: a step before its use
     int nri, npos;
     Run nrun;
+    float nw;
     bool more, fresh;
     int cnext; // longitude of the first band row, of the run staged last, that is not staged yet
     // first longitude to stage for the next step: c0 = longitude of band row 0 if that step starts a run (0 <= c0 < 2 W)
@@ -278,15 +280,19 @@ struct H16Walk {
         cnext = cs + (fresh_ ? FRESH : HK);
         return cs;
     }
-    __device__ inline void plan(const Run *runs)
+    __device__ inline void plan(const Run *runs, const float *weights = nullptr)
     {
         nri = ri;
         npos = pos + HK;
         nrun = run;
+        nw = w;
         if (npos >= run.len + HQ - 1) {
             nri++;
             npos = 0;
-            if (nri < rend) nrun = uniform_load(runs + nri);
+            if (nri < rend) {
+                nrun = uniform_load(runs + nri);
+                if (weights) nw = uniform_load(weights + nrun.pad);
+            }
         }
         more = nri < rend;
         fresh = npos == 0;
@@ -296,6 +302,7 @@ struct H16Walk {
         ri = nri;
         pos = npos;
         run = nrun;
+        w = nw;
     }
 };
 
@@ -343,8 +350,10 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
         else
             bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, cs, a.Wi, ldbk, piece_ok);
     };
+    wk.w = 1.f;
     if (wk.ri < wk.rend) {
         wk.run = a.gruns[wk.ri];
+        wk.w = a.quad_w[wk.run.pad];
         fetch(wk.run, true);
         bd.template commit<FRESH>(Ks, Vs, tid, 0);
     }
@@ -352,10 +361,10 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     settle(qop);
 
     while (wk.ri < wk.rend) {
-        wk.plan(a.gruns);
+        wk.plan(a.gruns, a.quad_w);
         if (wk.more) fetch(wk.nrun, wk.fresh);
         if (active) {
-            const float lw = fast_log2(uniform_load(a.quad_w + wk.run.pad));
+            const float lw = fast_log2(wk.w);
             const int len = wk.run.len, pos = wk.pos;
             const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
             const char *kblk[2] = {band_block<PITCH>(Ks, xw), band_block<PITCH>(Ks, xw + 16)};
@@ -499,8 +508,10 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
         else
             bd.template fetch<HK, PAD>(kx + lat_off, vx + lat_off, tid, cs, a.Wi, ldbk, piece_ok);
     };
+    wk.w = 1.f;
     if (wk.ri < wk.rend) {
         wk.run = a.gruns[wk.ri];
+        wk.w = a.quad_w[wk.run.pad];
         fetch(wk.run, true);
         bd.template commit<FRESH>(Ks, Vs, tid, 0);
     }
@@ -511,10 +522,10 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     settle(lse_);
 
     while (wk.ri < wk.rend) {
-        wk.plan(a.gruns);
+        wk.plan(a.gruns, a.quad_w);
         if (wk.more) fetch(wk.nrun, wk.fresh);
         if (active) {
-            const float lwl = fast_log2(uniform_load(a.quad_w + wk.run.pad)) - lse_;
+            const float lwl = fast_log2(wk.w) - lse_;
             const int len = wk.run.len, pos = wk.pos;
             const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
             const char *kblk[2] = {band_block<PITCH>(Ks, xw), band_block<PITCH>(Ks, xw + 16)};
@@ -622,6 +633,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     wk.rend = a.soff[hi + 1];
     wk.pos = 0;
     wk.run = Run{0, 0, 0, 0};
+    wk.w = 1.f;
     Tile bd;
     float2 st = make_float2(0.f, 0.f);
     const unsigned ldbq = ldb * a.qps; // bytes between two columns of a virtual output latitude
