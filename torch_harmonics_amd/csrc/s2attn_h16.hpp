@@ -598,7 +598,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
     constexpr int PITCH = Tile::PITCH, NS = D / 32, NCB = D / 16;
     extern __shared__ __attribute__((aligned(16))) char h16_lds[];
     char *Qs = h16_lds, *Gs = h16_lds + Tile::BYTES;
-    constexpr int STAT = 2 * D; // byte offset, in a row of Qs, of (lse, I = <dy, y>) of the staged query
+    constexpr int STAT = 2 * D; // the 32 bytes of padding of ring row 4 j of Qs hold (lse, I = <dy, y>) of the queries staged in rows 4 j .. 4 j + 3
 
     S2_H16_IDS(a.Wi, a.Hi)
     const int hi = a.sorder[a.row_first + rowsel];
@@ -661,7 +661,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
             bd.template commit<FRESH>(Qs, Gs, tid, 0);
         else
             bd.template commit<HK>(Qs, Gs, tid, x0);
-        if (tid < (x0 == 0 ? FRESH : HK)) *reinterpret_cast<float2 *>(Qs + ((x0 + tid) & (BR - 1)) * PITCH + STAT) = st;
+        if (tid < (x0 == 0 ? FRESH : HK)) *reinterpret_cast<float2 *>(Qs + ((x0 + tid) & (BR - 4)) * PITCH + STAT + 8 * (tid & 3)) = st;
     };
     if (wk.ri < wk.rend) {
         wk.run = a.sruns[wk.ri];
@@ -695,14 +695,16 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
             const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
 #pragma unroll
             for (int qb = 0; qb < 2; qb++) {
-                const char *sp = qblk[qb] + 4 * qd * PITCH + STAT;
+                const float4 *sp = reinterpret_cast<const float4 *>(qblk[qb] + 4 * qd * PITCH + STAT);
+                const float4 s01 = sp[0], s23 = sp[1];
+                const float lv[4] = {s01.x, s01.z, s23.x, s23.z};
+                const float iv[4] = {s01.y, s01.w, s23.y, s23.w};
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    const float2 li = *reinterpret_cast<const float2 *>(sp + v * PITCH);
-                    float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - li.x));
+                    float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v]));
                     if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
                     sc[qb][v] = p;
-                    gc[qb][v] = p * (gc[qb][v] - li.y);
+                    gc[qb][v] = p * (gc[qb][v] - iv[v]);
                 }
             }
             const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
