@@ -15,6 +15,17 @@ RING_CASES = [
 ]
 
 
+# gather direction on grids with at least 32 global output longitudes: with fp32 storage and ck == cv a multiple of 4 from 16 to
+# 128 the forward step runs on the band-staged matrix-core kernel (s2attn_ring_forward_step_plan)
+RING_BAND_CASES = [
+    ((9, 48), (9, 48), "equiangular", "equiangular", 0.5, (0, 9, 7, 30), [0, 10, 11, 37, 48]),  # self-attention, a one-column chunk, pole rows see whole circles
+    ((8, 96), (6, 48), "equiangular", "legendre-gauss", 0.6, (1, 4, 9, 33), [0, 40, 96]),  # longitude ratio 2, ragged last tile
+    ((7, 120), (5, 40), "legendre-gauss", "equiangular", 0.7, (0, 5, 0, 40), [0, 31, 32, 90, 120]),  # ratio 3, the whole output grid is local
+    ((6, 40), (6, 40), "equiangular", "equiangular", 7.0, (1, 3, 35, 5), [0, 20, 40]),  # every point sees every point, a window of five columns
+    ((12, 80), (12, 80), "legendre-gauss", "legendre-gauss", 0.2, (0, 12, 16, 64), [0, 20, 40, 60, 80]),  # short runs only: most tiles touch one chunk
+]
+
+
 def local_problem(case, batch=2, ck=5, cv=3, seed=0, tight_halo=True):
     """Global tensors plus the local CSR / window / halo of one rank.  Returns a dict."""
     ins, outs, gi, go, tc, (lat_lo, nlat_loc, lon_lo, nlon_loc), bounds = case

@@ -16,7 +16,7 @@ LIB_PATH = os.path.join(_HERE, "libs2attn.so")
 TORCH_LIB_PATH = os.path.join(_HERE, "_C.so")  # libtorch registration of the operators (csrc/s2attn_torch.cpp)
 
 S2ATTN_F32, S2ATTN_BF16, S2ATTN_F16 = 0, 1, 2
-ABI_VERSION = 11
+ABI_VERSION = 12
 NOALLOC_SCRATCH_BYTES = 64 * 1024 * 1024
 
 _vp = ctypes.c_void_p
@@ -107,6 +107,7 @@ SYMBOLS = {
     "s2attn_permute_to_nhwc": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "s2attn_permute_to_nchw": (_int, [_vp, _vp, _i64, _i64, _i64, _i64, _int, _vp]),
     "s2attn_ring_forward_step": (_int, [_vp] * 10 + [ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_forward_step_plan": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_regroup_psi": (_i64, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),

@@ -58,7 +58,7 @@ int s2attn_fail(int code, const char *fmt, ...)
 }
 
 extern "C" const char *s2attn_last_error(void) { return g_err; }
-extern "C" int s2attn_abi_version(void) { return 11; }
+extern "C" int s2attn_abi_version(void) { return 12; }
 #endif
 
 namespace s2 {
@@ -294,6 +294,10 @@ struct Args {
     int qps; // nlon_out / nlon_in when the output grid is the finer one, else 1; see query_point()
     int tile_rows; // LDS rows per staged band
     int row_first; // first entry of gorder / sorder this launch covers (dense rows come first, see s2attn_plan_split)
+    // one ring step of the forward (ring_fwd_m32_kernel): the chunk's first real input longitude and latitude, its extents,
+    // and the caller's running state
+    int r_lon_lo, r_nkx, r_lat0, r_nlat;
+    float *r_yacc, *r_asum, *r_qmax;
 };
 
 // Key-side addressing.  With nlon_in = kps * nlon_out, query column wo sees input columns ws + t + kps * wo: on the
@@ -2186,6 +2190,7 @@ enum Which { FWD, DQ, DKDV };
 
 template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream);
 template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream);
+template <int D> int launch_ring_fwd_m32(const Args &a0, hipStream_t stream);
 
 #if S2_PART == 0 || S2_PART == 2
 // 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
@@ -2268,7 +2273,24 @@ template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t
     return S2ATTN_OK;
 }
 #endif
+#if S2_PART == 0 || S2_PART == 3
+// one ring step of the forward on the fp32 16-longitude kernels: one wavefront per 16 local output longitudes
+template <int D> int launch_ring_fwd_m32(const Args &a0, hipStream_t stream)
+{
+    Args a = a0;
+    a.row_first = 0;
+    const long nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    hipLaunchKernelGGL(ring_fwd_m32_kernel<D>, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
+#endif
 #if S2_PART == 3
+template int launch_ring_fwd_m32<16>(const Args &, hipStream_t);
+template int launch_ring_fwd_m32<32>(const Args &, hipStream_t);
+template int launch_ring_fwd_m32<64>(const Args &, hipStream_t);
 template int launch_m32<16, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<32, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<64, 1>(Which, const Args &, hipStream_t);
@@ -2596,6 +2618,50 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     const size_t al = 4 * (size_t)esize(shape->dtype);
     const bool vec = shape->ck % 4 == 0 && shape->cv % 4 == 0 && aligned(k, al) && aligned(v, al) && aligned(q, al) && aligned(y, al);
     return launch(FWD, a, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
+}
+
+// One ring step of the forward on the band-staged kernels (see ring_fwd_m32_kernel).
+extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                                             const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
+{
+    if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "ring shape is null");
+    if (sh->batch < 1 || sh->nlat_halo < 1 || sh->nlon_kx < 1 || sh->nlat_out < 1 || sh->nlon_out < 1 || sh->nlon_in < 1)
+        return s2attn_fail(S2ATTN_E_INVALID, "batch and grid extents must be positive");
+    if (sh->pscale < 1 || sh->nlon_in % sh->pscale != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "pscale must be a positive divisor of nlon_in = %d, got %d", sh->nlon_in, sh->pscale);
+    if (sh->lon_lo_kx < 0 || sh->lon_lo_kx + sh->nlon_kx > sh->nlon_in)
+        return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", sh->lon_lo_kx, sh->lon_lo_kx + sh->nlon_kx, sh->nlon_in);
+    const int W = sh->nlon_in / sh->pscale; // global output longitudes = columns of a virtual input latitude
+    if (sh->nlon_out > W) return s2attn_fail(S2ATTN_E_INVALID, "pscale * nlon_out = %ld exceeds nlon_in = %d", (long)sh->pscale * sh->nlon_out, sh->nlon_in);
+    if (!k || !v || !q || !y_acc || !alpha_sum || !qdotk_max || !quad_weights) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!plan || !plan->data) return s2attn_fail(S2ATTN_E_INVALID, "plan is null");
+    const int32_t *h = plan->header;
+    if (h[S2ATTN_PH_MAGIC] != S2ATTN_PLAN_MAGIC) return s2attn_fail(S2ATTN_E_INVALID, "plan header does not carry this library's plan format");
+    if (h[S2ATTN_PH_NLON_IN] != sh->nlon_in || h[S2ATTN_PH_NLAT_OUT] != sh->nlat_out || h[S2ATTN_PH_NLON_OUT] != W)
+        return s2attn_fail(S2ATTN_E_INVALID, "plan was built for %d input longitudes and %dx%d output points, the step is for %d and %dx%d (global longitudes)",
+                           h[S2ATTN_PH_NLON_IN], h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], sh->nlon_in, sh->nlat_out, W);
+    if (sh->dtype != S2ATTN_F32 || !m32_width(sh->ck, sh->cv) || sh->ck > 64 || W < HK)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring step takes fp32 tensors with ck = cv a multiple of 4 from 16 to 64 and at least %d global output longitudes", HK);
+    const void *ptrs[] = {k, v, q, y_acc};
+    for (const void *p : ptrs)
+        if (!aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring step takes 16-byte aligned tensors");
+    Args a = {};
+    const int32_t *d = plan->data;
+    a.quad_w = quad_weights;
+    a.goff = d + h[S2ATTN_PH_GATHER_OFF];
+    a.gruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_GATHER_RUNS]);
+    a.gorder = d + h[S2ATTN_PH_GATHER_ORDER];
+    a.k = k, a.v = v, a.q = q;
+    a.B = sh->batch, a.nh = 1, a.kps = sh->pscale, a.qps = 1;
+    a.Hi = h[S2ATTN_PH_NLAT_IN] * sh->pscale, a.Wi = W;
+    a.Ho = sh->nlat_out, a.Wo = sh->nlon_out; // local output points; runs are relative to local column 0
+    a.dk_ = a.dv_ = sh->ck;
+    a.r_lon_lo = sh->lon_lo_kx, a.r_nkx = sh->nlon_kx, a.r_lat0 = sh->lat_halo_start, a.r_nlat = sh->nlat_halo;
+    a.r_yacc = y_acc, a.r_asum = alpha_sum, a.r_qmax = qdotk_max;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (sh->ck <= 16) return launch_ring_fwd_m32<16>(a, st);
+    if (sh->ck <= 32) return launch_ring_fwd_m32<32>(a, st);
+    return launch_ring_fwd_m32<64>(a, st);
 }
 
 namespace {

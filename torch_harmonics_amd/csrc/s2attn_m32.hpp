@@ -555,3 +555,193 @@ template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dkdv_m32_ker
         }
     }
 }
+
+// ---- forward, one ring step --------------------------------------------------------------------------------------
+// The forward above for ONE longitude chunk of K/V (input latitudes r_lat0 .. + r_nlat, real input longitudes
+// r_lon_lo .. + r_nkx; k, v = [batch, r_nlat, r_nkx, channels]) that continues a running softmax kept by the caller in the
+// reference's form: y_acc = sum_j alpha_j v_j, alpha_sum = sum_j alpha_j, qdotk_max = max_j q.k_j (natural units) with
+// alpha_j = exp(q.k_j - qdotk_max) w_j over the neighbors seen so far.  A row of the staged band is one input longitude, so
+// the chunk clips ROWS of the band, not queries: the band positions u of a run whose longitude (ws + w0 + u) mod W lies in
+// the chunk are up to three intervals, and the walk visits only the 32-position steps inside them (a chunk of a quarter of
+// the circle costs a polar tile a quarter of its steps, an equatorial tile one step per run in the one or two chunks its
+// neighborhood touches).  Tiles without any such step leave the state untouched.
+constexpr float NEG_BIG_NAT = -1.0e38f; // "no neighbor yet" for a maximum in natural units (times log2 e stays finite)
+
+struct RingWalk {
+    const Run *runs;
+    const float *weights;
+    int ri, rend;
+    int W, kps, w0, lon_lo, nkx, lat0, nlat;
+    // the run the walk stands in
+    Run run;
+    float w;
+    int rl, par, vlo, nv, u0, L, m;
+    // the step: band positions pos .. pos + HK of the interval [ua, ub); vca = virtual column of position ua
+    int pos, ua, ub, vca;
+    bool valid;
+    __device__ inline void start(const Run *runs_, const float *weights_, int first, int rend_)
+    {
+        runs = runs_, weights = weights_, ri = first - 1, rend = rend_, m = 1, valid = false;
+    }
+    __device__ inline bool advance()
+    {
+        if (valid && pos + HK < ub) {
+            pos += HK;
+            return true;
+        }
+        for (;;) {
+            m++;
+            if (m > 1) { // next run
+                ri++;
+                if (ri >= rend) return valid = false;
+                run = uniform_load(runs + ri);
+                rl = run.pad - lat0; // row of the chunk
+                m = 1;               // (skip the run unless the chunk holds part of it)
+                if (rl < 0 || rl >= nlat) continue;
+                par = run.lat - run.pad * kps; // column class: virtual column vc is real longitude vc * kps + par
+                vlo = (lon_lo - par + kps - 1) / kps;
+                nv = (lon_lo + nkx - par + kps - 1) / kps - vlo; // virtual columns vlo .. vlo + nv are in the chunk
+                if (nv <= 0) continue;
+                w = uniform_load(weights + run.pad);
+                L = run.len + HQ - 1;
+                u0 = (vlo - run.ws - w0) % W;
+                u0 += (u0 < 0) ? W : 0; // first band position at virtual column vlo
+                m = -2;
+                continue;
+            }
+            const int a0 = u0 + m * W;
+            const int a_ = a0 < 0 ? 0 : a0, b_ = a0 + nv > L ? L : a0 + nv;
+            if (a_ >= b_) continue;
+            ua = pos = a_, ub = b_, vca = vlo + (a_ - a0);
+            return valid = true;
+        }
+    }
+};
+
+template <int D> __global__ __launch_bounds__(64) void ring_fwd_m32_kernel(const Args a)
+{
+    constexpr int NS = 1;
+    typedef FTile<D> Tile;
+    constexpr int PITCH = Tile::PITCH, NCB = D / 16;
+    S2_M32_IDS(a.Wo, a.Ho)
+    (void)h; // heads are folded into the batch
+    char *lds = m32_lds<m32_lds_bytes<D, 1>(false), 1>();
+    char *Ks = lds, *Vs = Ks + HK * PITCH;
+    const int ho = a.gorder[a.row_first + rowsel];
+    const unsigned ldb = drt * 4; // bytes between two grid points
+    const char *kx = static_cast<const char *>(a.k) + (size_t)b * a.r_nlat * a.r_nkx * ldb;
+    const char *vx = static_cast<const char *>(a.v) + (size_t)b * a.r_nlat * a.r_nkx * ldb;
+    const bool mine = c < nvalid;
+    const size_t pt = ((size_t)b * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
+
+    RingWalk wk;
+    wk.W = a.Wi, wk.kps = a.kps, wk.w0 = w0, wk.lon_lo = a.r_lon_lo, wk.nkx = a.r_nkx, wk.lat0 = a.r_lat0, wk.nlat = a.r_nlat;
+    wk.start(a.gruns, a.quad_w, a.goff[ho], a.goff[ho + 1]);
+    if (!wk.advance()) return; // nothing of this tile's neighborhood is in the chunk
+
+    float qop[D / 4];
+    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb, qd, dr);
+    f4v acc[NCB]; // Y^T: register v of block cb is channel 16 cb + 4 qd + v of column c
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) {
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (16 * cb + 4 * qd < dr) x = *reinterpret_cast<const float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd);
+        acc[cb] = f4v{x.x, x.y, x.z, x.w};
+    }
+    float m = fmaxf(a.r_qmax[pt], NEG_BIG_NAT);
+    float S = qd == 0 ? a.r_asum[pt] : 0.f; // the four lanes of a column each keep a share of the sum
+
+    Tile kt, vt;
+    const int r0 = lane / Tile::CPR;
+    const unsigned pc = 16u * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
+    const unsigned colb = ldb * a.kps;                 // bytes between two virtual columns
+    auto fetch = [&]() { // the rows of the step the walk stands at; rows beyond the interval are staged as zeros
+        const size_t base = ((size_t)wk.rl * a.r_nkx + (size_t)((wk.vca + wk.pos - wk.ua) * a.kps + wk.par - a.r_lon_lo)) * ldb + pc;
+        const int nrows = wk.ub - wk.pos;
+#pragma unroll
+        for (int it = 0; it < Tile::NIT; it++) {
+            const int row = r0 + it * Tile::RPI;
+            kt.raw[it] = u4v{0u, 0u, 0u, 0u};
+            vt.raw[it] = u4v{0u, 0u, 0u, 0u};
+            if (row < nrows && piece_ok) {
+                kt.raw[it] = *reinterpret_cast<const u4v *>(kx + base + (size_t)row * colb);
+                vt.raw[it] = *reinterpret_cast<const u4v *>(vx + base + (size_t)row * colb);
+            }
+        }
+    };
+    fetch();
+    kt.commit(Ks, lane);
+    vt.commit(Vs, lane);
+    __syncthreads();
+    settle(qop);
+
+    for (;;) {
+        const float lw = fast_log2(wk.w);
+        const int len = wk.run.len, pos = wk.pos, ub = wk.ub;
+        const bool more = wk.advance();
+        if (more) fetch();
+
+        f4v sc[2];
+        m32_scores<D, PITCH>(sc, Ks, c, qd, qop);
+        // element (kb, v) is band position u = pos + 16 kb + 4 qd + v and neighbor t = u - c of column c: it counts iff
+        // 0 <= t < len and u < ub, i.e. t < min(len, ub - c) as unsigned numbers
+        const int tb = pos + 4 * qd - c;
+        const unsigned lim = (unsigned)max(0, min(len, ub - c));
+        float mx = -INFINITY;
+        if (pos >= HQ - 1 && pos + HK <= min(len, ub)) { // every element of the step counts
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) mx = fmaxf(mx, sc[kb][v]);
+            }
+        } else {
+#pragma unroll
+            for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+                for (int v = 0; v < 4; v++) {
+                    const unsigned t = (unsigned)(tb + 16 * kb + v);
+                    sc[kb][v] = (t < lim) ? sc[kb][v] : -INFINITY;
+                    mx = fmaxf(mx, sc[kb][v]);
+                }
+            }
+        }
+        mx = h16_quarter_max(mx);
+        const float mn = fmaxf(m, mx); // m is finite, so mn is
+        if (__any(mn > m)) {
+            const float corr = fast_exp2((m - mn) * LOG2E);
+            S *= corr;
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
+        }
+        m = mn;
+        const float sh = fmaf(-mn, LOG2E, lw);
+#pragma unroll
+        for (int kb = 0; kb < 2; kb++) {
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // = exp(q.k - max) w; not counted: exp2(-inf) = 0
+                sc[kb][v] = p;
+                S += p;
+            }
+        }
+        m32_accumulate<D, PITCH>(acc, Vs, c, qd, sc);
+
+        __syncthreads();
+        if (!more) break;
+        kt.commit(Ks, lane);
+        vt.commit(Vs, lane);
+        __syncthreads();
+    }
+
+    S = h16_quarter_sum(S);
+    if (mine) {
+        if (qd == 0) {
+            a.r_asum[pt] = S;
+            a.r_qmax[pt] = m <= 0.5f * NEG_BIG_NAT ? -INFINITY : m;
+        }
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++)
+            if (16 * cb + 4 * qd < dr) *reinterpret_cast<float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+    }
+}

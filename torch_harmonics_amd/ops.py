@@ -22,6 +22,7 @@ import torch
 
 from . import _lib
 from ._attention_utils import _setup_context_attention_backward
+from . import plan as _plan
 from .plan import get_row_order, get_transposed_csr
 
 _DTYPE_CODE = {torch.float32: _lib.S2ATTN_F32, torch.bfloat16: _lib.S2ATTN_BF16, torch.float16: _lib.S2ATTN_F16}
@@ -251,6 +252,14 @@ def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out
     return _lib.RingShapeStruct(B, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, vx.shape[3], nlon_in, pscale, lon_lo_kx, lat_halo_start, _DTYPE_CODE[qy.dtype])
 
 
+def _ring_takes_plan(kx, vx, qy, y_acc, nlon_in, pscale) -> bool:
+    """Shapes of the band-staged ring forward step (s2attn_ring_forward_step_plan in include/s2attn.h)."""
+    ck, cv = kx.shape[3], vx.shape[3]
+    if qy.dtype != torch.float32 or ck != cv or ck % 4 or not 16 <= ck <= 64 or nlon_in // pscale < 32:
+        return False
+    return all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, y_acc))
+
+
 def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out, nrows=None):
     """state: (name, tensor, trailing channel count or None) fp32 buffers shaped like the local output grid; nrows: rows of
     the CSR (output latitudes in the gather direction, the chunk's input latitudes in the scatter direction); row_idx only
@@ -309,6 +318,16 @@ def forward_ring_step(
     if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:  # nothing to fold in
         return
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    if _ring_takes_plan(kx, vx, qy, y_acc, nlon_in, pscale):
+        # band-staged matrix-core step on the run-length plan of the local psi (built on the host once per psi, cached)
+        p = _plan.get_plan(col_idx, row_off, quad_weights.numel(), nlon_in, nlat_out, nlon_in // pscale)
+        with torch.cuda.device(kx.device):
+            rc = _lib.load().s2attn_ring_forward_step_plan(
+                kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+                quad_weights.data_ptr(), ctypes.byref(p.struct), ctypes.byref(shape), _stream_ptr(kx.device),
+            )  # fmt: skip
+        _lib.check(rc, "s2attn_ring_forward_step_plan")
+        return
     with torch.cuda.device(kx.device):
         rc = _lib.load().s2attn_ring_forward_step(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
