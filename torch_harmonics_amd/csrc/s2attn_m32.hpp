@@ -598,13 +598,17 @@ struct RingWalk {
                 rl = run.pad - lat0; // row of the chunk
                 m = 1;               // (skip the run unless the chunk holds part of it)
                 if (rl < 0 || rl >= nlat) continue;
-                par = run.lat - run.pad * kps; // column class: virtual column vc is real longitude vc * kps + par
-                vlo = (lon_lo - par + kps - 1) / kps;
-                nv = (lon_lo + nkx - par + kps - 1) / kps - vlo; // virtual columns vlo .. vlo + nv are in the chunk
-                if (nv <= 0) continue;
+                par = 0, vlo = lon_lo, nv = nkx;
+                if (kps > 1) {
+                    par = run.lat - run.pad * kps; // column class: virtual column vc is real longitude vc * kps + par
+                    vlo = (lon_lo - par + kps - 1) / kps;
+                    nv = (lon_lo + nkx - par + kps - 1) / kps - vlo; // virtual columns vlo .. vlo + nv are in the chunk
+                    if (nv <= 0) continue;
+                }
                 w = uniform_load(weights + run.pad);
                 L = run.len + HQ - 1;
-                u0 = (vlo - run.ws - w0) % W;
+                u0 = vlo - run.ws - w0; // in (-2 W, W)
+                u0 += (u0 < 0) ? W : 0;
                 u0 += (u0 < 0) ? W : 0; // first band position at virtual column vlo
                 m = -2;
                 continue;
@@ -618,7 +622,7 @@ struct RingWalk {
     }
 };
 
-template <int D> __global__ __launch_bounds__(64) void ring_fwd_m32_kernel(const Args a)
+template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd_m32_kernel(const Args a)
 {
     constexpr int NS = 1;
     typedef FTile<D> Tile;
@@ -648,7 +652,11 @@ template <int D> __global__ __launch_bounds__(64) void ring_fwd_m32_kernel(const
         if (16 * cb + 4 * qd < dr) x = *reinterpret_cast<const float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd);
         acc[cb] = f4v{x.x, x.y, x.z, x.w};
     }
-    float m = fmaxf(a.r_qmax[pt], NEG_BIG_NAT);
+    // The exponentials are taken relative to a reference point m that is moved lazily (when a column's maximum has grown by
+    // more than RESCALE_THR binary orders: after a tile's first steps that is rare, and a step then needs neither an exchange
+    // between the four lanes of a column nor a rescaling); the exact maximum the state asks for is kept per lane (mtrue)
+    // and the sums are brought to it once, at the end.
+    float m = fmaxf(a.r_qmax[pt], NEG_BIG_NAT), mtrue = -INFINITY;
     float S = qd == 0 ? a.r_asum[pt] : 0.f; // the four lanes of a column each keep a share of the sum
 
     Tile kt, vt;
@@ -706,16 +714,18 @@ template <int D> __global__ __launch_bounds__(64) void ring_fwd_m32_kernel(const
                 }
             }
         }
-        mx = h16_quarter_max(mx);
-        const float mn = fmaxf(m, mx); // m is finite, so mn is
-        if (__any(mn > m)) {
+        mtrue = fmaxf(mtrue, mx);
+        constexpr float THR = RESCALE_THR * 0.69314718f; // natural units
+        if (__any(mx > m + THR)) {
+            const float cm = h16_quarter_max(mx);
+            const float mn = cm > m + THR ? cm : m; // m is finite, so mn is
             const float corr = fast_exp2((m - mn) * LOG2E);
             S *= corr;
 #pragma unroll
             for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
+            m = mn;
         }
-        m = mn;
-        const float sh = fmaf(-mn, LOG2E, lw);
+        const float sh = fmaf(-m, LOG2E, lw);
 #pragma unroll
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
@@ -735,13 +745,16 @@ template <int D> __global__ __launch_bounds__(64) void ring_fwd_m32_kernel(const
     }
 
     S = h16_quarter_sum(S);
+    mtrue = fmaxf(h16_quarter_max(mtrue), a.r_qmax[pt]); // the maximum over everything this column has seen, earlier chunks included (read again: a register less in the loop)
+    const float f = mtrue > -INFINITY ? fast_exp2((m - mtrue) * LOG2E) : 1.f; // m <= mtrue <= m + THR; a column without neighbors keeps its zeros
     if (mine) {
         if (qd == 0) {
-            a.r_asum[pt] = S;
-            a.r_qmax[pt] = m <= 0.5f * NEG_BIG_NAT ? -INFINITY : m;
+            a.r_asum[pt] = S * f;
+            a.r_qmax[pt] = mtrue;
         }
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++)
-            if (16 * cb + 4 * qd < dr) *reinterpret_cast<float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd) = make_float4(acc[cb][0], acc[cb][1], acc[cb][2], acc[cb][3]);
+            if (16 * cb + 4 * qd < dr)
+                *reinterpret_cast<float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd) = make_float4(acc[cb][0] * f, acc[cb][1] * f, acc[cb][2] * f, acc[cb][3] * f);
     }
 }
