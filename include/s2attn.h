@@ -83,6 +83,9 @@ int s2attn_abi_version(void);
  *     *_pair_off [npairs+1], *_pair_runs [8 * ...]   merged runs of each pair: (lat, ws, len, aux, dA, lenA, dB, lenB) =
  *                 the union band in the form of a run of that grouping; band position i belongs to the first latitude of
  *                 the pair iff dA <= i < dA + lenA, to the second iff dB <= i < dB + lenB (len < 32)
+ *     gather_span [2*nvout]   per virtual output latitude (first column, columns): an arc of the circle that holds every
+ *                 neighbor column of query column 0 (of query column j: the arc shifted by j); columns = the whole
+ *                 circle when the runs do not fit a shorter arc
  * The builder runs on the host; the caller copies the blob to the device unchanged (it can also be stored and reused:
  * it depends only on the CSR and the four grid extents) and passes the device address with a host copy of the header.
  *
@@ -118,6 +121,7 @@ enum {
     S2ATTN_PH_SCATTER_PAIR_OFF = 23,
     S2ATTN_PH_SCATTER_PAIR_RUNS = 24,
     S2ATTN_PH_SCATTER_NPAIRS = 25,
+    S2ATTN_PH_GATHER_SPAN = 26, /* nvout x (first column, columns): an arc holding every neighbor column of query column 0 */
     S2ATTN_PH_NLAT_IN = 28, /* the grid extents the plan was built for: checked against the shape of every call */
     S2ATTN_PH_NLON_IN = 29,
     S2ATTN_PH_NLAT_OUT = 30,

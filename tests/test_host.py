@@ -223,6 +223,33 @@ def test_plan_blob_is_self_describing():
     assert rc == -1 and b"built for" in lib.s2attn_last_error()
 
 
+@pytest.mark.parametrize(
+    "ins,outs,cut", [((12, 24), (6, 12), 0.6), ((9, 48), (9, 48), 0.5), ((7, 120), (5, 40), 0.7), ((6, 40), (6, 40), 7.0), ((12, 80), (12, 80), 0.2)]
+)
+def test_plan_neighbor_arcs_hold_every_run(ins, outs, cut):
+    """gather_span: per virtual output latitude an arc (first column, columns) of the circle; every column a run of that latitude
+    gives query column 0 lies on it, rows without neighbors have an empty arc, and no arc is longer than the circle."""
+    from torch_harmonics_amd.plan import build_host_blob
+
+    col, roff, _ = precompute_neighborhood_s2(ins, outs, "equiangular", "equiangular", cut)
+    plan = build_host_blob(col, roff, ins[0], ins[1], outs[0], outs[1])
+    h, PH = plan.header, _lib.PH
+    goff, gruns = plan.arrays()[0].tolist(), plan.arrays()[1].tolist()
+    nvout, W = h[PH["NVOUT"]], min(ins[1], outs[1])
+    span = plan.blob[h[PH["GATHER_SPAN"]] : h[PH["GATHER_SPAN"]] + 2 * nvout].view(nvout, 2).tolist()
+    short = 0
+    for r in range(nvout):
+        s0, n = span[r]
+        assert 0 <= n <= W and 0 <= s0 < W
+        assert (n == 0) == (goff[r] == goff[r + 1])
+        for g in range(goff[r], goff[r + 1]):
+            _, ws, ln, _ = gruns[g]
+            assert all(((ws + t - s0) % W) < n for t in range(ln)), (r, span[r], gruns[g])
+        short += 0 < n < W
+    if cut < 1.0:
+        assert short > 0  # the arcs are not all whole circles
+
+
 def test_plan_handles_arbitrary_unsorted_csr_with_duplicates():
     gen = torch.Generator().manual_seed(5)
     Hi, Wi, Ho, Wo = 5, 12, 4, 6

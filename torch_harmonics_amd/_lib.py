@@ -32,7 +32,7 @@ PH = dict(
     GATHER_OFF=8, GATHER_RUNS=9, GATHER_ORDER=10, GATHER_ORDER_MIXED=11,
     SCATTER_OFF=12, SCATTER_RUNS=13, SCATTER_ORDER=14, SCATTER_ORDER_MIXED=15,
     GATHER_NITEMS=16, GATHER_ITEMS=17, GATHER_PAIR_OFF=18, GATHER_PAIR_RUNS=19, GATHER_NPAIRS=20,
-    SCATTER_NITEMS=21, SCATTER_ITEMS=22, SCATTER_PAIR_OFF=23, SCATTER_PAIR_RUNS=24, SCATTER_NPAIRS=25,
+    SCATTER_NITEMS=21, SCATTER_ITEMS=22, SCATTER_PAIR_OFF=23, SCATTER_PAIR_RUNS=24, SCATTER_NPAIRS=25, GATHER_SPAN=26,
     NLAT_IN=28, NLON_IN=29, NLAT_OUT=30, NLON_OUT=31,
 )  # fmt: skip
 

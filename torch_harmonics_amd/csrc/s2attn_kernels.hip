@@ -298,6 +298,7 @@ struct Args {
     // and the caller's running state
     int r_lon_lo, r_nkx, r_lat0, r_nlat;
     float *r_yacc, *r_asum, *r_qmax;
+    const int2 *gspan; // per virtual output latitude: the arc of neighbor columns of query column 0 (see the plan)
 };
 
 // Key-side addressing.  With nlon_in = kps * nlon_out, query column wo sees input columns ws + t + kps * wo: on the
@@ -2546,8 +2547,8 @@ int check_plan(const s2attn_plan *plan, const s2attn_shape *sh)
         return s2attn_fail(S2ATTN_E_INVALID, "plan was built for grids %dx%d -> %dx%d, the call is for %dx%d -> %dx%d", h[S2ATTN_PH_NLAT_IN], h[S2ATTN_PH_NLON_IN],
                            h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], sh->nlat_in, sh->nlon_in, sh->nlat_out, sh->nlon_out);
     const int32_t total = h[S2ATTN_PH_TOTAL];
-    for (int i = S2ATTN_PH_GATHER_OFF; i <= S2ATTN_PH_SCATTER_PAIR_RUNS; i++) {
-        if (i == S2ATTN_PH_GATHER_NITEMS || i == S2ATTN_PH_GATHER_NPAIRS || i == S2ATTN_PH_SCATTER_NITEMS) continue;
+    for (int i = S2ATTN_PH_GATHER_OFF; i <= S2ATTN_PH_GATHER_SPAN; i++) {
+        if (i == S2ATTN_PH_GATHER_NITEMS || i == S2ATTN_PH_GATHER_NPAIRS || i == S2ATTN_PH_SCATTER_NITEMS || i == S2ATTN_PH_SCATTER_NPAIRS) continue;
         if (h[i] < S2ATTN_PLAN_HEADER_INTS || h[i] > total) return s2attn_fail(S2ATTN_E_INVALID, "plan header: offset %d of array %d lies outside the plan", h[i], i);
     }
     return S2ATTN_OK;
@@ -2645,12 +2646,15 @@ extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const
     const void *ptrs[] = {k, v, q, y_acc};
     for (const void *p : ptrs)
         if (!aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring step takes 16-byte aligned tensors");
+    for (int i : {S2ATTN_PH_GATHER_OFF, S2ATTN_PH_GATHER_RUNS, S2ATTN_PH_GATHER_ORDER, S2ATTN_PH_GATHER_SPAN})
+        if (h[i] < S2ATTN_PLAN_HEADER_INTS || h[i] > h[S2ATTN_PH_TOTAL]) return s2attn_fail(S2ATTN_E_INVALID, "plan header: offset %d of array %d lies outside the plan", h[i], i);
     Args a = {};
     const int32_t *d = plan->data;
     a.quad_w = quad_weights;
     a.goff = d + h[S2ATTN_PH_GATHER_OFF];
     a.gruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_GATHER_RUNS]);
     a.gorder = d + h[S2ATTN_PH_GATHER_ORDER];
+    a.gspan = reinterpret_cast<const int2 *>(d + h[S2ATTN_PH_GATHER_SPAN]);
     a.k = k, a.v = v, a.q = q;
     a.B = sh->batch, a.nh = 1, a.kps = sh->pscale, a.qps = 1;
     a.Hi = h[S2ATTN_PH_NLAT_IN] * sh->pscale, a.Wi = W;

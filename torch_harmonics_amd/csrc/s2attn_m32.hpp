@@ -638,6 +638,18 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
     const bool mine = c < nvalid;
     const size_t pt = ((size_t)b * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
 
+    { // the arc of columns this tile's queries can see, against the virtual columns that can lie in the chunk: most tiles of
+      // an equatorial latitude leave here, without reading a run
+        typedef int i2v __attribute__((ext_vector_type(2)));
+        const i2v span = uniform_load(reinterpret_cast<const i2v *>(a.gspan) + ho);
+        const int la = span[1] + HQ - 1, b0 = a.r_lon_lo / a.kps, lb = (a.r_lon_lo + a.r_nkx - 1) / a.kps + 1 - b0;
+        if (span[1] <= 0) return;
+        if (la < a.Wi && lb < a.Wi) {
+            int dab = (b0 - (w0 + span[0])) % a.Wi; // chunk start relative to the arc's start
+            dab += dab < 0 ? a.Wi : 0;
+            if (dab >= la && a.Wi - dab >= lb) return;
+        }
+    }
     RingWalk wk;
     wk.W = a.Wi, wk.kps = a.kps, wk.w0 = w0, wk.lon_lo = a.r_lon_lo, wk.nkx = a.r_nkx, wk.lat0 = a.r_lat0, wk.nlat = a.r_nlat;
     wk.start(a.gruns, a.quad_w, a.goff[ho], a.goff[ho + 1]);

@@ -325,6 +325,20 @@ int build_blob(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int 
         gcost[r.ho].add(r.len);
         scost[r.hi].add(r.len);
     }
+    // per virtual output latitude: an arc (first column, columns) of the circle that holds every neighbor column of query
+    // column 0 (of query column j: shifted by j); the ring step uses it to leave a tile whose arc misses the chunk at once
+    std::vector<int32_t> gspan(2 * (size_t)nvout, 0);
+    for (int r = 0; r < nvout; r++) {
+        int lo = 0, hi = 0;
+        for (int32_t g = goff[r]; g < goff[r + 1]; g++) {
+            const int c0 = centred(gruns[4 * g + 1], W), c1 = c0 + gruns[4 * g + 2];
+            if (g == goff[r] || c0 < lo) lo = c0;
+            if (g == goff[r] || c1 > hi) hi = c1;
+        }
+        const int n_ = hi - lo >= W ? W : hi - lo;
+        gspan[2 * r + 0] = n_ >= W ? 0 : ((lo % W) + W) % W;
+        gspan[2 * r + 1] = n_;
+    }
     std::vector<int32_t> gorder(nvout), gmixed(nvout), sorder(nvin), smixed(nvin);
     const int32_t gnd = order_rows(gcost, gorder.data(), gmixed.data());
     const int32_t snd = order_rows(scost, sorder.data(), smixed.data());
@@ -356,6 +370,7 @@ int build_blob(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int 
     h[S2ATTN_PH_SCATTER_PAIR_OFF] = append(blob, spoff.data(), spoff.size());
     h[S2ATTN_PH_SCATTER_PAIR_RUNS] = append(blob, spruns.data(), spruns.size());
     h[S2ATTN_PH_SCATTER_NPAIRS] = (int32_t)spoff.size() - 1;
+    h[S2ATTN_PH_GATHER_SPAN] = append(blob, gspan.data(), gspan.size());
     while (blob.size() % 4) blob.push_back(0);
     if (blob.size() > 0x7fffffffULL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the plan needs %zu ints, more than its 32-bit offsets index", blob.size());
     h[S2ATTN_PH_TOTAL] = (int32_t)blob.size();
