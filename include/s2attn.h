@@ -305,20 +305,24 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
                                const int32_t *row_idx, const s2attn_ring_shape *shape, void *stream);
 
 /*
- * s2attn_ring_forward_step on the band-staged matrix-core kernels (same reference operator, attention_interface.cpp:138-143,
- * attention_cuda_fwd_ring.cu:66-175; same tensors and state, same result up to the order of the fp32 sums): instead of the
- * CSR it takes the run-length plan of the LOCAL psi, built once per psi by s2attn_plan_build(col_idx, row_off, nnz,
- * nlat_in = global input latitudes, nlon_in, nlat_out = local output latitudes, nlon_out = nlon_in / pscale) on host copies
- * of the same col_idx / row_off.  A row of a staged band is one input longitude, so the chunk clips rows of the band and
- * the kernel walks only the steps of each run that hold a longitude of the chunk.  Shapes: fp32 storage, ck == cv a
- * multiple of 4 from 16 to 64, nlon_in / pscale >= 32, 16-byte aligned tensors; anything else returns
- * S2ATTN_E_UNSUPPORTED and the caller uses s2attn_ring_forward_step.  (alpha_sum of this kernel and of
- * s2attn_ring_backward_pass1 are the same sum in two orders; the dq formula above, fed the forward's alpha_sum as the
- * reference does, amplifies their last-bit difference by |alpha_kvw| / alpha_sum, which grows with the head width: at 128
- * channels it reaches 2e-5 on values of magnitude 1, which is why wider heads stay on the gather formulation.)
+ * s2attn_ring_forward_step and s2attn_ring_backward_pass1 on the band-staged matrix-core kernels (same reference operators,
+ * attention_interface.cpp:138-150, attention_cuda_fwd_ring.cu:66-175, attention_cuda_bwd_ring.cu:78-205; same tensors and
+ * state, same results up to the order of the fp32 sums): instead of the CSR they take the run-length plan of the LOCAL psi,
+ * built once per psi by s2attn_plan_build(col_idx, row_off, nnz, nlat_in = global input latitudes, nlon_in, nlat_out =
+ * local output latitudes, nlon_out = nlon_in / pscale) on host copies of the same col_idx / row_off.  A row of a staged
+ * band is one input longitude, so the chunk clips rows of the band and the kernels walk only the steps of each run that
+ * hold a longitude of the chunk.  Shapes: fp32 storage, ck == cv a multiple of 4 from 16 to 128, nlon_in / pscale >= 32,
+ * 16-byte aligned tensors; anything else returns S2ATTN_E_UNSUPPORTED and the caller uses the entry points above.
+ * Pass 1 re-accumulates alpha_sum and qdotk_max with the forward step's operations in the forward step's order: fed the
+ * same chunks in the same order the two alpha_sum are bit-identical, which the dq formula above (the forward's alpha_sum
+ * with pass 1's other sums, as the reference combines them) relies on for wide heads - use the two together.
  */
 int s2attn_ring_forward_step_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
                                   const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *shape, void *stream);
+
+int s2attn_ring_backward_pass1_plan(const void *k, const void *v, const void *q, const void *dy, float *alpha_sum, float *qdotk_max,
+                                    float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                                    const s2attn_plan *plan, const s2attn_ring_shape *shape, void *stream);
 
 /*
  * Regrouped psi.  Every ring kernel of this library is a gather: the cell that owns a sum walks the entries of its own

@@ -298,6 +298,7 @@ struct Args {
     // and the caller's running state
     int r_lon_lo, r_nkx, r_lat0, r_nlat;
     float *r_yacc, *r_asum, *r_qmax;
+    float *r_integral, *r_ak, *r_akvw; // pass 1 of the backward
     const int2 *gspan; // per virtual output latitude: the arc of neighbor columns of query column 0 (see the plan)
 };
 
@@ -2191,7 +2192,7 @@ enum Which { FWD, DQ, DKDV };
 
 template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream);
 template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream);
-template <int D> int launch_ring_fwd_m32(const Args &a0, hipStream_t stream);
+template <int D, bool PASS1> int launch_ring_m32(const Args &a0, hipStream_t stream);
 
 #if S2_PART == 0 || S2_PART == 2
 // 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
@@ -2275,23 +2276,28 @@ template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t
 }
 #endif
 #if S2_PART == 0 || S2_PART == 3
-// one ring step of the forward on the fp32 16-longitude kernels: one wavefront per 16 local output longitudes
-template <int D> int launch_ring_fwd_m32(const Args &a0, hipStream_t stream)
+// one ring step (forward, or pass 1 of the backward) on the fp32 16-longitude kernels: one wavefront per 16 local output longitudes
+template <int D, bool PASS1> int launch_ring_m32(const Args &a0, hipStream_t stream)
 {
     Args a = a0;
     a.row_first = 0;
     const long nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    hipLaunchKernelGGL(ring_fwd_m32_kernel<D>, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL((ring_m32_kernel<D, PASS1>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
 #endif
 #if S2_PART == 3
-template int launch_ring_fwd_m32<16>(const Args &, hipStream_t);
-template int launch_ring_fwd_m32<32>(const Args &, hipStream_t);
-template int launch_ring_fwd_m32<64>(const Args &, hipStream_t);
+template int launch_ring_m32<16, false>(const Args &, hipStream_t);
+template int launch_ring_m32<32, false>(const Args &, hipStream_t);
+template int launch_ring_m32<64, false>(const Args &, hipStream_t);
+template int launch_ring_m32<128, false>(const Args &, hipStream_t);
+template int launch_ring_m32<16, true>(const Args &, hipStream_t);
+template int launch_ring_m32<32, true>(const Args &, hipStream_t);
+template int launch_ring_m32<64, true>(const Args &, hipStream_t);
+template int launch_ring_m32<128, true>(const Args &, hipStream_t);
 template int launch_m32<16, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<32, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<64, 1>(Which, const Args &, hipStream_t);
@@ -2621,9 +2627,10 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     return launch(FWD, a, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
 }
 
-// One ring step of the forward on the band-staged kernels (see ring_fwd_m32_kernel).
-extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
-                                             const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
+// Ring steps on the band-staged kernels (ring_m32_kernel): checks and kernel arguments shared by the forward step and pass 1.
+namespace {
+int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, const s2attn_plan *plan,
+                   const s2attn_ring_shape *sh)
 {
     if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "ring shape is null");
     if (sh->batch < 1 || sh->nlat_halo < 1 || sh->nlon_kx < 1 || sh->nlat_out < 1 || sh->nlon_out < 1 || sh->nlon_in < 1)
@@ -2634,38 +2641,66 @@ extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const
         return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", sh->lon_lo_kx, sh->lon_lo_kx + sh->nlon_kx, sh->nlon_in);
     const int W = sh->nlon_in / sh->pscale; // global output longitudes = columns of a virtual input latitude
     if (sh->nlon_out > W) return s2attn_fail(S2ATTN_E_INVALID, "pscale * nlon_out = %ld exceeds nlon_in = %d", (long)sh->pscale * sh->nlon_out, sh->nlon_in);
-    if (!k || !v || !q || !y_acc || !alpha_sum || !qdotk_max || !quad_weights) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!k || !v || !q || !quad_weights) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!plan || !plan->data) return s2attn_fail(S2ATTN_E_INVALID, "plan is null");
     const int32_t *h = plan->header;
     if (h[S2ATTN_PH_MAGIC] != S2ATTN_PLAN_MAGIC) return s2attn_fail(S2ATTN_E_INVALID, "plan header does not carry this library's plan format");
     if (h[S2ATTN_PH_NLON_IN] != sh->nlon_in || h[S2ATTN_PH_NLAT_OUT] != sh->nlat_out || h[S2ATTN_PH_NLON_OUT] != W)
         return s2attn_fail(S2ATTN_E_INVALID, "plan was built for %d input longitudes and %dx%d output points, the step is for %d and %dx%d (global longitudes)",
                            h[S2ATTN_PH_NLON_IN], h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], sh->nlon_in, sh->nlat_out, W);
-    if (sh->dtype != S2ATTN_F32 || !m32_width(sh->ck, sh->cv) || sh->ck > 64 || W < HK)
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring step takes fp32 tensors with ck = cv a multiple of 4 from 16 to 64 and at least %d global output longitudes", HK);
-    const void *ptrs[] = {k, v, q, y_acc};
+    if (sh->dtype != S2ATTN_F32 || !m32_width(sh->ck, sh->cv) || sh->ck > 128 || W < HK)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take fp32 tensors with ck = cv a multiple of 4 from 16 to 128 and at least %d global output longitudes", HK);
+    const void *ptrs[] = {k, v, q, dy};
     for (const void *p : ptrs)
-        if (!aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring step takes 16-byte aligned tensors");
+        if (p && !aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     for (int i : {S2ATTN_PH_GATHER_OFF, S2ATTN_PH_GATHER_RUNS, S2ATTN_PH_GATHER_ORDER, S2ATTN_PH_GATHER_SPAN})
         if (h[i] < S2ATTN_PLAN_HEADER_INTS || h[i] > h[S2ATTN_PH_TOTAL]) return s2attn_fail(S2ATTN_E_INVALID, "plan header: offset %d of array %d lies outside the plan", h[i], i);
-    Args a = {};
     const int32_t *d = plan->data;
     a.quad_w = quad_weights;
     a.goff = d + h[S2ATTN_PH_GATHER_OFF];
     a.gruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_GATHER_RUNS]);
     a.gorder = d + h[S2ATTN_PH_GATHER_ORDER];
     a.gspan = reinterpret_cast<const int2 *>(d + h[S2ATTN_PH_GATHER_SPAN]);
-    a.k = k, a.v = v, a.q = q;
+    a.k = k, a.v = v, a.q = q, a.dy = dy;
     a.B = sh->batch, a.nh = 1, a.kps = sh->pscale, a.qps = 1;
     a.Hi = h[S2ATTN_PH_NLAT_IN] * sh->pscale, a.Wi = W;
     a.Ho = sh->nlat_out, a.Wo = sh->nlon_out; // local output points; runs are relative to local column 0
     a.dk_ = a.dv_ = sh->ck;
     a.r_lon_lo = sh->lon_lo_kx, a.r_nkx = sh->nlon_kx, a.r_lat0 = sh->lat_halo_start, a.r_nlat = sh->nlat_halo;
+    return S2ATTN_OK;
+}
+template <bool PASS1> int launch_ring_plan(const Args &a, hipStream_t st)
+{
+    if (a.dk_ <= 16) return launch_ring_m32<16, PASS1>(a, st);
+    if (a.dk_ <= 32) return launch_ring_m32<32, PASS1>(a, st);
+    if (a.dk_ <= 64) return launch_ring_m32<64, PASS1>(a, st);
+    return launch_ring_m32<128, PASS1>(a, st);
+}
+} // namespace
+
+extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                                             const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
+{
+    Args a = {};
+    const int rc = ring_plan_args(a, k, v, q, nullptr, quad_weights, plan, sh);
+    if (rc != S2ATTN_OK) return rc;
+    if (!y_acc || !alpha_sum || !qdotk_max) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!aligned(y_acc, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_yacc = y_acc, a.r_asum = alpha_sum, a.r_qmax = qdotk_max;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (sh->ck <= 16) return launch_ring_fwd_m32<16>(a, st);
-    if (sh->ck <= 32) return launch_ring_fwd_m32<32>(a, st);
-    return launch_ring_fwd_m32<64>(a, st);
+    return launch_ring_plan<false>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2attn_ring_backward_pass1_plan(const void *k, const void *v, const void *q, const void *dy, float *alpha_sum, float *qdotk_max,
+                                               float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                                               const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
+{
+    Args a = {};
+    const int rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, sh);
+    if (rc != S2ATTN_OK) return rc;
+    if (!dy || !alpha_sum || !qdotk_max || !integral || !alpha_k || !alpha_kvw) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!aligned(alpha_k, 16) || !aligned(alpha_kvw, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
+    a.r_asum = alpha_sum, a.r_qmax = qdotk_max, a.r_integral = integral, a.r_ak = alpha_k, a.r_akvw = alpha_kvw;
+    return launch_ring_plan<true>(a, static_cast<hipStream_t>(stream));
 }
 
 namespace {

@@ -622,7 +622,11 @@ struct RingWalk {
     }
 };
 
-template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd_m32_kernel(const Args a)
+// PASS1 = false: the forward step (state y_acc, alpha_sum, qdotk_max).  PASS1 = true: pass 1 of the backward, which walks
+// the same steps and re-accumulates alpha_sum and qdotk_max (the same operations in the same order as the forward step:
+// the two sums are bit-identical) together with integral = sum_j alpha_j <dy, v_j>, alpha_k = sum_j alpha_j k_j and
+// alpha_kvw = sum_j alpha_j <dy, v_j> k_j: a second score product G^T = V dY^T and two accumulations against K^T.
+template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1) ? 4 : (D <= 32 ? 3 : (D <= 64 && !PASS1 ? 2 : 1))) void ring_m32_kernel(const Args a)
 {
     constexpr int NS = 1;
     typedef FTile<D> Tile;
@@ -655,21 +659,30 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
     wk.start(a.gruns, a.quad_w, a.goff[ho], a.goff[ho + 1]);
     if (!wk.advance()) return; // nothing of this tile's neighborhood is in the chunk
 
-    float qop[D / 4];
+    float qop[D / 4], gop[PASS1 ? D / 4 : 1];
     m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb, qd, dr);
-    f4v acc[NCB]; // Y^T: register v of block cb is channel 16 cb + 4 qd + v of column c
+    if constexpr (PASS1) m32_load_quarter<D>(gop, static_cast<const char *>(a.dy) + pt * ldb, qd, dr);
+    // forward: Y^T; pass 1: alpha_k^T (acc) and alpha_kvw^T (acc2): register v of block cb is channel 16 cb + 4 qd + v of column c
+    float *const acc_state = PASS1 ? a.r_ak : a.r_yacc;
+    f4v acc[NCB], acc2[PASS1 ? NCB : 1];
 #pragma unroll
     for (int cb = 0; cb < NCB; cb++) {
-        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (16 * cb + 4 * qd < dr) x = *reinterpret_cast<const float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd);
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f), x2 = x;
+        if (16 * cb + 4 * qd < dr) {
+            x = *reinterpret_cast<const float4 *>(acc_state + pt * drt + 16 * cb + 4 * qd);
+            if constexpr (PASS1) x2 = *reinterpret_cast<const float4 *>(a.r_akvw + pt * drt + 16 * cb + 4 * qd);
+        }
         acc[cb] = f4v{x.x, x.y, x.z, x.w};
+        if constexpr (PASS1) acc2[cb] = f4v{x2.x, x2.y, x2.z, x2.w};
     }
     // The exponentials are taken relative to a reference point m that is moved lazily (when a column's maximum has grown by
     // more than RESCALE_THR binary orders: after a tile's first steps that is rare, and a step then needs neither an exchange
     // between the four lanes of a column nor a rescaling); the exact maximum the state asks for is kept per lane (mtrue)
     // and the sums are brought to it once, at the end.
     float m = fmaxf(a.r_qmax[pt], NEG_BIG_NAT), mtrue = -INFINITY;
-    float S = qd == 0 ? a.r_asum[pt] : 0.f; // the four lanes of a column each keep a share of the sum
+    float S = qd == 0 ? a.r_asum[pt] : 0.f; // the four lanes of a column each keep a share of the sums
+    float I = 0.f;
+    if constexpr (PASS1) I = qd == 0 ? a.r_integral[pt] : 0.f;
 
     Tile kt, vt;
     const int r0 = lane / Tile::CPR;
@@ -695,6 +708,7 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
     vt.commit(Vs, lane);
     __syncthreads();
     settle(qop);
+    if constexpr (PASS1) settle(gop);
 
     for (;;) {
         const float lw = fast_log2(wk.w);
@@ -702,8 +716,9 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
         const bool more = wk.advance();
         if (more) fetch();
 
-        f4v sc[2];
+        f4v sc[2], gc[2];
         m32_scores<D, PITCH>(sc, Ks, c, qd, qop);
+        if constexpr (PASS1) m32_scores<D, PITCH>(gc, Vs, c, qd, gop);
         // element (kb, v) is band position u = pos + 16 kb + 4 qd + v and neighbor t = u - c of column c: it counts iff
         // 0 <= t < len and u < ub, i.e. t < min(len, ub - c) as unsigned numbers
         const int tb = pos + 4 * qd - c;
@@ -735,6 +750,11 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
             S *= corr;
 #pragma unroll
             for (int cb = 0; cb < NCB; cb++) acc[cb] *= corr;
+            if constexpr (PASS1) {
+                I *= corr;
+#pragma unroll
+                for (int cb = 0; cb < NCB; cb++) acc2[cb] *= corr;
+            }
             m = mn;
         }
         const float sh = fmaf(-m, LOG2E, lw);
@@ -742,12 +762,21 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
         for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
             for (int v = 0; v < 4; v++) {
-                const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // = exp(q.k - max) w; not counted: exp2(-inf) = 0
+                const float p = fast_exp2(fmaf(sc[kb][v], LOG2E, sh)); // = exp(q.k - m) w; not counted: exp2(-inf) = 0
                 sc[kb][v] = p;
                 S += p;
+                if constexpr (PASS1) {
+                    gc[kb][v] *= p; // rows outside the chunk are staged as zeros, so <dy, v> is finite wherever p = 0
+                    I += gc[kb][v];
+                }
             }
         }
-        m32_accumulate<D, PITCH>(acc, Vs, c, qd, sc);
+        if constexpr (PASS1) {
+            m32_accumulate<D, PITCH>(acc, Ks, c, qd, sc);
+            m32_accumulate<D, PITCH>(acc2, Ks, c, qd, gc);
+        } else {
+            m32_accumulate<D, PITCH>(acc, Vs, c, qd, sc);
+        }
 
         __syncthreads();
         if (!more) break;
@@ -757,16 +786,22 @@ template <int D> __global__ __launch_bounds__(64, D <= 32 ? 4 : 2) void ring_fwd
     }
 
     S = h16_quarter_sum(S);
+    if constexpr (PASS1) I = h16_quarter_sum(I);
     mtrue = fmaxf(h16_quarter_max(mtrue), a.r_qmax[pt]); // the maximum over everything this column has seen, earlier chunks included (read again: a register less in the loop)
     const float f = mtrue > -INFINITY ? fast_exp2((m - mtrue) * LOG2E) : 1.f; // m <= mtrue <= m + THR; a column without neighbors keeps its zeros
     if (mine) {
         if (qd == 0) {
             a.r_asum[pt] = S * f;
             a.r_qmax[pt] = mtrue;
+            if constexpr (PASS1) a.r_integral[pt] = I * f;
         }
 #pragma unroll
-        for (int cb = 0; cb < NCB; cb++)
-            if (16 * cb + 4 * qd < dr)
-                *reinterpret_cast<float4 *>(a.r_yacc + pt * drt + 16 * cb + 4 * qd) = make_float4(acc[cb][0] * f, acc[cb][1] * f, acc[cb][2] * f, acc[cb][3] * f);
+        for (int cb = 0; cb < NCB; cb++) {
+            if (16 * cb + 4 * qd < dr) {
+                *reinterpret_cast<float4 *>(acc_state + pt * drt + 16 * cb + 4 * qd) = make_float4(acc[cb][0] * f, acc[cb][1] * f, acc[cb][2] * f, acc[cb][3] * f);
+                if constexpr (PASS1)
+                    *reinterpret_cast<float4 *>(a.r_akvw + pt * drt + 16 * cb + 4 * qd) = make_float4(acc2[cb][0] * f, acc2[cb][1] * f, acc2[cb][2] * f, acc2[cb][3] * f);
+            }
+        }
     }
 }

@@ -252,12 +252,14 @@ def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out
     return _lib.RingShapeStruct(B, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, vx.shape[3], nlon_in, pscale, lon_lo_kx, lat_halo_start, _DTYPE_CODE[qy.dtype])
 
 
-def _ring_takes_plan(kx, vx, qy, y_acc, nlon_in, pscale) -> bool:
-    """Shapes of the band-staged ring forward step (s2attn_ring_forward_step_plan in include/s2attn.h)."""
+def _ring_takes_plan(kx, vx, qy, nlon_in, pscale) -> bool:
+    """Shapes of the band-staged ring steps (s2attn_ring_forward_step_plan, s2attn_ring_backward_pass1_plan in include/s2attn.h).
+    Decided by the shape alone, so that the forward step and pass 1 of one problem always run the same formulation (their
+    alpha_sum are then bit-identical; the state buffers are fresh torch allocations, 16-byte aligned like every tensor)."""
     ck, cv = kx.shape[3], vx.shape[3]
-    if qy.dtype != torch.float32 or ck != cv or ck % 4 or not 16 <= ck <= 64 or nlon_in // pscale < 32:
+    if qy.dtype != torch.float32 or ck != cv or ck % 4 or not 16 <= ck <= 128 or nlon_in // pscale < 32:
         return False
-    return all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, y_acc))
+    return True
 
 
 def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_idx, nlat_out, nlon_out, nrows=None):
@@ -318,7 +320,7 @@ def forward_ring_step(
     if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:  # nothing to fold in
         return
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
-    if _ring_takes_plan(kx, vx, qy, y_acc, nlon_in, pscale):
+    if _ring_takes_plan(kx, vx, qy, nlon_in, pscale) and all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, y_acc)):
         # band-staged matrix-core step on the run-length plan of the local psi (built on the host once per psi, cached)
         p = _plan.get_plan(col_idx, row_off, quad_weights.numel(), nlon_in, nlat_out, nlon_in // pscale)
         with torch.cuda.device(kx.device):
@@ -375,6 +377,16 @@ def backward_ring_step_pass1(
     if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:  # nothing to fold in
         return
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    if _ring_takes_plan(kx, vx, qy, nlon_in, pscale) and all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, dy, alpha_k_buf, alpha_kvw_buf)):
+        p = _plan.get_plan(col_idx, row_off, quad_weights.numel(), nlon_in, nlat_out, nlon_in // pscale)
+        with torch.cuda.device(kx.device):
+            rc = _lib.load().s2attn_ring_backward_pass1_plan(
+                kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+                integral_buf.data_ptr(), alpha_k_buf.data_ptr(), alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(),
+                ctypes.byref(p.struct), ctypes.byref(shape), _stream_ptr(kx.device),
+            )  # fmt: skip
+        _lib.check(rc, "s2attn_ring_backward_pass1_plan")
+        return
     with torch.cuda.device(kx.device):
         rc = _lib.load().s2attn_ring_backward_pass1(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
