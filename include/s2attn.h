@@ -305,8 +305,8 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
                                const int32_t *row_idx, const s2attn_ring_shape *shape, void *stream);
 
 /*
- * s2attn_ring_forward_step and s2attn_ring_backward_pass1 on the band-staged matrix-core kernels (same reference operators,
- * attention_interface.cpp:138-150, attention_cuda_fwd_ring.cu:66-175, attention_cuda_bwd_ring.cu:78-205; same tensors and
+ * s2attn_ring_forward_step and s2attn_ring_backward_pass1 / pass2 on the band-staged matrix-core kernels (same reference operators,
+ * attention_interface.cpp:138-156, attention_cuda_fwd_ring.cu:66-175, attention_cuda_bwd_ring.cu:78-205; same tensors and
  * state, same results up to the order of the fp32 sums): instead of the CSR they take the run-length plan of the LOCAL psi,
  * built once per psi by s2attn_plan_build(col_idx, row_off, nnz, nlat_in = global input latitudes, nlon_in, nlat_out =
  * local output latitudes, nlon_out = nlon_in / pscale) on host copies of the same col_idx / row_off.  A row of a staged
@@ -323,6 +323,12 @@ int s2attn_ring_forward_step_plan(const void *k, const void *v, const void *q, f
 int s2attn_ring_backward_pass1_plan(const void *k, const void *v, const void *q, const void *dy, float *alpha_sum, float *qdotk_max,
                                     float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
                                     const s2attn_plan *plan, const s2attn_ring_shape *shape, void *stream);
+
+/* s2attn_ring_backward_pass2 likewise (attention_interface.cpp:151-156, attention_cuda_bwd_ring.cu:1312-1440): a wavefront owns 16
+ * keys of the chunk and gathers over the plan's runs grouped by input latitude; dk, dv are added to plainly (no atomics). */
+int s2attn_ring_backward_pass2_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                    const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                    const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *shape, void *stream);
 
 /*
  * Regrouped psi.  Every ring kernel of this library is a gather: the cell that owns a sum walks the entries of its own

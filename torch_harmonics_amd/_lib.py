@@ -109,6 +109,7 @@ SYMBOLS = {
     "s2attn_ring_forward_step": (_int, [_vp] * 10 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_forward_step_plan": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1_plan": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_backward_pass2_plan": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_regroup_psi": (_i64, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),

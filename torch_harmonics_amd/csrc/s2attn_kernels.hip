@@ -2193,6 +2193,7 @@ enum Which { FWD, DQ, DKDV };
 template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream);
 template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream);
 template <int D, bool PASS1> int launch_ring_m32(const Args &a0, hipStream_t stream);
+template <int D> int launch_ring_pass2_m32(const Args &a0, hipStream_t stream);
 
 #if S2_PART == 0 || S2_PART == 2
 // 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
@@ -2288,8 +2289,23 @@ template <int D, bool PASS1> int launch_ring_m32(const Args &a0, hipStream_t str
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
+// pass 2 of a ring step: one wavefront per 16 virtual columns of a column class of a chunk latitude
+template <int D> int launch_ring_pass2_m32(const Args &a, hipStream_t stream)
+{
+    const int ntile = (a.r_nkx / a.kps + 1 + HQ - 1) / HQ + 1; // as in the kernel
+    const long nblocks = (long)a.Hi * ntile * a.B;
+    if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
+    hipLaunchKernelGGL(ring_pass2_m32_kernel<D>, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    const hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
+    return S2ATTN_OK;
+}
 #endif
 #if S2_PART == 3
+template int launch_ring_pass2_m32<16>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128>(const Args &, hipStream_t);
 template int launch_ring_m32<16, false>(const Args &, hipStream_t);
 template int launch_ring_m32<32, false>(const Args &, hipStream_t);
 template int launch_ring_m32<64, false>(const Args &, hipStream_t);
@@ -2653,7 +2669,7 @@ int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const v
     const void *ptrs[] = {k, v, q, dy};
     for (const void *p : ptrs)
         if (p && !aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
-    for (int i : {S2ATTN_PH_GATHER_OFF, S2ATTN_PH_GATHER_RUNS, S2ATTN_PH_GATHER_ORDER, S2ATTN_PH_GATHER_SPAN})
+    for (int i : {S2ATTN_PH_GATHER_OFF, S2ATTN_PH_GATHER_RUNS, S2ATTN_PH_GATHER_ORDER, S2ATTN_PH_GATHER_SPAN, S2ATTN_PH_SCATTER_OFF, S2ATTN_PH_SCATTER_RUNS, S2ATTN_PH_SCATTER_ORDER})
         if (h[i] < S2ATTN_PLAN_HEADER_INTS || h[i] > h[S2ATTN_PH_TOTAL]) return s2attn_fail(S2ATTN_E_INVALID, "plan header: offset %d of array %d lies outside the plan", h[i], i);
     const int32_t *d = plan->data;
     a.quad_w = quad_weights;
@@ -2661,6 +2677,9 @@ int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const v
     a.gruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_GATHER_RUNS]);
     a.gorder = d + h[S2ATTN_PH_GATHER_ORDER];
     a.gspan = reinterpret_cast<const int2 *>(d + h[S2ATTN_PH_GATHER_SPAN]);
+    a.soff = d + h[S2ATTN_PH_SCATTER_OFF];
+    a.sruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_SCATTER_RUNS]);
+    a.sorder = d + h[S2ATTN_PH_SCATTER_ORDER];
     a.k = k, a.v = v, a.q = q, a.dy = dy;
     a.B = sh->batch, a.nh = 1, a.kps = sh->pscale, a.qps = 1;
     a.Hi = h[S2ATTN_PH_NLAT_IN] * sh->pscale, a.Wi = W;
@@ -2688,6 +2707,24 @@ extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const
     if (!aligned(y_acc, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_yacc = y_acc, a.r_asum = alpha_sum, a.r_qmax = qdotk_max;
     return launch_ring_plan<false>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2attn_ring_backward_pass2_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                               const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                               const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
+{
+    Args a = {};
+    const int rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, sh);
+    if (rc != S2ATTN_OK) return rc;
+    if (!dy || !alpha_sum || !qdotk_max || !integral_norm || !dk || !dv) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!aligned(dk, 16) || !aligned(dv, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
+    a.r_asum = const_cast<float *>(alpha_sum), a.r_qmax = const_cast<float *>(qdotk_max), a.r_integral = const_cast<float *>(integral_norm);
+    a.dk = dk, a.dv = dv;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (a.dk_ <= 16) return launch_ring_pass2_m32<16>(a, st);
+    if (a.dk_ <= 32) return launch_ring_pass2_m32<32>(a, st);
+    if (a.dk_ <= 64) return launch_ring_pass2_m32<64>(a, st);
+    return launch_ring_pass2_m32<128>(a, st);
 }
 
 extern "C" int s2attn_ring_backward_pass1_plan(const void *k, const void *v, const void *q, const void *dy, float *alpha_sum, float *qdotk_max,

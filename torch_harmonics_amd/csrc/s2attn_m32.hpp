@@ -805,3 +805,157 @@ template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1
         }
     }
 }
+
+// ---- backward, pass 2 of a ring step ---------------------------------------------------------------------------------
+// The dk/dv pass above for the keys of ONE chunk: a wavefront owns 16 consecutive virtual columns of one column class of a
+// chunk latitude (real longitudes (w0 + c) * kps + par) and walks the scatter runs of that virtual latitude; staged rows are
+// local queries with their statistics (alpha_sum, qdotk_max, integral_norm of the caller, natural units) - a row whose query
+// column lies outside the local window of Wo longitudes is staged as zeros and weighs nothing.  dk, dv (fp32, shaped like
+// the chunk) are ADDED to; every key belongs to one wavefront, so plainly.
+template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(const Args a)
+{
+    typedef FTile<D> Tile;
+    constexpr int PITCH = Tile::PITCH, NCB = D / 16;
+    const int lane = threadIdx.x, c = lane & 15, qd = lane >> 4;
+    const int drt = a.dk_, dr = min(D, drt);
+    // workgroup -> (batch, virtual input latitude in the plan's order, tile of 16 virtual columns of the chunk)
+    const int ntile = (a.r_nkx / a.kps + 1 + HQ - 1) / HQ + 1; // enough for every column class and any alignment of the chunk
+    int id = blockIdx.x;
+    const int b = id % a.B;
+    id /= a.B;
+    const int hv = a.sorder[id / ntile], tile = id % ntile;
+    const int hreal = hv / a.kps, par = hv - hreal * a.kps, rl = hreal - a.r_lat0;
+    if (rl < 0 || rl >= a.r_nlat) return;
+    const int vlo = (a.r_lon_lo - par + a.kps - 1) / a.kps, nv = (a.r_lon_lo + a.r_nkx - par + a.kps - 1) / a.kps - vlo;
+    const int w0 = vlo + HQ * tile; // first virtual column of the tile
+    const int nvalid = min(HQ, vlo + nv - w0);
+    if (nvalid <= 0) return;
+    int ri = a.soff[hv];
+    const int rend = a.soff[hv + 1];
+    if (ri >= rend) return; // no query sees this latitude
+
+    char *lds = m32_lds<m32_lds_bytes<D, 1>(true), 1>();
+    char *Qs = lds, *Gs = Qs + HK * PITCH;
+    float *Ls = reinterpret_cast<float *>(Gs + HK * PITCH), *Is = Ls + HK;
+    const unsigned ldb = drt * 4; // bytes between two grid points
+    const char *qy = static_cast<const char *>(a.q) + (size_t)b * a.Ho * a.Wo * ldb;
+    const char *gy = static_cast<const char *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldb;
+    const size_t sbase = (size_t)b * a.Ho * a.Wo;
+    const bool mine = c < nvalid;
+    const size_t pt = ((size_t)b * a.r_nlat + rl) * a.r_nkx + (size_t)((w0 + (mine ? c : 0)) * a.kps + par - a.r_lon_lo); // the key in the chunk
+
+    float kop[D / 4], vop[D / 4]; // this lane's quarter of key c
+    m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + pt * ldb, qd, dr);
+    m32_load_quarter<D>(vop, static_cast<const char *>(a.v) + pt * ldb, qd, dr);
+    f4v dkt[NCB], dvt[NCB];
+#pragma unroll
+    for (int cb = 0; cb < NCB; cb++) {
+        dkt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
+        dvt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
+    }
+    const float lw = fast_log2(a.quad_w[hreal]);
+
+    int pos = 0;
+    Run run = {0, 0, 0, 0};
+    Tile qt, gt;
+    float2 st = make_float2(0.f, 0.f);
+    const int r0 = lane / Tile::CPR;
+    const unsigned pc = 16u * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
+    auto fetch = [&](const Run &rn, int p) {
+        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wi; // query column of staged row 0, on the circle of the global output longitudes
+        c0 += (c0 < 0) ? a.Wi : 0;
+        const size_t lat = (size_t)rn.lat * a.Wo; // local output latitude
+#pragma unroll
+        for (int it = 0; it < Tile::NIT; it++) {
+            int col = c0 + r0 + it * Tile::RPI;
+            col -= (col >= a.Wi) ? a.Wi : 0;
+            qt.raw[it] = u4v{0u, 0u, 0u, 0u};
+            gt.raw[it] = u4v{0u, 0u, 0u, 0u};
+            if (col < a.Wo && piece_ok) { // inside the local window
+                qt.raw[it] = *reinterpret_cast<const u4v *>(qy + (lat + col) * ldb + pc);
+                gt.raw[it] = *reinterpret_cast<const u4v *>(gy + (lat + col) * ldb + pc);
+            }
+        }
+        if (lane < HK) { // lanes 0..31 fetch the statistics of the staged rows: (log2-sum-exp, integral_norm)
+            int col = c0 + lane;
+            col -= (col >= a.Wi) ? a.Wi : 0;
+            st = make_float2(INFINITY, 0.f); // a row outside the window weighs exp2(-inf) = 0
+            if (col < a.Wo) {
+                const size_t s = sbase + lat + col;
+                const float as = a.r_asum[s];
+                if (as > 0.f) st = make_float2(fmaf(a.r_qmax[s], LOG2E, fast_log2(as)), a.r_integral[s]); // (a query that saw nothing weighs nothing)
+            }
+        }
+    };
+    auto commit = [&]() {
+        qt.commit(Qs, lane);
+        gt.commit(Gs, lane);
+        if (lane < HK) {
+            Ls[lane] = st.x;
+            Is[lane] = st.y;
+        }
+    };
+    run = a.sruns[ri];
+    fetch(run, 0);
+    commit();
+    __syncthreads();
+    settle(kop);
+    settle(vop);
+
+    while (ri < rend) {
+        const int len = run.len;
+        int nri = ri, npos = pos + HK;
+        Run nrun = run;
+        if (npos >= len + HQ - 1) {
+            nri++;
+            npos = 0;
+            if (nri < rend) nrun = a.sruns[nri];
+        }
+        const bool more = nri < rend;
+        if (more) fetch(nrun, npos);
+
+        f4v sc[2], gc[2];
+        m32_scores<D, PITCH>(sc, Qs, c, qd, kop);
+        m32_scores<D, PITCH>(gc, Gs, c, qd, vop);
+        const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
+        const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
+#pragma unroll
+        for (int qb = 0; qb < 2; qb++) {
+            const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 16 * qb + 4 * qd);
+            const float4 i4 = *reinterpret_cast<const float4 *>(Is + 16 * qb + 4 * qd);
+            const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+            const float iv[4] = {i4.x, i4.y, i4.z, i4.w};
+#pragma unroll
+            for (int v = 0; v < 4; v++) {
+                float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v])); // = alpha / alpha_sum
+                if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
+                sc[qb][v] = p;
+                gc[qb][v] = p * (gc[qb][v] - iv[v]);
+            }
+        }
+        m32_accumulate<D, PITCH>(dvt, Gs, c, qd, sc);
+        m32_accumulate<D, PITCH>(dkt, Qs, c, qd, gc);
+
+        __syncthreads();
+        if (more) commit();
+        __syncthreads();
+        ri = nri;
+        pos = npos;
+        run = nrun;
+    }
+
+    if (mine) {
+        float *dk = static_cast<float *>(a.dk) + pt * drt + 4 * qd, *dv = static_cast<float *>(a.dv) + pt * drt + 4 * qd;
+#pragma unroll
+        for (int cb = 0; cb < NCB; cb++) {
+            if (16 * cb + 4 * qd < dr) {
+                float4 x = *reinterpret_cast<const float4 *>(dk + 16 * cb), y = *reinterpret_cast<const float4 *>(dv + 16 * cb);
+                x.x += dkt[cb][0], x.y += dkt[cb][1], x.z += dkt[cb][2], x.w += dkt[cb][3];
+                y.x += dvt[cb][0], y.y += dvt[cb][1], y.z += dvt[cb][2], y.w += dvt[cb][3];
+                *reinterpret_cast<float4 *>(dk + 16 * cb) = x;
+                *reinterpret_cast<float4 *>(dv + 16 * cb) = y;
+            }
+        }
+    }
+}

@@ -253,7 +253,7 @@ def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out
 
 
 def _ring_takes_plan(kx, vx, qy, nlon_in, pscale) -> bool:
-    """Shapes of the band-staged ring steps (s2attn_ring_forward_step_plan, s2attn_ring_backward_pass1_plan in include/s2attn.h).
+    """Shapes of the band-staged ring steps (s2attn_ring_forward_step_plan, s2attn_ring_backward_pass1_plan / pass2_plan in include/s2attn.h).
     Decided by the shape alone, so that the forward step and pass 1 of one problem always run the same formulation (their
     alpha_sum are then bit-identical; the state buffers are fresh torch allocations, 16-byte aligned like every tensor)."""
     ck, cv = kx.shape[3], vx.shape[3]
@@ -442,6 +442,12 @@ def backward_ring_step_pass2(
     shape = _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
     head = (kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
             integral_norm_buf.data_ptr(), dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr())  # fmt: skip
+    if not _RING_PASS2_FROM_CSR and _ring_takes_plan(kx, vx, qy, nlon_in, pscale) and all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, dy, dkx, dvx)):
+        p = _plan.get_plan(col_idx, row_off, quad_weights.numel(), nlon_in, nlat_out, nlon_in // pscale)
+        with torch.cuda.device(kx.device):
+            rc = _lib.load().s2attn_ring_backward_pass2_plan(*head, ctypes.byref(p.struct), ctypes.byref(shape), _stream_ptr(kx.device))
+        _lib.check(rc, "s2attn_ring_backward_pass2_plan")
+        return
     with torch.cuda.device(kx.device):
         if _RING_PASS2_FROM_CSR:
             rc = _lib.load().s2attn_ring_backward_pass2(*head, col_idx.data_ptr(), row_off.data_ptr(), row_idx.data_ptr(), ctypes.byref(shape), _stream_ptr(kx.device))
