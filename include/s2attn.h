@@ -396,6 +396,27 @@ int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void
                                         const float *quad_weights, const int64_t *col_idx, const int64_t *row_off,
                                         const int32_t *row_order, const s2attn_ring_up_shape *shape, void *stream);
 
+/*
+ * The three up-sampling steps on the band-staged matrix-core kernels (same operators, same tensors and state): they take the
+ * run-length plan of the local psi, built once per psi by s2attn_plan_build(col_idx, row_off, nnz, nlat_in = nlat_halo (the
+ * chunk's rows, pole padding included), nlon_in, nlat_out = local output latitudes, nlon_out = nlon_out_global) on host
+ * copies of the same col_idx / row_off.  Shapes as for the gather direction: fp32 storage, ck == cv a multiple of 4 from 16
+ * to 128, nlon_in >= 32, 16-byte aligned tensors; anything else returns S2ATTN_E_UNSUPPORTED.  (Pass 1 of this direction
+ * works from the forward's final maximum, so its sums and the forward's alpha_sum are rounded differently whatever the
+ * kernels; the dq formula amplifies that by |alpha_kvw| / alpha_sum, which grows with the head width: 3.5e-5 on values of
+ * magnitude 1 at 128 channels.  The Python operators therefore take these entry points up to 64 channels.)
+ */
+int s2attn_ring_forward_step_upsample_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                                           const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_up_shape *shape, void *stream);
+
+int s2attn_ring_backward_pass1_upsample_plan(const void *k, const void *v, const void *q, const void *dy, const float *qdotk_max,
+                                             float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                                             const s2attn_plan *plan, const s2attn_ring_up_shape *shape, void *stream);
+
+int s2attn_ring_backward_pass2_upsample_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                             const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                             const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_up_shape *shape, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -83,6 +83,16 @@ RING_UP_CASES = [
 ]
 
 
+# up-sampling direction on grids with at least 32 input longitudes: with fp32 storage and ck == cv a multiple of 4 from 16 to 128
+# the three steps run on the band-staged matrix-core kernels
+RING_UP_BAND_CASES = [
+    ((6, 40), (11, 80), "equiangular", "equiangular", 0.6, (2, 6, 9, 50), [0, 13, 14, 40], 0),  # ratio 2, a one-column chunk, odd window
+    ((5, 32), (9, 96), "legendre-gauss", "equiangular", 0.7, (0, 9, 80, 16), [0, 16, 32], 1),  # ratio 3, halo padded past the poles
+    ((7, 48), (13, 96), "equiangular", "legendre-gauss", 0.25, (0, 13, 0, 96), [0, 12, 24, 36, 48], 0),  # short runs, the whole output grid local
+    ((6, 36), (6, 72), "equiangular", "equiangular", 7.0, (1, 4, 60, 7), [0, 18, 36], 0),  # every point sees every point, a seven-column window
+]
+
+
 def local_problem_upsample(case, batch=2, ck=5, cv=3, seed=0):
     """Global tensors plus one rank's local view in the scatter direction (psi keyed by input latitude): rows = the halo's input
     latitudes (pad rows past the poles are empty), entries restricted to the local output latitudes and re-based, output

@@ -166,7 +166,7 @@ def test_ring_ops_pass_opcheck_and_leave_state_alone_without_neighbors():
         ops.forward_ring_step(kc, vc, qd, st3["y_acc"], st3["alpha_sum"], st3["qdotk_max"], quad, col_l, roff_l, row_idx, Wi, p["pscale"], Wi - 1, 0, p["nlat_loc"], p["nlon_loc"], *split)
 
 
-from tests.ring_util import RING_UP_CASES, local_problem_upsample  # noqa: E402
+from tests.ring_util import RING_UP_BAND_CASES, RING_UP_CASES, local_problem_upsample  # noqa: E402
 
 
 @pytest.mark.parametrize("case", RING_UP_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
@@ -181,6 +181,20 @@ def test_upsample_ring_steps_against_oracle_and_dense_attention(case, dtype):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16], ids=["f32", "bf16", "f16"])
 def test_upsample_ring_steps_vector_load_paths(case, dtype, chan):
     _upsample_direction(case, dtype, *chan)
+
+
+@pytest.mark.parametrize("d", [16, 32, 40, 64], ids=lambda d: f"d{d}")
+@pytest.mark.parametrize("case", RING_UP_BAND_CASES, ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
+def test_upsample_ring_steps_on_the_band_staged_kernels(case, d, monkeypatch):
+    """Grids wide enough for the band-staged kernels (fp32, ck == cv): the same checks as everywhere else, with all three steps on
+    those kernels."""
+    from torch_harmonics_amd import ops
+
+    taken = []
+    real = ops._ring_takes_plan
+    monkeypatch.setattr(ops, "_ring_takes_plan", lambda *a: taken.append(real(*a)) or taken[-1])
+    _upsample_direction(case, torch.float32, d, d)
+    assert taken and all(taken)
 
 
 def _upsample_direction(case, dtype, ck, cv):

@@ -110,6 +110,9 @@ SYMBOLS = {
     "s2attn_ring_forward_step_plan": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass1_plan": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2_plan": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingShapeStruct), _vp]),
+    "s2attn_ring_forward_step_upsample_plan": (_int, [_vp] * 7 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingUpShapeStruct), _vp]),
+    "s2attn_ring_backward_pass1_upsample_plan": (_int, [_vp] * 9 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingUpShapeStruct), _vp]),
+    "s2attn_ring_backward_pass2_upsample_plan": (_int, [_vp] * 10 + [ctypes.POINTER(PlanStruct), ctypes.POINTER(RingUpShapeStruct), _vp]),
     "s2attn_ring_backward_pass1": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_backward_pass2": (_int, [_vp] * 13 + [ctypes.POINTER(RingShapeStruct), _vp]),
     "s2attn_ring_regroup_psi": (_i64, [_vp, _vp, _int, _int, _int, _int, _vp, _vp, _vp, _vp]),

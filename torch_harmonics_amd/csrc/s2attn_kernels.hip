@@ -297,6 +297,9 @@ struct Args {
     // one ring step of the forward (ring_fwd_m32_kernel): the chunk's first real input longitude and latitude, its extents,
     // and the caller's running state
     int r_lon_lo, r_nkx, r_lat0, r_nlat;
+    int r_qps;   // nlon_out / nlon_in in the up-sampling direction (the plan's output latitudes are then virtual), else 1
+    int r_wo;    // local output longitudes
+    int r_wlat0; // quadrature weight of a run's input latitude Run::pad is quad_w[pad + r_wlat0]
     float *r_yacc, *r_asum, *r_qmax;
     float *r_integral, *r_ak, *r_akvw; // pass 1 of the backward
     const int2 *gspan; // per virtual output latitude: the arc of neighbor columns of query column 0 (see the plan)
@@ -2192,8 +2195,8 @@ enum Which { FWD, DQ, DKDV };
 
 template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream);
 template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream);
-template <int D, bool PASS1> int launch_ring_m32(const Args &a0, hipStream_t stream);
-template <int D> int launch_ring_pass2_m32(const Args &a0, hipStream_t stream);
+template <int D, int MODE> int launch_ring_m32(const Args &a0, hipStream_t stream);
+template <int D, bool WRITE> int launch_ring_pass2_m32(const Args &a0, hipStream_t stream);
 
 #if S2_PART == 0 || S2_PART == 2
 // 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
@@ -2278,42 +2281,50 @@ template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t
 #endif
 #if S2_PART == 0 || S2_PART == 3
 // one ring step (forward, or pass 1 of the backward) on the fp32 16-longitude kernels: one wavefront per 16 local output longitudes
-template <int D, bool PASS1> int launch_ring_m32(const Args &a0, hipStream_t stream)
+template <int D, int MODE> int launch_ring_m32(const Args &a0, hipStream_t stream)
 {
     Args a = a0;
     a.row_first = 0;
     const long nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    hipLaunchKernelGGL((ring_m32_kernel<D, PASS1>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL((ring_m32_kernel<D, MODE>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
 // pass 2 of a ring step: one wavefront per 16 virtual columns of a column class of a chunk latitude
-template <int D> int launch_ring_pass2_m32(const Args &a, hipStream_t stream)
+template <int D, bool WRITE> int launch_ring_pass2_m32(const Args &a, hipStream_t stream)
 {
     const int ntile = (a.r_nkx / a.kps + 1 + HQ - 1) / HQ + 1; // as in the kernel
     const long nblocks = (long)a.Hi * ntile * a.B;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    hipLaunchKernelGGL(ring_pass2_m32_kernel<D>, dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL((ring_pass2_m32_kernel<D, WRITE>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
 #endif
 #if S2_PART == 3
-template int launch_ring_pass2_m32<16>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<32>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<64>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<128>(const Args &, hipStream_t);
-template int launch_ring_m32<16, false>(const Args &, hipStream_t);
-template int launch_ring_m32<32, false>(const Args &, hipStream_t);
-template int launch_ring_m32<64, false>(const Args &, hipStream_t);
-template int launch_ring_m32<128, false>(const Args &, hipStream_t);
-template int launch_ring_m32<16, true>(const Args &, hipStream_t);
-template int launch_ring_m32<32, true>(const Args &, hipStream_t);
-template int launch_ring_m32<64, true>(const Args &, hipStream_t);
-template int launch_ring_m32<128, true>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, false>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, true>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 0>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 1>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 2>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, false>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, true>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 0>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 1>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 2>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, false>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, true>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 0>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 1>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 2>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, false>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, true>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 0>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 1>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 2>(const Args &, hipStream_t);
 template int launch_m32<16, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<32, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<64, 1>(Which, const Args &, hipStream_t);
@@ -2643,29 +2654,35 @@ extern "C" int s2attn_forward_lse(const void *k, const void *v, const void *q, c
     return launch(FWD, a, shape->dtype, vec, plan->header[S2ATTN_PH_GATHER_NDENSE], static_cast<hipStream_t>(stream));
 }
 
-// Ring steps on the band-staged kernels (ring_m32_kernel): checks and kernel arguments shared by the forward step and pass 1.
+// Ring steps on the band-staged kernels (ring_m32_kernel, ring_pass2_m32_kernel): checks and kernel arguments shared by the
+// six entry points.  The two directions differ in what the plan's latitudes mean: gather direction - input latitudes global
+// (the chunk holds r_lat0 .. + r_nlat of them), output longitudes nlon_in / pscale on the circle, of which nlon_out are
+// local; up-sampling direction - input latitudes are the chunk's rows as they stand, the plan's output latitudes are
+// virtual (nlat_out * pscale_out of them, nlon_in columns each).
 namespace {
-int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, const s2attn_plan *plan,
-                   const s2attn_ring_shape *sh)
+struct RingGeo {
+    int batch, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, cv, dtype, lon_lo_kx, lat_halo_start;
+    int nlon_in, kps, qps; // global input longitudes; nlon_in / nlon_out_global and its inverse, one of them 1
+};
+int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const void *dy, const float *quad_weights, const s2attn_plan *plan, const RingGeo &g)
 {
-    if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "ring shape is null");
-    if (sh->batch < 1 || sh->nlat_halo < 1 || sh->nlon_kx < 1 || sh->nlat_out < 1 || sh->nlon_out < 1 || sh->nlon_in < 1)
+    if (g.batch < 1 || g.nlat_halo < 1 || g.nlon_kx < 1 || g.nlat_out < 1 || g.nlon_out < 1 || g.nlon_in < 1)
         return s2attn_fail(S2ATTN_E_INVALID, "batch and grid extents must be positive");
-    if (sh->pscale < 1 || sh->nlon_in % sh->pscale != 0)
-        return s2attn_fail(S2ATTN_E_INVALID, "pscale must be a positive divisor of nlon_in = %d, got %d", sh->nlon_in, sh->pscale);
-    if (sh->lon_lo_kx < 0 || sh->lon_lo_kx + sh->nlon_kx > sh->nlon_in)
-        return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", sh->lon_lo_kx, sh->lon_lo_kx + sh->nlon_kx, sh->nlon_in);
-    const int W = sh->nlon_in / sh->pscale; // global output longitudes = columns of a virtual input latitude
-    if (sh->nlon_out > W) return s2attn_fail(S2ATTN_E_INVALID, "pscale * nlon_out = %ld exceeds nlon_in = %d", (long)sh->pscale * sh->nlon_out, sh->nlon_in);
+    if (g.lon_lo_kx < 0 || g.lon_lo_kx + g.nlon_kx > g.nlon_in)
+        return s2attn_fail(S2ATTN_E_INVALID, "chunk [%d, %d) leaves the input grid of %d longitudes", g.lon_lo_kx, g.lon_lo_kx + g.nlon_kx, g.nlon_in);
+    const int W = g.nlon_in / g.kps;                    // columns of a (virtual) latitude of the plan
+    const int wout = g.qps > 1 ? g.nlon_in * g.qps : W; // global output longitudes
+    if (g.nlon_out > wout) return s2attn_fail(S2ATTN_E_INVALID, "%d local output longitudes on a grid of %d", g.nlon_out, wout);
     if (!k || !v || !q || !quad_weights) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!plan || !plan->data) return s2attn_fail(S2ATTN_E_INVALID, "plan is null");
     const int32_t *h = plan->header;
     if (h[S2ATTN_PH_MAGIC] != S2ATTN_PLAN_MAGIC) return s2attn_fail(S2ATTN_E_INVALID, "plan header does not carry this library's plan format");
-    if (h[S2ATTN_PH_NLON_IN] != sh->nlon_in || h[S2ATTN_PH_NLAT_OUT] != sh->nlat_out || h[S2ATTN_PH_NLON_OUT] != W)
-        return s2attn_fail(S2ATTN_E_INVALID, "plan was built for %d input longitudes and %dx%d output points, the step is for %d and %dx%d (global longitudes)",
-                           h[S2ATTN_PH_NLON_IN], h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], sh->nlon_in, sh->nlat_out, W);
-    if (sh->dtype != S2ATTN_F32 || !m32_width(sh->ck, sh->cv) || sh->ck > 128 || W < HK)
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take fp32 tensors with ck = cv a multiple of 4 from 16 to 128 and at least %d global output longitudes", HK);
+    if (h[S2ATTN_PH_NLON_IN] != g.nlon_in || h[S2ATTN_PH_NLAT_OUT] != g.nlat_out || h[S2ATTN_PH_NLON_OUT] != wout || (g.qps > 1 && h[S2ATTN_PH_NLAT_IN] != g.nlat_halo))
+        return s2attn_fail(S2ATTN_E_INVALID, "plan was built for grids %dx%d -> %dx%d, the step needs %s x%d -> %dx%d (local latitudes, global longitudes)",
+                           h[S2ATTN_PH_NLAT_IN], h[S2ATTN_PH_NLON_IN], h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], g.qps > 1 ? "the chunk's latitudes" : "all input latitudes",
+                           g.nlon_in, g.nlat_out, wout);
+    if (g.dtype != S2ATTN_F32 || !m32_width(g.ck, g.cv) || g.ck > 128 || W < HK)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take fp32 tensors with ck = cv a multiple of 4 from 16 to 128 on at least %d longitudes", HK);
     const void *ptrs[] = {k, v, q, dy};
     for (const void *p : ptrs)
         if (p && !aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
@@ -2681,50 +2698,103 @@ int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const v
     a.sruns = reinterpret_cast<const Run *>(d + h[S2ATTN_PH_SCATTER_RUNS]);
     a.sorder = d + h[S2ATTN_PH_SCATTER_ORDER];
     a.k = k, a.v = v, a.q = q, a.dy = dy;
-    a.B = sh->batch, a.nh = 1, a.kps = sh->pscale, a.qps = 1;
-    a.Hi = h[S2ATTN_PH_NLAT_IN] * sh->pscale, a.Wi = W;
-    a.Ho = sh->nlat_out, a.Wo = sh->nlon_out; // local output points; runs are relative to local column 0
-    a.dk_ = a.dv_ = sh->ck;
-    a.r_lon_lo = sh->lon_lo_kx, a.r_nkx = sh->nlon_kx, a.r_lat0 = sh->lat_halo_start, a.r_nlat = sh->nlat_halo;
+    a.B = g.batch, a.nh = 1, a.kps = g.kps, a.qps = 1;
+    a.Hi = h[S2ATTN_PH_NLAT_IN] * g.kps, a.Wi = W;
+    a.Ho = g.nlat_out * g.qps;                   // (virtual) output latitudes of the plan
+    a.Wo = (g.nlon_out + g.qps - 1) / g.qps;     // columns of one of them that can be local: the tiles' domain
+    a.r_qps = g.qps, a.r_wo = g.nlon_out;
+    a.dk_ = a.dv_ = g.ck;
+    a.r_lon_lo = g.lon_lo_kx, a.r_nkx = g.nlon_kx, a.r_nlat = g.nlat_halo;
+    a.r_lat0 = g.qps > 1 ? 0 : g.lat_halo_start;   // the plan's input latitude of the chunk's row 0
+    a.r_wlat0 = g.qps > 1 ? g.lat_halo_start : 0;  // the plan's input latitude -> index of its quadrature weight
     return S2ATTN_OK;
 }
-template <bool PASS1> int launch_ring_plan(const Args &a, hipStream_t st)
+int ring_geo(RingGeo &g, const s2attn_ring_shape *sh)
 {
-    if (a.dk_ <= 16) return launch_ring_m32<16, PASS1>(a, st);
-    if (a.dk_ <= 32) return launch_ring_m32<32, PASS1>(a, st);
-    if (a.dk_ <= 64) return launch_ring_m32<64, PASS1>(a, st);
-    return launch_ring_m32<128, PASS1>(a, st);
+    if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "ring shape is null");
+    if (sh->pscale < 1 || sh->nlon_in < 1 || sh->nlon_in % sh->pscale != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "pscale must be a positive divisor of nlon_in = %d, got %d", sh->nlon_in, sh->pscale);
+    g = RingGeo{sh->batch, sh->nlat_halo, sh->nlon_kx, sh->nlat_out, sh->nlon_out, sh->ck, sh->cv, sh->dtype, sh->lon_lo_kx, sh->lat_halo_start, sh->nlon_in, sh->pscale, 1};
+    return S2ATTN_OK;
+}
+int ring_geo(RingGeo &g, const s2attn_ring_up_shape *sh)
+{
+    if (!sh) return s2attn_fail(S2ATTN_E_INVALID, "ring shape is null");
+    if (sh->pscale_out < 1 || sh->nlon_out_global < 1 || sh->nlon_out_global % sh->pscale_out != 0)
+        return s2attn_fail(S2ATTN_E_INVALID, "pscale_out must be a positive divisor of nlon_out_global = %d, got %d", sh->nlon_out_global, sh->pscale_out);
+    g = RingGeo{sh->batch, sh->nlat_halo, sh->nlon_kx, sh->nlat_out, sh->nlon_out, sh->ck, sh->cv, sh->dtype, sh->lon_lo_kx, sh->lat_halo_start,
+                sh->nlon_out_global / sh->pscale_out, 1, sh->pscale_out};
+    return S2ATTN_OK;
+}
+template <int MODE> int launch_ring_plan(const Args &a, hipStream_t st)
+{
+    if (a.dk_ <= 16) return launch_ring_m32<16, MODE>(a, st);
+    if (a.dk_ <= 32) return launch_ring_m32<32, MODE>(a, st);
+    if (a.dk_ <= 64) return launch_ring_m32<64, MODE>(a, st);
+    return launch_ring_m32<128, MODE>(a, st);
+}
+template <bool WRITE> int launch_ring_pass2_plan(const Args &a, hipStream_t st)
+{
+    if (a.dk_ <= 16) return launch_ring_pass2_m32<16, WRITE>(a, st);
+    if (a.dk_ <= 32) return launch_ring_pass2_m32<32, WRITE>(a, st);
+    if (a.dk_ <= 64) return launch_ring_pass2_m32<64, WRITE>(a, st);
+    return launch_ring_pass2_m32<128, WRITE>(a, st);
+}
+template <typename SHAPE>
+int ring_forward_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max, const float *quad_weights,
+                      const s2attn_plan *plan, const SHAPE *sh, void *stream)
+{
+    Args a = {};
+    RingGeo g;
+    int rc = ring_geo(g, sh);
+    if (rc == S2ATTN_OK) rc = ring_plan_args(a, k, v, q, nullptr, quad_weights, plan, g);
+    if (rc != S2ATTN_OK) return rc;
+    if (!y_acc || !alpha_sum || !qdotk_max) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!aligned(y_acc, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
+    a.r_yacc = y_acc, a.r_asum = alpha_sum, a.r_qmax = qdotk_max;
+    return launch_ring_plan<0>(a, static_cast<hipStream_t>(stream));
+}
+template <typename SHAPE, bool WRITE>
+int ring_pass2_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum, const float *qdotk_max, const float *integral_norm,
+                    float *dk, float *dv, const float *quad_weights, const s2attn_plan *plan, const SHAPE *sh, void *stream)
+{
+    Args a = {};
+    RingGeo g;
+    int rc = ring_geo(g, sh);
+    if (rc == S2ATTN_OK) rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, g);
+    if (rc != S2ATTN_OK) return rc;
+    if (!dy || !alpha_sum || !qdotk_max || !integral_norm || !dk || !dv) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!aligned(dk, 16) || !aligned(dv, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
+    a.r_asum = const_cast<float *>(alpha_sum), a.r_qmax = const_cast<float *>(qdotk_max), a.r_integral = const_cast<float *>(integral_norm);
+    a.dk = dk, a.dv = dv;
+    return launch_ring_pass2_plan<WRITE>(a, static_cast<hipStream_t>(stream));
 }
 } // namespace
 
 extern "C" int s2attn_ring_forward_step_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
                                              const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
 {
-    Args a = {};
-    const int rc = ring_plan_args(a, k, v, q, nullptr, quad_weights, plan, sh);
-    if (rc != S2ATTN_OK) return rc;
-    if (!y_acc || !alpha_sum || !qdotk_max) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
-    if (!aligned(y_acc, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
-    a.r_yacc = y_acc, a.r_asum = alpha_sum, a.r_qmax = qdotk_max;
-    return launch_ring_plan<false>(a, static_cast<hipStream_t>(stream));
+    return ring_forward_plan(k, v, q, y_acc, alpha_sum, qdotk_max, quad_weights, plan, sh, stream);
+}
+
+extern "C" int s2attn_ring_forward_step_upsample_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max,
+                                                      const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_up_shape *sh, void *stream)
+{
+    return ring_forward_plan(k, v, q, y_acc, alpha_sum, qdotk_max, quad_weights, plan, sh, stream);
 }
 
 extern "C" int s2attn_ring_backward_pass2_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
                                                const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
                                                const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
 {
-    Args a = {};
-    const int rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, sh);
-    if (rc != S2ATTN_OK) return rc;
-    if (!dy || !alpha_sum || !qdotk_max || !integral_norm || !dk || !dv) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
-    if (!aligned(dk, 16) || !aligned(dv, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
-    a.r_asum = const_cast<float *>(alpha_sum), a.r_qmax = const_cast<float *>(qdotk_max), a.r_integral = const_cast<float *>(integral_norm);
-    a.dk = dk, a.dv = dv;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    if (a.dk_ <= 16) return launch_ring_pass2_m32<16>(a, st);
-    if (a.dk_ <= 32) return launch_ring_pass2_m32<32>(a, st);
-    if (a.dk_ <= 64) return launch_ring_pass2_m32<64>(a, st);
-    return launch_ring_pass2_m32<128>(a, st);
+    return ring_pass2_plan<s2attn_ring_shape, false>(k, v, q, dy, alpha_sum, qdotk_max, integral_norm, dk, dv, quad_weights, plan, sh, stream);
+}
+
+extern "C" int s2attn_ring_backward_pass2_upsample_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum,
+                                                        const float *qdotk_max, const float *integral_norm, float *dk, float *dv,
+                                                        const float *quad_weights, const s2attn_plan *plan, const s2attn_ring_up_shape *sh, void *stream)
+{
+    return ring_pass2_plan<s2attn_ring_up_shape, true>(k, v, q, dy, alpha_sum, qdotk_max, integral_norm, dk, dv, quad_weights, plan, sh, stream);
 }
 
 extern "C" int s2attn_ring_backward_pass1_plan(const void *k, const void *v, const void *q, const void *dy, float *alpha_sum, float *qdotk_max,
@@ -2732,12 +2802,29 @@ extern "C" int s2attn_ring_backward_pass1_plan(const void *k, const void *v, con
                                                const s2attn_plan *plan, const s2attn_ring_shape *sh, void *stream)
 {
     Args a = {};
-    const int rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, sh);
+    RingGeo g;
+    int rc = ring_geo(g, sh);
+    if (rc == S2ATTN_OK) rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, g);
     if (rc != S2ATTN_OK) return rc;
     if (!dy || !alpha_sum || !qdotk_max || !integral || !alpha_k || !alpha_kvw) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!aligned(alpha_k, 16) || !aligned(alpha_kvw, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_asum = alpha_sum, a.r_qmax = qdotk_max, a.r_integral = integral, a.r_ak = alpha_k, a.r_akvw = alpha_kvw;
-    return launch_ring_plan<true>(a, static_cast<hipStream_t>(stream));
+    return launch_ring_plan<1>(a, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int s2attn_ring_backward_pass1_upsample_plan(const void *k, const void *v, const void *q, const void *dy, const float *qdotk_max,
+                                                        float *integral, float *alpha_k, float *alpha_kvw, const float *quad_weights,
+                                                        const s2attn_plan *plan, const s2attn_ring_up_shape *sh, void *stream)
+{
+    Args a = {};
+    RingGeo g;
+    int rc = ring_geo(g, sh);
+    if (rc == S2ATTN_OK) rc = ring_plan_args(a, k, v, q, dy, quad_weights, plan, g);
+    if (rc != S2ATTN_OK) return rc;
+    if (!dy || !qdotk_max || !integral || !alpha_k || !alpha_kvw) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
+    if (!aligned(alpha_k, 16) || !aligned(alpha_kvw, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
+    a.r_qmax = const_cast<float *>(qdotk_max), a.r_integral = integral, a.r_ak = alpha_k, a.r_akvw = alpha_kvw;
+    return launch_ring_plan<2>(a, static_cast<hipStream_t>(stream));
 }
 
 namespace {

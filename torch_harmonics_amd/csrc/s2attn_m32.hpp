@@ -571,7 +571,7 @@ struct RingWalk {
     const Run *runs;
     const float *weights;
     int ri, rend;
-    int W, kps, w0, lon_lo, nkx, lat0, nlat;
+    int W, kps, w0, lon_lo, nkx, lat0, nlat, wlat0; // wlat0: quadrature weight of the run's latitude Run::pad is weights[pad + wlat0]
     // the run the walk stands in
     Run run;
     float w;
@@ -605,7 +605,7 @@ struct RingWalk {
                     nv = (lon_lo + nkx - par + kps - 1) / kps - vlo; // virtual columns vlo .. vlo + nv are in the chunk
                     if (nv <= 0) continue;
                 }
-                w = uniform_load(weights + run.pad);
+                w = uniform_load(weights + (run.pad + wlat0));
                 L = run.len + HQ - 1;
                 u0 = vlo - run.ws - w0; // in (-2 W, W)
                 u0 += (u0 < 0) ? W : 0;
@@ -622,25 +622,35 @@ struct RingWalk {
     }
 };
 
-// PASS1 = false: the forward step (state y_acc, alpha_sum, qdotk_max).  PASS1 = true: pass 1 of the backward, which walks
-// the same steps and re-accumulates alpha_sum and qdotk_max (the same operations in the same order as the forward step:
-// the two sums are bit-identical) together with integral = sum_j alpha_j <dy, v_j>, alpha_k = sum_j alpha_j k_j and
-// alpha_kvw = sum_j alpha_j <dy, v_j> k_j: a second score product G^T = V dY^T and two accumulations against K^T.
-template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1) ? 4 : (D <= 32 ? 3 : (D <= 64 && !PASS1 ? 2 : 1))) void ring_m32_kernel(const Args a)
+// MODE 0: the forward step (state y_acc, alpha_sum, qdotk_max).  MODE 1: pass 1 of the backward in the gather direction,
+// which walks the same steps and re-accumulates alpha_sum and qdotk_max (the same operations in the same order as the
+// forward step: the two sums are bit-identical) together with integral = sum_j alpha_j <dy, v_j>, alpha_k = sum_j alpha_j k_j
+// and alpha_kvw = sum_j alpha_j <dy, v_j> k_j: a second score product G^T = V dY^T and two accumulations against K^T.
+// MODE 2: pass 1 of the up-sampling direction, which is handed the forward's FINAL qdotk_max and adds the same three sums
+// relative to it (no running maximum, no alpha_sum).
+// Both directions: in the up-sampling direction (r_qps = nlon_out / nlon_in > 1) the plan's output latitudes are virtual
+// (real latitude * r_qps + column class), a tile's queries are the local output columns (w0 + c) * r_qps + class, input
+// latitudes are rows of the chunk as they stand and r_wlat0 turns them into quadrature-weight indices.
+template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 0) ? 4 : (D <= 32 ? 3 : (D <= 64 && MODE == 0 ? 2 : 1))) void ring_m32_kernel(const Args a)
 {
     constexpr int NS = 1;
+    constexpr bool PASS1 = MODE != 0, FIXED = MODE == 2;
     typedef FTile<D> Tile;
     constexpr int PITCH = Tile::PITCH, NCB = D / 16;
     S2_M32_IDS(a.Wo, a.Ho)
     (void)h; // heads are folded into the batch
+    (void)nvalid;
     char *lds = m32_lds<m32_lds_bytes<D, 1>(false), 1>();
     char *Ks = lds, *Vs = Ks + HK * PITCH;
-    const int ho = a.gorder[a.row_first + rowsel];
+    const int ho = a.gorder[a.row_first + rowsel]; // (virtual) output latitude
+    const int hor = ho / a.r_qps, parq = ho - hor * a.r_qps;
+    const int nval = min(HQ, (a.r_wo - parq + a.r_qps - 1) / a.r_qps - w0); // queries of the tile inside the local window
+    if (nval <= 0) return;
     const unsigned ldb = drt * 4; // bytes between two grid points
     const char *kx = static_cast<const char *>(a.k) + (size_t)b * a.r_nlat * a.r_nkx * ldb;
     const char *vx = static_cast<const char *>(a.v) + (size_t)b * a.r_nlat * a.r_nkx * ldb;
-    const bool mine = c < nvalid;
-    const size_t pt = ((size_t)b * a.Ho + ho) * a.Wo + w0 + (mine ? c : 0);
+    const bool mine = c < nval;
+    const size_t pt = ((size_t)b * (a.Ho / a.r_qps) + hor) * a.r_wo + (size_t)(w0 + (mine ? c : 0)) * a.r_qps + parq;
 
     { // the arc of columns this tile's queries can see, against the virtual columns that can lie in the chunk: most tiles of
       // an equatorial latitude leave here, without reading a run
@@ -655,7 +665,7 @@ template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1
         }
     }
     RingWalk wk;
-    wk.W = a.Wi, wk.kps = a.kps, wk.w0 = w0, wk.lon_lo = a.r_lon_lo, wk.nkx = a.r_nkx, wk.lat0 = a.r_lat0, wk.nlat = a.r_nlat;
+    wk.W = a.Wi, wk.kps = a.kps, wk.w0 = w0, wk.lon_lo = a.r_lon_lo, wk.nkx = a.r_nkx, wk.lat0 = a.r_lat0, wk.nlat = a.r_nlat, wk.wlat0 = a.r_wlat0;
     wk.start(a.gruns, a.quad_w, a.goff[ho], a.goff[ho + 1]);
     if (!wk.advance()) return; // nothing of this tile's neighborhood is in the chunk
 
@@ -680,8 +690,8 @@ template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1
     // between the four lanes of a column nor a rescaling); the exact maximum the state asks for is kept per lane (mtrue)
     // and the sums are brought to it once, at the end.
     float m = fmaxf(a.r_qmax[pt], NEG_BIG_NAT), mtrue = -INFINITY;
-    float S = qd == 0 ? a.r_asum[pt] : 0.f; // the four lanes of a column each keep a share of the sums
-    float I = 0.f;
+    float S = 0.f, I = 0.f; // the four lanes of a column each keep a share of the sums
+    if constexpr (!FIXED) S = qd == 0 ? a.r_asum[pt] : 0.f;
     if constexpr (PASS1) I = qd == 0 ? a.r_integral[pt] : 0.f;
 
     Tile kt, vt;
@@ -741,9 +751,9 @@ template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1
                 }
             }
         }
-        mtrue = fmaxf(mtrue, mx);
+        if constexpr (!FIXED) mtrue = fmaxf(mtrue, mx);
         constexpr float THR = RESCALE_THR * 0.69314718f; // natural units
-        if (__any(mx > m + THR)) {
+        if (!FIXED && __any(mx > m + THR)) {
             const float cm = h16_quarter_max(mx);
             const float mn = cm > m + THR ? cm : m; // m is finite, so mn is
             const float corr = fast_exp2((m - mn) * LOG2E);
@@ -787,12 +797,17 @@ template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1
 
     S = h16_quarter_sum(S);
     if constexpr (PASS1) I = h16_quarter_sum(I);
-    mtrue = fmaxf(h16_quarter_max(mtrue), a.r_qmax[pt]); // the maximum over everything this column has seen, earlier chunks included (read again: a register less in the loop)
-    const float f = mtrue > -INFINITY ? fast_exp2((m - mtrue) * LOG2E) : 1.f; // m <= mtrue <= m + THR; a column without neighbors keeps its zeros
+    float f = 1.f;
+    if constexpr (!FIXED) {
+        mtrue = fmaxf(h16_quarter_max(mtrue), a.r_qmax[pt]); // the maximum over everything this column has seen, earlier chunks included (read again: a register less in the loop)
+        f = mtrue > -INFINITY ? fast_exp2((m - mtrue) * LOG2E) : 1.f; // m <= mtrue <= m + THR; a column without neighbors keeps its zeros
+    }
     if (mine) {
         if (qd == 0) {
-            a.r_asum[pt] = S * f;
-            a.r_qmax[pt] = mtrue;
+            if constexpr (!FIXED) {
+                a.r_asum[pt] = S * f;
+                a.r_qmax[pt] = mtrue;
+            }
             if constexpr (PASS1) a.r_integral[pt] = I * f;
         }
 #pragma unroll
@@ -812,7 +827,10 @@ template <int D, bool PASS1> __global__ __launch_bounds__(64, (D <= 32 && !PASS1
 // local queries with their statistics (alpha_sum, qdotk_max, integral_norm of the caller, natural units) - a row whose query
 // column lies outside the local window of Wo longitudes is staged as zeros and weighs nothing.  dk, dv (fp32, shaped like
 // the chunk) are ADDED to; every key belongs to one wavefront, so plainly.
-template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(const Args a)
+// WRITE = false (gather direction): dk, dv are added to.  WRITE = true (up-sampling direction: r_qps > 1, the plan's output
+// latitudes are virtual, a staged row of virtual column j is the local query column j * r_qps + class): every element of
+// the chunk's dk, dv is written, zeros where no query sees the key.
+template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(const Args a)
 {
     typedef FTile<D> Tile;
     constexpr int PITCH = Tile::PITCH, NCB = D / 16;
@@ -830,19 +848,32 @@ template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(con
     const int w0 = vlo + HQ * tile; // first virtual column of the tile
     const int nvalid = min(HQ, vlo + nv - w0);
     if (nvalid <= 0) return;
+    const bool mine = c < nvalid;
+    const size_t pt = ((size_t)b * a.r_nlat + rl) * a.r_nkx + (size_t)((w0 + (mine ? c : 0)) * a.kps + par - a.r_lon_lo); // the key in the chunk
     int ri = a.soff[hv];
     const int rend = a.soff[hv + 1];
-    if (ri >= rend) return; // no query sees this latitude
+    if (ri >= rend) { // no query sees this latitude
+        if (WRITE && mine) {
+            float *dk = static_cast<float *>(a.dk) + pt * drt + 4 * qd, *dv = static_cast<float *>(a.dv) + pt * drt + 4 * qd;
+#pragma unroll
+            for (int cb = 0; cb < NCB; cb++) {
+                if (16 * cb + 4 * qd < dr) {
+                    *reinterpret_cast<float4 *>(dk + 16 * cb) = make_float4(0.f, 0.f, 0.f, 0.f);
+                    *reinterpret_cast<float4 *>(dv + 16 * cb) = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
+        }
+        return;
+    }
 
     char *lds = m32_lds<m32_lds_bytes<D, 1>(true), 1>();
     char *Qs = lds, *Gs = Qs + HK * PITCH;
     float *Ls = reinterpret_cast<float *>(Gs + HK * PITCH), *Is = Ls + HK;
     const unsigned ldb = drt * 4; // bytes between two grid points
-    const char *qy = static_cast<const char *>(a.q) + (size_t)b * a.Ho * a.Wo * ldb;
-    const char *gy = static_cast<const char *>(a.dy) + (size_t)b * a.Ho * a.Wo * ldb;
-    const size_t sbase = (size_t)b * a.Ho * a.Wo;
-    const bool mine = c < nvalid;
-    const size_t pt = ((size_t)b * a.r_nlat + rl) * a.r_nkx + (size_t)((w0 + (mine ? c : 0)) * a.kps + par - a.r_lon_lo); // the key in the chunk
+    const int Hor = a.Ho / a.r_qps; // real local output latitudes
+    const size_t sbase = (size_t)b * Hor * a.r_wo;
+    const char *qy = static_cast<const char *>(a.q) + sbase * ldb;
+    const char *gy = static_cast<const char *>(a.dy) + sbase * ldb;
 
     float kop[D / 4], vop[D / 4]; // this lane's quarter of key c
     m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + pt * ldb, qd, dr);
@@ -853,7 +884,7 @@ template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(con
         dkt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
         dvt[cb] = f4v{0.f, 0.f, 0.f, 0.f};
     }
-    const float lw = fast_log2(a.quad_w[hreal]);
+    const float lw = fast_log2(a.quad_w[hreal + a.r_wlat0]);
 
     int pos = 0;
     Run run = {0, 0, 0, 0};
@@ -863,16 +894,20 @@ template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(con
     const unsigned pc = 16u * (lane % Tile::CPR);
     const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
     auto fetch = [&](const Run &rn, int p) {
-        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wi; // query column of staged row 0, on the circle of the global output longitudes
+        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wi; // (virtual) query column of staged row 0, on the circle of a.Wi columns
         c0 += (c0 < 0) ? a.Wi : 0;
-        const size_t lat = (size_t)rn.lat * a.Wo; // local output latitude
+        // the run's output latitude is virtual (real latitude Run::pad, column class parq): virtual column j is the local
+        // query column j * r_qps + parq
+        const int parq = rn.lat - rn.pad * a.r_qps;
+        const size_t lat = (size_t)rn.pad * a.r_wo + parq;
 #pragma unroll
         for (int it = 0; it < Tile::NIT; it++) {
             int col = c0 + r0 + it * Tile::RPI;
             col -= (col >= a.Wi) ? a.Wi : 0;
+            col *= a.r_qps;
             qt.raw[it] = u4v{0u, 0u, 0u, 0u};
             gt.raw[it] = u4v{0u, 0u, 0u, 0u};
-            if (col < a.Wo && piece_ok) { // inside the local window
+            if (col + parq < a.r_wo && piece_ok) { // inside the local window
                 qt.raw[it] = *reinterpret_cast<const u4v *>(qy + (lat + col) * ldb + pc);
                 gt.raw[it] = *reinterpret_cast<const u4v *>(gy + (lat + col) * ldb + pc);
             }
@@ -880,8 +915,9 @@ template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(con
         if (lane < HK) { // lanes 0..31 fetch the statistics of the staged rows: (log2-sum-exp, integral_norm)
             int col = c0 + lane;
             col -= (col >= a.Wi) ? a.Wi : 0;
+            col *= a.r_qps;
             st = make_float2(INFINITY, 0.f); // a row outside the window weighs exp2(-inf) = 0
-            if (col < a.Wo) {
+            if (col + parq < a.r_wo) {
                 const size_t s = sbase + lat + col;
                 const float as = a.r_asum[s];
                 if (as > 0.f) st = make_float2(fmaf(a.r_qmax[s], LOG2E, fast_log2(as)), a.r_integral[s]); // (a query that saw nothing weighs nothing)
@@ -950,7 +986,8 @@ template <int D> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(con
 #pragma unroll
         for (int cb = 0; cb < NCB; cb++) {
             if (16 * cb + 4 * qd < dr) {
-                float4 x = *reinterpret_cast<const float4 *>(dk + 16 * cb), y = *reinterpret_cast<const float4 *>(dv + 16 * cb);
+                float4 x = make_float4(0.f, 0.f, 0.f, 0.f), y = x;
+                if (!WRITE) x = *reinterpret_cast<const float4 *>(dk + 16 * cb), y = *reinterpret_cast<const float4 *>(dv + 16 * cb);
                 x.x += dkt[cb][0], x.y += dkt[cb][1], x.z += dkt[cb][2], x.w += dkt[cb][3];
                 y.x += dvt[cb][0], y.y += dvt[cb][1], y.z += dvt[cb][2], y.w += dvt[cb][3];
                 *reinterpret_cast<float4 *>(dk + 16 * cb) = x;

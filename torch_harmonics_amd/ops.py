@@ -252,12 +252,15 @@ def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out
     return _lib.RingShapeStruct(B, nlat_halo, nlon_kx, nlat_out, nlon_out, ck, vx.shape[3], nlon_in, pscale, lon_lo_kx, lat_halo_start, _DTYPE_CODE[qy.dtype])
 
 
-def _ring_takes_plan(kx, vx, qy, nlon_in, pscale) -> bool:
+def _ring_takes_plan(kx, vx, qy, nlon_in, pscale, max_ck=128) -> bool:
     """Shapes of the band-staged ring steps (s2attn_ring_forward_step_plan, s2attn_ring_backward_pass1_plan / pass2_plan in include/s2attn.h).
     Decided by the shape alone, so that the forward step and pass 1 of one problem always run the same formulation (their
-    alpha_sum are then bit-identical; the state buffers are fresh torch allocations, 16-byte aligned like every tensor)."""
+    alpha_sum are then bit-identical; the state buffers are fresh torch allocations, 16-byte aligned like every tensor).
+    The up-sampling direction stops at 64 channels (max_ck): its pass 1 works from the forward's FINAL maximum, so its sums and
+    the forward's alpha_sum are rounded differently whatever the kernels, and the dq formula that combines them amplifies that
+    by |alpha_kvw| / alpha_sum, which grows with the head width (3.5e-5 on values of magnitude 1 at 128 channels)."""
     ck, cv = kx.shape[3], vx.shape[3]
-    if qy.dtype != torch.float32 or ck != cv or ck % 4 or not 16 <= ck <= 128 or nlon_in // pscale < 32:
+    if qy.dtype != torch.float32 or ck != cv or ck % 4 or not 16 <= ck <= max_ck or nlon_in // pscale < 32:
         return False
     return True
 
@@ -496,6 +499,16 @@ def forward_ring_step_upsample(
     if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    if _ring_takes_plan(kx, vx, qy, nlon_in, 1, 64) and all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, y_acc)):
+        # band-staged matrix-core step on the run-length plan of the local psi (rows = the chunk's latitudes)
+        p = _plan.get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out_global)
+        with torch.cuda.device(kx.device):
+            rc = _lib.load().s2attn_ring_forward_step_upsample_plan(
+                kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), y_acc.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(),
+                quad_weights.data_ptr(), ctypes.byref(p.struct), ctypes.byref(shape), _stream_ptr(kx.device),
+            )  # fmt: skip
+        _lib.check(rc, "s2attn_ring_forward_step_upsample_plan")
+        return
     with torch.cuda.device(kx.device):
         t_lat, t_lon, t_off, _ = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)  # psi regrouped by output latitude
         rc = _lib.load().s2attn_ring_forward_step_upsample(
@@ -537,6 +550,15 @@ def backward_ring_step_upsample_pass1(
     if qy.numel() == 0 or kx.numel() == 0 or col_idx.numel() == 0:
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    if _ring_takes_plan(kx, vx, qy, nlon_in, 1, 64) and all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, dy, alpha_k_buf, alpha_kvw_buf)):
+        p = _plan.get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out_global)
+        with torch.cuda.device(kx.device):
+            rc = _lib.load().s2attn_ring_backward_pass1_upsample_plan(
+                kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), qdotk_max_buf.data_ptr(), integral_buf.data_ptr(), alpha_k_buf.data_ptr(),
+                alpha_kvw_buf.data_ptr(), quad_weights.data_ptr(), ctypes.byref(p.struct), ctypes.byref(shape), _stream_ptr(kx.device),
+            )  # fmt: skip
+        _lib.check(rc, "s2attn_ring_backward_pass1_upsample_plan")
+        return
     with torch.cuda.device(kx.device):
         t_lat, t_lon, t_off, _ = get_transposed_csr(col_idx, row_off, nlon_out_global, 0, nlat_out)
         rc = _lib.load().s2attn_ring_backward_pass1_upsample(
@@ -586,6 +608,15 @@ def backward_ring_step_upsample_pass2(
         dvx.zero_()
         return
     shape = _ring_up_shape(kx, vx, qy, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out)
+    if _ring_takes_plan(kx, vx, qy, nlon_in, 1, 64) and all(t.data_ptr() % 16 == 0 for t in (kx, vx, qy, dy, dkx, dvx)):
+        p = _plan.get_plan(col_idx, row_off, kx.shape[1], nlon_in, nlat_out, nlon_out_global)
+        with torch.cuda.device(kx.device):
+            rc = _lib.load().s2attn_ring_backward_pass2_upsample_plan(
+                kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(), integral_norm_buf.data_ptr(),
+                dkx.data_ptr(), dvx.data_ptr(), quad_weights.data_ptr(), ctypes.byref(p.struct), ctypes.byref(shape), _stream_ptr(kx.device),
+            )  # fmt: skip
+        _lib.check(rc, "s2attn_ring_backward_pass2_upsample_plan")
+        return
     with torch.cuda.device(kx.device):
         rc = _lib.load().s2attn_ring_backward_pass2_upsample(
             kx.data_ptr(), vx.data_ptr(), qy.data_ptr(), dy.data_ptr(), alpha_sum_buf.data_ptr(), qdotk_max_buf.data_ptr(), integral_norm_buf.data_ptr(),
