@@ -134,16 +134,18 @@ def _gather_direction(case, dtype, ck, cv, monkeypatch):
         assert_close(f"dv (from_csr={from_csr})", dv, v.grad, **tol)
 
 
-def test_ring_ops_pass_opcheck_and_leave_state_alone_without_neighbors():
+@pytest.mark.parametrize("band", [False, True], ids=["gather_kernels", "band_staged_kernels"])
+def test_ring_ops_pass_opcheck_and_leave_state_alone_without_neighbors(band):
     from torch_harmonics_amd import ops
 
-    p = local_problem(RING_CASES[2])
+    p = local_problem(RING_BAND_CASES[1], ck=32, cv=32) if band else local_problem(RING_CASES[2])
     B, ck, cv, Wi = p["k"].shape[0], p["k"].shape[3], p["v"].shape[3], p["ins"][1]
     quad, col_l, roff_l, row_idx = _geo_dev(p)
     split = ops.split_csr_rows(p["row_idx"], p["roff_l"], p["nlat_loc"])
     qd, gd = p["q_l"].to(DEV), p["dy_l"].to(DEV)
     kc, vc = chunk_of(p, p["k"], 1).to(DEV), chunk_of(p, p["v"], 1).to(DEV)
     tail = (Wi, p["pscale"], p["chunks"][1][0], p["halo"][0], p["nlat_loc"], p["nlon_loc"], *split)
+    assert ops._ring_takes_plan(kc, vc, qd, Wi, p["pscale"]) == band
     st = fresh_state(B, p["nlat_loc"], p["nlon_loc"], ck, cv, torch.float32, DEV)
     torch.library.opcheck(ops.forward_ring_step, (kc, vc, qd, st["y_acc"], st["alpha_sum"], st["qdotk_max"], quad, col_l, roff_l, row_idx, *tail))
     torch.library.opcheck(
