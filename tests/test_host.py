@@ -650,3 +650,36 @@ def test_fused_projection_function_matches_separate_linears():
             t.grad = None
         torch.autograd.backward([torch.nn.functional.linear(x, w, b) for w, b in zip(ws, bs)], grads)
         assert all(torch.allclose(a, t.grad) for a, t in zip(got, [x] + ws + bs))
+
+
+def test_projections_fed_from_and_to_nchw_match_plain_linear():
+    """_FusedLinear1x1NCHW (several projections of an NCHW input as one GEMM with a transposed operand, NHWC column blocks out) and
+    _Linear1x1ToNCHW (NHWC in, NCHW out): outputs and every gradient against F.linear on permuted tensors, on a grid long enough
+    for the split weight-gradient reduction."""
+    from torch_harmonics_amd.attention import _FusedLinear1x1NCHW, _Linear1x1ToNCHW
+
+    torch.manual_seed(0)
+    B, C, H, W = 2, 12, 5, 3501  # 17505 points: three slices of the reduction
+    x = torch.randn(B, C, H, W, dtype=torch.float64, requires_grad=True)
+    ws = [torch.randn(n, C, dtype=torch.float64, requires_grad=True) for n in (8, 4, 16)]
+    bs = [torch.randn(n, dtype=torch.float64, requires_grad=True) for n in (8, 4, 16)]
+    outs = _FusedLinear1x1NCHW.apply(x, ws[0], bs[0], ws[1], bs[1], ws[2], bs[2])
+    assert outs[0].untyped_storage().data_ptr() == outs[2].untyped_storage().data_ptr()  # column blocks of one buffer
+    ref = [torch.nn.functional.linear(x.permute(0, 2, 3, 1), w, b) for w, b in zip(ws, bs)]
+    for o, r in zip(outs, ref):
+        assert torch.allclose(o, r, atol=1e-10)
+    gs = [torch.randn_like(o) for o in outs]
+    for a, r in zip(torch.autograd.grad(outs, [x] + ws + bs, gs), torch.autograd.grad(ref, [x] + ws + bs, gs)):
+        assert torch.allclose(a, r, atol=1e-8)
+    (single,) = _FusedLinear1x1NCHW.apply(x, ws[1], None)
+    assert torch.allclose(single, torch.nn.functional.linear(x.permute(0, 2, 3, 1), ws[1]), atol=1e-10)
+
+    y = torch.randn(B, H, W, C, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(7, C, dtype=torch.float64, requires_grad=True)
+    b = torch.randn(7, dtype=torch.float64, requires_grad=True)
+    o = _Linear1x1ToNCHW.apply(y, w, b)
+    r = torch.nn.functional.linear(y, w, b).permute(0, 3, 1, 2)
+    assert o.is_contiguous() and torch.allclose(o, r, atol=1e-10)
+    g = torch.randn_like(o)
+    for a, rr in zip(torch.autograd.grad(o, [y, w, b], g), torch.autograd.grad(r, [y, w, b], g)):
+        assert torch.allclose(a, rr, atol=1e-8)
