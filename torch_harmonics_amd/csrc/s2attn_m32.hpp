@@ -821,6 +821,59 @@ template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 
     }
 }
 
+// The walk of pass 2 over the scatter runs of one (virtual) input latitude: staged rows are queries, and only the band
+// positions whose query column lies in the local window are visited (the window is the whole circle on one device, a sector
+// of it in a longitude-sharded layer, where most positions of a polar run fall outside).  Band position u of run (ws, len)
+// of a tile at key column w0 is (virtual) query column (w0 - ws - len + 1 + u) mod W; the window holds the virtual
+// columns 0 .. nv of the run's column class.
+struct RingWalk2 {
+    const Run *runs;
+    int ri, rend, W, w0, qps, wo;
+    Run run;
+    int parq, nv, c0, u0, L, m;
+    int pos, ua, ub, col; // the step: positions pos .. pos + HK of [ua, ub); col = query column of position pos (no wrap inside an interval)
+    bool valid;
+    __device__ inline void start(const Run *runs_, int first, int rend_) { runs = runs_, ri = first - 1, rend = rend_, m = 1, valid = false; }
+    __device__ inline bool advance()
+    {
+        if (valid && pos + HK < ub) {
+            pos += HK;
+            col += HK;
+            col -= (col >= W) ? W : 0; // (the whole-circle interval; W >= HK)
+            return true;
+        }
+        for (;;) {
+            m++;
+            if (m > 1) { // next run
+                ri++;
+                if (ri >= rend) return valid = false;
+                run = uniform_load(runs + ri);
+                m = 1;
+                parq = run.lat - run.pad * qps;
+                nv = (wo - parq + qps - 1) / qps; // virtual columns of this class inside the window
+                if (nv <= 0) continue;
+                L = run.len + HQ - 1;
+                c0 = w0 - run.ws - run.len + 1; // in (-2 W, W): query column of position 0
+                c0 += (c0 < 0) ? W : 0;
+                c0 += (c0 < 0) ? W : 0;
+                if (nv >= W) { // the whole circle is local: one interval
+                    ua = pos = 0, ub = L, col = c0;
+                    m = 2;
+                    return valid = true;
+                }
+                u0 = c0 == 0 ? 0 : W - c0; // first position at column 0
+                m = -2;
+                continue;
+            }
+            const int a0 = u0 + m * W;
+            const int a_ = a0 < 0 ? 0 : a0, b_ = a0 + nv > L ? L : a0 + nv;
+            if (a_ >= b_) continue;
+            ua = pos = a_, ub = b_, col = a_ - a0;
+            return valid = true;
+        }
+    }
+};
+
 // ---- backward, pass 2 of a ring step ---------------------------------------------------------------------------------
 // The dk/dv pass above for the keys of ONE chunk: a wavefront owns 16 consecutive virtual columns of one column class of a
 // chunk latitude (real longitudes (w0 + c) * kps + par) and walks the scatter runs of that virtual latitude; staged rows are
@@ -886,39 +939,39 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
     }
     const float lw = fast_log2(a.quad_w[hreal + a.r_wlat0]);
 
-    int pos = 0;
-    Run run = {0, 0, 0, 0};
     Tile qt, gt;
     float2 st = make_float2(0.f, 0.f);
     const int r0 = lane / Tile::CPR;
     const unsigned pc = 16u * (lane % Tile::CPR);
     const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
-    auto fetch = [&](const Run &rn, int p) {
-        int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wi; // (virtual) query column of staged row 0, on the circle of a.Wi columns
-        c0 += (c0 < 0) ? a.Wi : 0;
+    RingWalk2 wk;
+    wk.W = a.Wi, wk.w0 = w0, wk.qps = a.r_qps, wk.wo = a.r_wo;
+    wk.start(a.sruns, ri, rend);
+    const bool any = wk.advance(); // false: none of the queries that see these keys is local
+    auto fetch = [&]() { // the rows of the step the walk stands at; rows beyond the interval are staged as zeros and weigh nothing
         // the run's output latitude is virtual (real latitude Run::pad, column class parq): virtual column j is the local
         // query column j * r_qps + parq
-        const int parq = rn.lat - rn.pad * a.r_qps;
-        const size_t lat = (size_t)rn.pad * a.r_wo + parq;
+        const size_t lat = (size_t)wk.run.pad * a.r_wo + wk.parq;
+        const int nrows = wk.ub - wk.pos;
 #pragma unroll
         for (int it = 0; it < Tile::NIT; it++) {
-            int col = c0 + r0 + it * Tile::RPI;
-            col -= (col >= a.Wi) ? a.Wi : 0;
-            col *= a.r_qps;
+            const int row = r0 + it * Tile::RPI;
             qt.raw[it] = u4v{0u, 0u, 0u, 0u};
             gt.raw[it] = u4v{0u, 0u, 0u, 0u};
-            if (col + parq < a.r_wo && piece_ok) { // inside the local window
-                qt.raw[it] = *reinterpret_cast<const u4v *>(qy + (lat + col) * ldb + pc);
-                gt.raw[it] = *reinterpret_cast<const u4v *>(gy + (lat + col) * ldb + pc);
+            if (row < nrows && piece_ok) {
+                int cr = wk.col + row; // wraps only when the window is the whole circle
+                cr -= (cr >= a.Wi) ? a.Wi : 0;
+                const size_t o = (lat + (size_t)cr * a.r_qps) * ldb + pc;
+                qt.raw[it] = *reinterpret_cast<const u4v *>(qy + o);
+                gt.raw[it] = *reinterpret_cast<const u4v *>(gy + o);
             }
         }
         if (lane < HK) { // lanes 0..31 fetch the statistics of the staged rows: (log2-sum-exp, integral_norm)
-            int col = c0 + lane;
-            col -= (col >= a.Wi) ? a.Wi : 0;
-            col *= a.r_qps;
-            st = make_float2(INFINITY, 0.f); // a row outside the window weighs exp2(-inf) = 0
-            if (col + parq < a.r_wo) {
-                const size_t s = sbase + lat + col;
+            st = make_float2(INFINITY, 0.f); // exp2(-inf) = 0
+            if (lane < nrows) {
+                int cr = wk.col + lane;
+                cr -= (cr >= a.Wi) ? a.Wi : 0;
+                const size_t s = sbase + lat + (size_t)cr * a.r_qps;
                 const float as = a.r_asum[s];
                 if (as > 0.f) st = make_float2(fmaf(a.r_qmax[s], LOG2E, fast_log2(as)), a.r_integral[s]); // (a query that saw nothing weighs nothing)
             }
@@ -932,30 +985,27 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
             Is[lane] = st.y;
         }
     };
-    run = a.sruns[ri];
-    fetch(run, 0);
-    commit();
+    if (any) {
+        fetch();
+        commit();
+    }
     __syncthreads();
     settle(kop);
     settle(vop);
 
-    while (ri < rend) {
-        const int len = run.len;
-        int nri = ri, npos = pos + HK;
-        Run nrun = run;
-        if (npos >= len + HQ - 1) {
-            nri++;
-            npos = 0;
-            if (nri < rend) nrun = a.sruns[nri];
-        }
-        const bool more = nri < rend;
-        if (more) fetch(nrun, npos);
+    while (any) {
+        const int len = wk.run.len, pos = wk.pos, ub = wk.ub;
+        const bool more = wk.advance();
+        if (more) fetch();
 
         f4v sc[2], gc[2];
         m32_scores<D, PITCH>(sc, Qs, c, qd, kop);
         m32_scores<D, PITCH>(gc, Gs, c, qd, vop);
-        const int tb = pos + 4 * qd - c; // r - c of element (qb, v): tb + 16 qb + v
-        const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
+        // element (qb, v) is staged row u = pos + 16 qb + 4 qd + v, which sees key c as its neighbor t = u - c: it counts iff
+        // 0 <= t < len and u < ub, i.e. t < min(len, ub - c) as unsigned numbers
+        const int tb = pos + 4 * qd - c;
+        const unsigned lim = (unsigned)max(0, min(len, ub - c));
+        const bool inner = pos >= HQ - 1 && pos + HK <= min(len, ub); // every element of the step counts
 #pragma unroll
         for (int qb = 0; qb < 2; qb++) {
             const float4 l4 = *reinterpret_cast<const float4 *>(Ls + 16 * qb + 4 * qd);
@@ -965,7 +1015,7 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
 #pragma unroll
             for (int v = 0; v < 4; v++) {
                 float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v])); // = alpha / alpha_sum
-                if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
+                if (!inner) p = ((unsigned)(tb + 16 * qb + v) < lim) ? p : 0.f;
                 sc[qb][v] = p;
                 gc[qb][v] = p * (gc[qb][v] - iv[v]);
             }
@@ -974,11 +1024,9 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
         m32_accumulate<D, PITCH>(dkt, Qs, c, qd, gc);
 
         __syncthreads();
-        if (more) commit();
+        if (!more) break;
+        commit();
         __syncthreads();
-        ri = nri;
-        pos = npos;
-        run = nrun;
     }
 
     if (mine) {
