@@ -13,7 +13,7 @@ q/k/v weights) and resident in HBM before the timed region.  Prints ONE JSON lin
 Reported alongside the throughput:
   roofline      the slowest kernel of the step, timed with events recorded on the launch stream
                 around every launch of it inside the timed region
-  cpu_baseline  the CPU port of the reference algorithm (oracle/, reference release flags, OpenMP)
+  cpu_baseline  the reference's own CPU operators (oracle/_ref, its release flags, OpenMP) and the C restatement of them (oracle/)
                 on a bounded sample of the same workload, on this machine's host cores
   other_configs op-level forward and backward times of the other four benchmark configurations
 """
@@ -249,60 +249,132 @@ def time_ring_steps(device, nchunk=4, reps=2):
     return res
 
 
-def cpu_baseline(cfg, mod, k, v, q, dy):
-    """
-    Times the fp32 CPU port of the reference algorithm (oracle/s2attn_oracle.c, built with the reference's
-    release flags) forward + backward on a sample of the workload: the first four heads and every 6th output
-    latitude (both pole rows included, so the reference backward's per-neighbor scratch is sized by the longest
-    row, as in the full problem).  Throughput is neighbor pairs of the sample per second.
-    """
-    from oracle import cpu_attention as oracle
-
+def cpu_sample(cfg, col, ro):
+    """The bounded sample of a workload that the CPU legs time: the first four heads and every 6th output latitude (both pole
+    rows included, so the reference backward's per-neighbor scratch is sized by the longest row, as in the full problem)."""
     nh_s = min(4, cfg["nh"])
-    ck, cv = mod.k_channels // cfg["nh"], mod.out_channels // cfg["nh"]
     Ho, Wo = cfg["out_shape"]
     stride = 6 if Ho >= 120 else 1
     rows = torch.arange(0, Ho, stride)
     if rows[-1] != Ho - 1:
         rows = torch.cat([rows, torch.tensor([Ho - 1])])
-    col, ro = mod.psi_col_idx.cpu(), mod.psi_roff_idx.cpu()
     lens = (ro[1:] - ro[:-1])[rows]
     ro_s = torch.zeros(len(rows) + 1, dtype=torch.int64)
     ro_s[1:] = torch.cumsum(lens, 0)
     col_s = torch.cat([col[ro[r] : ro[r + 1]] for r in rows.tolist()])
+    pairs = cfg["B"] * nh_s * Wo * int(lens.sum())
+    scratch_gb = 2 * cfg["B"] * nh_s * len(rows) * Wo * int(lens.max()) * 4 / 1e9
+    full_pairs = cfg["B"] * cfg["nh"] * Wo * int(col.numel())
+    return dict(nh=nh_s, rows=rows, stride=stride, col=col_s, ro=ro_s, pairs=pairs, scratch_gb=scratch_gb, full_pairs=full_pairs, full=full_pairs <= 4e9)
+
+
+def reference_cpu_times(config_name, others):
+    """
+    The reference's OWN CPU operators (oracle/_ref/attention_ref.so: its CPU sources compiled with its release flags) on the
+    sample of `config_name`, on its full forward where that is feasible, and on the configurations of `others` in full.
+    They run in a child process, and this function is called before this process touches the GPU (a process that holds a
+    GPU context starts no other program).  The child makes its own N(0,1) tensors of the workload's shapes (the algorithm
+    has no data-dependent control flow), on psi from the oracle's geometry, which the tests hold element-equal to the
+    module's.  Returns None where the library has not been built.
+    """
+    from oracle import geometry as ogeo
+    from oracle import reference_ops as reference
+
+    if not reference.available():
+        return None
+    cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
+    jobs, keys = [], []
+
+    def add(key, cfg, col, ro, nh, nlat_out, bwd):
+        (Hi, Wi), (_, Wo) = cfg["in_shape"], cfg["out_shape"]
+        ck = cfg["C"] // cfg["nh"]
+        w = ogeo.attention_quad_weights(Hi, Wi, cfg["grid_in"])
+        kk = {"randn": [cfg["B"], Hi, Wi, nh * ck], "seed": 1, "scale": 1.0}
+        vv = {"randn": [cfg["B"], Hi, Wi, nh * ck], "seed": 2, "scale": 1.0}
+        qq = {"randn": [cfg["B"], nlat_out, Wo, nh * ck], "seed": 3, "scale": 1.0 / math.sqrt(ck)}
+        gg = {"randn": [cfg["B"], nlat_out, Wo, nh * ck], "seed": 4, "scale": 1.0}
+        jobs.append(dict(op="forward", args=[kk, vv, qq, w, col, ro, nh, Wi, nlat_out, Wo], discard=True))
+        keys.append((key, "fwd_ms"))
+        if bwd:
+            jobs.append(dict(op="backward", args=[dict(kk), dict(vv), dict(qq), gg, w, col, ro, nh, Wi, nlat_out, Wo], discard=True))
+            keys.append((key, "bwd_ms"))
+
+    cfg = CONFIGS[config_name]
+    col, ro = ogeo.neighborhood_csr(cfg["in_shape"], cfg["out_shape"], cfg["grid_in"], cfg["grid_out"], cfg["theta_cutoff"])
+    smp = cpu_sample(cfg, col, ro)
+    add("sample", cfg, smp["col"], smp["ro"], smp["nh"], len(smp["rows"]), True)
+    if smp["full"]:
+        add("full", cfg, col, ro, cfg["nh"], cfg["out_shape"][0], False)
+    for name in others:
+        c = CONFIGS[name]
+        oc, orr = ogeo.neighborhood_csr(c["in_shape"], c["out_shape"], c["grid_in"], c["grid_out"], c["theta_cutoff"])
+        add(name, c, oc, orr, c["nh"], c["out_shape"][0], True)
+    res = reference.run(jobs, threads=cores)
+    out = {}
+    for (key, what), r in zip(keys, res):
+        out.setdefault(key, {})[what] = 1e3 * r["seconds"][0]
+    return out
+
+
+def cpu_baseline(cfg, mod, k, v, q, dy, ref_times=None):
+    """
+    Times the reference's CPU algorithm forward + backward on a sample of the workload (cpu_sample).  Throughput is
+    neighbor pairs of the sample per second.  Two builds: the reference's OWN CPU operators (`ref_times`, from
+    reference_cpu_times; `kind` "reference") and the C restatement of the same algorithm (oracle/s2attn_oracle.c, the
+    same flags, on the workload's own tensors; `port_*`).  Without the reference build the restatement is the baseline
+    (`kind` "port").
+    """
+    from oracle import cpu_attention as oracle
+
+    ck, cv = mod.k_channels // cfg["nh"], mod.out_channels // cfg["nh"]
+    Ho, Wo = cfg["out_shape"]
+    col, ro = mod.psi_col_idx.cpu(), mod.psi_roff_idx.cpu()
+    smp = cpu_sample(cfg, col, ro)
+    nh_s, rows, col_s, ro_s, pairs = smp["nh"], smp["rows"], smp["col"], smp["ro"], smp["pairs"]
     ks = k[..., : nh_s * ck].float().cpu().contiguous()
     vs = v[..., : nh_s * cv].float().cpu().contiguous()
     qs = q[:, rows][..., : nh_s * ck].float().cpu().contiguous()
     gs = dy[:, rows][..., : nh_s * cv].float().cpu().contiguous()
     w = mod.quad_weights.float().cpu()
-    pairs = cfg["B"] * nh_s * Wo * int(lens.sum())
-    scratch_gb = 2 * cfg["B"] * nh_s * len(rows) * Wo * int(lens.max()) * 4 / 1e9
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     t0 = time.perf_counter()
     oracle.forward_f32(ks, vs, qs, w, col_s, ro_s, nh_s, fast=True)
     t1 = time.perf_counter()
     oracle.backward_f32(ks, vs, qs, gs, w, col_s, ro_s, nh_s, fast=True)
     t2 = time.perf_counter()
-    out = {
-        "value": pairs / (t2 - t0),
-        "unit": "pairs/s",
-        "cores": cores,
-        "kind": "port",
-        "sample": f"{nh_s} of {cfg['nh']} heads x {len(rows)} of {Ho} output latitudes (every {stride}th, both poles) = {pairs} pairs; "
-        f"fwd {1e3 * (t1 - t0):.0f} ms + bwd {1e3 * (t2 - t1):.0f} ms; reference bwd scratch {scratch_gb:.1f} GB",
-        "fwd_ms": 1e3 * (t1 - t0),
-        "bwd_ms": 1e3 * (t2 - t1),
-    }
+    port = {"fwd_ms": 1e3 * (t1 - t0), "bwd_ms": 1e3 * (t2 - t1)}
     # The forward alone has no scratch and is feasible in full: all heads, all latitudes of the workload (the reference backward
     # would need 2 * B * heads * nlat_out * nlon_out * max_row_len floats, 383 GB at 721x1440 with 8 heads).
-    full_pairs = cfg["B"] * cfg["nh"] * Wo * int(col.numel())
-    if full_pairs <= 4e9:
+    if smp["full"]:
         kf, vf, qf = k.float().cpu().contiguous(), v.float().cpu().contiguous(), q.float().cpu().contiguous()
         t0 = time.perf_counter()
         oracle.forward_f32(kf, vf, qf, w, col, ro, cfg["nh"], fast=True)
-        t1 = time.perf_counter()
-        out["full_forward_ms"] = 1e3 * (t1 - t0)
-        out["full_forward_pairs_per_s"] = full_pairs / (t1 - t0)
+        port["full_forward_ms"] = 1e3 * (time.perf_counter() - t0)
+
+    timed, kind = port, "port"
+    if ref_times and "sample" in ref_times:
+        timed, kind = dict(ref_times["sample"]), "reference"
+        if smp["full"] and "full" in ref_times:
+            timed["full_forward_ms"] = ref_times["full"]["fwd_ms"]
+    out = {
+        "value": pairs / (1e-3 * (timed["fwd_ms"] + timed["bwd_ms"])),
+        "unit": "pairs/s",
+        "cores": cores,
+        "kind": kind,
+        "sample": f"{nh_s} of {cfg['nh']} heads x {len(rows)} of {Ho} output latitudes (every {smp['stride']}th, both poles) = {pairs} pairs; "
+        f"fwd {timed['fwd_ms']:.0f} ms + bwd {timed['bwd_ms']:.0f} ms; reference bwd scratch {smp['scratch_gb']:.1f} GB"
+        + ("; the reference's own CPU operators on N(0,1) tensors of these shapes, in a child process" if kind == "reference" else ""),
+        "fwd_ms": timed["fwd_ms"],
+        "bwd_ms": timed["bwd_ms"],
+    }
+    if "full_forward_ms" in timed:
+        out["full_forward_ms"] = timed["full_forward_ms"]
+        out["full_forward_pairs_per_s"] = smp["full_pairs"] / (1e-3 * timed["full_forward_ms"])
+    if kind == "reference":  # the restatement beside it: same algorithm, same flags, the workload's own tensors
+        out["port_value"] = pairs / (1e-3 * (port["fwd_ms"] + port["bwd_ms"]))
+        out["port_fwd_ms"], out["port_bwd_ms"] = port["fwd_ms"], port["bwd_ms"]
+        if "full_forward_ms" in port:
+            out["port_full_forward_ms"] = port["full_forward_ms"]
     return out
 
 
@@ -321,6 +393,10 @@ def main():
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)", file=sys.stderr)
         sys.exit(2)
+    # the reference's own CPU build is timed first, in a child process, while this process has not touched the GPU yet
+    ref_times = None
+    if not args.no_cpu_baseline and not args.ring_only and torch.cuda.device_count() > 0:
+        ref_times = reference_cpu_times(args.config, [] if args.no_other_configs else [n for n in ("cfg1", "cfg2") if n != args.config])
     if not torch.cuda.is_available():
         print("bench.py needs a ROCm GPU", file=sys.stderr)
         sys.exit(2)
@@ -499,10 +575,13 @@ def main():
         out["other_configs"] = {
             name: time_other_config(name, dev, cpu=(not args.no_cpu_baseline) and name in ("cfg1", "cfg2")) for name in sorted(CONFIGS) if name != args.config
         }
+        for name, t in (ref_times or {}).items():  # cfg1, cfg2 in full on the reference's own CPU operators
+            if name in out["other_configs"]:
+                out["other_configs"][name]["cpu_reference_fwd_ms"], out["other_configs"][name]["cpu_reference_bwd_ms"] = t["fwd_ms"], t["bwd_ms"]
         out["ring_steps"] = time_ring_steps(dev)
 
     if not args.no_cpu_baseline:
-        out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy)
+        out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy, ref_times)
 
     print(json.dumps(out))
 

@@ -32,7 +32,11 @@
  * masked softmax evaluated by torch in float64 with autograd, against
  * F.scaled_dot_product_attention for a cutoff covering the sphere, against the
  * closed forms (constant v, single-neighbor rows, longitude-roll equivariance)
- * and against the committed vectors in tests/golden/.
+ * and against the committed vectors in tests/golden/.  On top of those, both
+ * families are held against the reference's OWN CPU operators: its CPU sources
+ * compiled by `make -C oracle ref` and run on the same seeded inputs
+ * (tests/test_oracle_reference.py, where that build exists), and their outputs
+ * committed as vectors (tests/golden/reference_cpu/, tests/test_golden_reference.py).
  *
  * Tensor layout everywhere: physical NHWC with heads packed along channels,
  *   k : [B, Hi, Wi, nh*Ck]   v : [B, Hi, Wi, nh*Cv]
