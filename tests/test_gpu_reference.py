@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import reference_ops as ref
-from tests.test_gpu_large import TOL, _hip, _setup
+from tests.test_gpu_large import DEV, TOL, _hip, _setup
 from tests.util import assert_close
 
 pytestmark = [pytest.mark.gpu, pytest.mark.skipif(not ref.available(), reason="oracle/_ref/attention_ref.so is not built (make -C oracle ref)")]
@@ -65,3 +65,23 @@ def test_upsampling_against_the_reference_cpu_operators():
     want = _reference(k, v, q, dy, w, col, roff, nh)
     for saved in (False, True):
         _compare(f"up-sampling (saved={saved})", _hip(k, v, q, dy, w, col, roff, nh, (Hi, Wi, Ho, Wo), saved=saved), want)
+
+
+def test_cfg5_one_head_bf16_every_latitude_against_the_reference_cpu_operators():
+    """Legendre-Gauss 361x720 self-attention at cfg5's cutoff, one head of 64 channels, bf16 storage (the 16-bit matrix-core
+    kernels).  The reference's CPU operators take the same bf16 tensors (they compute in fp32 and return bf16); tolerance
+    2e-2 relative to each tensor's scale, as for every bf16 check."""
+    from tests.test_gpu_large import _bf16_close
+    from torch_harmonics_amd import ops
+
+    c, (Hi, Wi, Ho, Wo, nh, d), col, roff, w, k, v, q, dy = _setup("cfg5", heads=1, batch=1)
+    k, v, q, dy = [(0.5 * t).to(torch.bfloat16) for t in (k, v, q, dy)]
+    want = _reference(k, v, q, dy, w, col, roff, nh)
+    assert want[0].dtype == torch.bfloat16
+    kd, vd, qd, gd = [t.to(DEV) for t in (k, v, q, dy)]
+    args = tuple(t.to(DEV) for t in (w, col, roff)) + (nh, Wi, Ho, Wo)
+    y, lse = ops.forward_lse(kd, vd, qd, *args)
+    dk, dv, dq = ops.backward_saved(kd, vd, qd, gd, y, lse, *args)
+    torch.cuda.synchronize()
+    for key, got, r in zip(("y", "dk", "dv", "dq"), (y, dk, dv, dq), want):
+        _bf16_close(f"cfg5 {key}", got.cpu(), r.double())
