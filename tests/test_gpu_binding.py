@@ -187,3 +187,105 @@ def test_column_blocks_of_a_fused_projection_are_read_and_written_in_place(share
     qs, ks, vs = small.split([16, 16, 16], dim=-1)
     with pytest.raises(RuntimeError, match="point stride"):
         ops.forward_lse(ks, vs, qs, geo[0], geo[1], geo[2], 1, W, H, W)
+
+
+def _geo(ins, outs, tc):
+    col, roff = ogeo.neighborhood_csr(ins, outs, "equiangular", "equiangular", tc)
+    w = ogeo.attention_quad_weights(ins[0], ins[1], "equiangular")
+    return w.to(DEV), col.to(DEV), roff.to(DEV)
+
+
+@pytest.mark.parametrize("d,dtype", [(16, torch.float32), (64, torch.bfloat16), (32, torch.bfloat16), (32, torch.float32)], ids=["d16_fp32", "d64_bf16", "d32_bf16", "d32_fp32"])
+def test_slices_of_a_fused_buffer_work_for_every_kernel_family(d, dtype):
+    """q, k, v given as column blocks of one (B, H, W, 3C) buffer: only the fp32 32-channel heads on wide grids are read in place;
+    every other shape must be copied by the Python operators (and give what contiguous tensors give), not refused by the library."""
+    from torch_harmonics_amd import ops
+
+    nh, ins = 2, (12, 96)
+    w, col, roff = _geo(ins, ins, 0.5)
+    g = torch.Generator().manual_seed(SEED)
+    buf = (0.5 * torch.randn(2, *ins, 3 * nh * d, generator=g)).to(dtype).to(DEV)
+    dy = torch.randn(2, *ins, nh * d, generator=g).to(dtype).to(DEV)
+    geo = (w, col, roff, nh, ins[1], ins[0], ins[1])
+
+    def run(q, k, v):
+        q, k, v = [t.detach().requires_grad_(True) for t in (q, k, v)]
+        y = ops.neighborhood_s2_attention(k, v, q, *geo)
+        y.backward(dy)
+        return y.detach(), k.grad, v.grad, q.grad
+
+    q, k, v = buf.chunk(3, dim=-1)
+    assert not k.is_contiguous()
+    got = run(q, k, v)
+    want = run(q.contiguous(), k.contiguous(), v.contiguous())
+    for name, g_, w_ in zip(("y", "dk", "dv", "dq"), got, want):
+        assert torch.equal(g_, w_), f"{name}: slices of a fused buffer give something else than contiguous copies"
+    # an expanded (stride 0) tensor is not a column block either
+    ke = k[:, :, :1].expand(-1, -1, ins[1], -1)
+    got = run(q, ke, v)
+    want = run(q.contiguous(), ke.contiguous(), v.contiguous())
+    for name, g_, w_ in zip(("y", "dk", "dv", "dq"), got, want):
+        assert torch.equal(g_, w_), f"{name}: expanded key"
+
+
+def test_backward_operators_pass_opcheck_on_column_blocks():
+    """The fake kernels of the backward operators describe the gradients as the binding lays them out: column blocks of one new
+    buffer when k | v | q are disjoint column blocks of one buffer."""
+    nh, d, ins = 2, 32, (12, 96)
+    w, col, roff = _geo(ins, ins, 0.5)
+    g = torch.Generator().manual_seed(SEED)
+    buf = (0.5 * torch.randn(2, *ins, 3 * nh * d, generator=g)).to(DEV)
+    dy = torch.randn(2, *ins, nh * d, generator=g).to(DEV)
+    q, k, v = buf.chunk(3, dim=-1)
+    geo = (w, col, roff, nh, ins[1], ins[0], ins[1])
+    sk = torch.ops.s2attn_kernels
+    y, lse = sk.forward_lse(k, v, q, *geo)
+    dk, dv, dq = sk.backward_saved(k, v, q, dy, y, lse, *geo)
+    assert dk.stride() == k.stride() and dv.stride() == v.stride() and dq.stride() == q.stride()
+    assert dk.untyped_storage().data_ptr() == dv.untyped_storage().data_ptr() == dq.untyped_storage().data_ptr()
+    torch.library.opcheck(sk.forward_lse, (k, v, q, *geo))
+    torch.library.opcheck(sk.backward_saved, (k, v, q, dy, y, lse, *geo))
+    torch.library.opcheck(torch.ops.attention_kernels.backward, (k, v, q, dy, *geo))
+    # k | v fused, q separate
+    qs = q.contiguous()
+    torch.library.opcheck(sk.backward_saved, (k, v, qs, dy, y, lse, *geo))
+
+
+def test_overlapping_column_blocks_get_separate_gradients():
+    """k and v given as the SAME slice of a wider buffer: their gradients must not share memory."""
+    nh, d, ins = 2, 32, (12, 96)
+    w, col, roff = _geo(ins, ins, 0.5)
+    g = torch.Generator().manual_seed(SEED)
+    buf = (0.5 * torch.randn(2, *ins, 2 * nh * d, generator=g)).to(DEV)
+    dy = torch.randn(2, *ins, nh * d, generator=g).to(DEV)
+    q, kv = buf.chunk(2, dim=-1)
+    geo = (w, col, roff, nh, ins[1], ins[0], ins[1])
+    sk = torch.ops.s2attn_kernels
+    y, lse = sk.forward_lse(kv, kv, q, *geo)
+    dk, dv, dq = sk.backward_saved(kv, kv, q, dy, y, lse, *geo)
+    kc = kv.contiguous()
+    yc, lsec = sk.forward_lse(kc, kc.clone(), q.contiguous(), *geo)
+    dkc, dvc, dqc = sk.backward_saved(kc, kc.clone(), q.contiguous(), dy, yc, lsec, *geo)
+    assert torch.equal(y, yc)
+    for name, g_, w_ in (("dk", dk, dkc), ("dv", dv, dvc), ("dq", dq, dqc)):
+        assert torch.equal(g_, w_), f"{name}: k and v as one slice"
+    torch.library.opcheck(sk.backward_saved, (kv, kv, q, dy, y, lse, *geo))
+
+
+def test_fused_module_compiles_with_matching_gradient_strides():
+    """A 64-channel module with 32-channel heads on a 96-longitude grid takes the fused q | k | v path; traced through AOT autograd
+    the backward's outputs must have the strides its fake kernel announced."""
+    m, x = _module_and_inputs(C=64, nh=2)
+    gout = torch.randn(2, 64, 24, 96, device=DEV)
+
+    def run(fn):
+        a = x.detach().clone().requires_grad_(True)
+        m.zero_grad(set_to_none=True)
+        out = fn(a)
+        out.backward(gout)
+        return [out.detach(), a.grad] + [p.grad.clone() for p in m.parameters()]
+
+    eager = run(m)
+    compiled = run(torch.compile(m, backend="aot_eager", fullgraph=True))
+    for i, (e, c) in enumerate(zip(eager, compiled)):
+        assert_close(f"tensor {i}", c, e, rtol=1e-6, atol=1e-6)

@@ -59,14 +59,43 @@ def test_noalloc_backward_matches_the_workspace_entry_point_twice():
     for name, prob in (("first call", big), ("second call, smaller", small), ("third call, another kernel family", other)):
         print(name, flush=True)
         want = _run(lib, prob, noalloc=False)
-        before = torch.cuda.memory_allocated()
-        k, v, q, dy, w, plan, shape = prob
         got = _run(lib, prob, noalloc=True)
         for t_name, g_, w_ in zip(("dk", "dv", "dq"), got, want):
             assert torch.isfinite(g_).all(), f"{name}: {t_name} has non-finite values"
             assert torch.equal(g_, w_), f"{name}: {t_name} differs from s2attn_backward_saved, max |diff| {(g_ - w_).abs().max().item():.3e}"
-        del got, want
-        assert torch.cuda.memory_allocated() <= before + 0  # the library itself allocated nothing through torch either
+
+
+@pytest.mark.gpu
+def test_noalloc_backward_is_capturable_into_a_graph():
+    """A device allocation inside a stream capture fails the capture, so recording the entry point into a HIP graph (after one call
+    outside the capture, which looks up the scratch array's address) shows that it allocates nothing; every replay must equal
+    s2attn_backward_saved bit for bit, with eager work and synchronisations between the replays."""
+    lib = _lib.load()
+    prob = _problem(1, 2, 32, (16, 96), (16, 96), 0.5, seed=4)
+    k, v, q, dy, w, plan, shape = prob
+    want = _run(lib, prob, noalloc=False)
+    _run(lib, prob, noalloc=True)  # first call on this device: outside the capture
+    pl, sh = ctypes.byref(plan.struct), ctypes.byref(shape)
+    y = torch.empty_like(dy)
+    lse = torch.empty((shape.batch, shape.num_heads, shape.nlat_out, shape.nlon_out), device=DEV)
+    dk, dv, dq = torch.empty_like(k), torch.empty_like(v), torch.empty_like(q)
+    _lib.check(lib.s2attn_forward_lse(k.data_ptr(), v.data_ptr(), q.data_ptr(), w.data_ptr(), y.data_ptr(), lse.data_ptr(), pl, sh, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)), "forward")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    with torch.cuda.graph(graph, stream=side):
+        stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        rc = lib.s2attn_backward_saved_noalloc(k.data_ptr(), v.data_ptr(), q.data_ptr(), dy.data_ptr(), y.data_ptr(), lse.data_ptr(), w.data_ptr(), dk.data_ptr(), dv.data_ptr(), dq.data_ptr(), pl, sh, stream)
+    _lib.check(rc, "s2attn_backward_saved_noalloc under capture")
+    for it in range(3):
+        for t in (dk, dv, dq):
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for t_name, g_, w_ in zip(("dk", "dv", "dq"), (dk, dv, dq), want):
+            assert torch.equal(g_, w_), f"replay {it}: {t_name} differs from s2attn_backward_saved"
+        _run(lib, _problem(1, 1, 32, (12, 64), (12, 64), 0.6, seed=5 + it), noalloc=True)  # eager work on the same scratch between replays
 
 
 def test_noalloc_backward_rejects_shapes_beyond_its_scratch():

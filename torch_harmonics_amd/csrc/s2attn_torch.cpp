@@ -16,6 +16,7 @@
 
 #include <list>
 #include <mutex>
+#include <utility>
 #include <tuple>
 #include <vector>
 
@@ -248,9 +249,15 @@ std::tuple<Tensor, Tensor, Tensor> backward_impl(const Tensor &kx, const Tensor 
     // same column blocks of ONE new buffer, so that the caller's input gradient is a single GEMM over it.
     Tensor dk, dv, dq;
     const int64_t ldk = point_stride(kx, "kx"), ldv = point_stride(vx, "vx"), ldq = point_stride(qy, "qy");
-    const bool kv_fused = ldk > 0 && ldk == ldv && kx.storage().is_alias_of(vx.storage()) && kx.storage_offset() / ldk == vx.storage_offset() / ldk;
-    const bool all_fused = kv_fused && ldq == ldk && qy.storage().is_alias_of(kx.storage()) && qy.sizes().slice(0, 3) == kx.sizes().slice(0, 3)
-                           && qy.storage_offset() / ldk == kx.storage_offset() / ldk;
+    // (the column ranges must lie inside one row of the buffer and be pairwise disjoint: k and v given as the same or overlapping
+    // slices would otherwise have their gradients written to the same addresses)
+    auto cols = [](const Tensor &t, int64_t ld) { return std::pair<int64_t, int64_t>(t.storage_offset() % ld, t.storage_offset() % ld + t.size(3)); };
+    auto disjoint = [](std::pair<int64_t, int64_t> a, std::pair<int64_t, int64_t> b) { return a.second <= b.first || b.second <= a.first; };
+    bool kv_fused = ldk > 0 && ldk == ldv && kx.storage().is_alias_of(vx.storage()) && kx.storage_offset() / ldk == vx.storage_offset() / ldk;
+    if (kv_fused) kv_fused = cols(kx, ldk).second <= ldk && cols(vx, ldk).second <= ldk && disjoint(cols(kx, ldk), cols(vx, ldk));
+    bool all_fused = kv_fused && ldq == ldk && qy.storage().is_alias_of(kx.storage()) && qy.sizes().slice(0, 3) == kx.sizes().slice(0, 3)
+                     && qy.storage_offset() / ldk == kx.storage_offset() / ldk;
+    if (all_fused) all_fused = cols(qy, ldk).second <= ldk && disjoint(cols(qy, ldk), cols(kx, ldk)) && disjoint(cols(qy, ldk), cols(vx, ldk));
     if (kv_fused) {
         Tensor buf = at::empty({kx.size(0), kx.size(1), kx.size(2), ldk}, kx.options());
         const int64_t used = kx.size(3) + vx.size(3) + (all_fused ? qy.size(3) : 0);

@@ -65,14 +65,53 @@ def _(kx, vx, qy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, 
     return y, torch.empty((kx.shape[0], num_heads, nlat_out, nlon_out), dtype=torch.float32, device=kx.device)
 
 
+def _point_stride(t: torch.Tensor) -> int:
+    """Elements between two grid points when t is a column block of a wider buffer, 0 when it is packed (the binding's point_stride)."""
+    return 0 if t.is_contiguous() else t.stride(2)
+
+
+def _same_buffer(a: torch.Tensor, b: torch.Tensor) -> bool:
+    return a.untyped_storage().data_ptr() == b.untyped_storage().data_ptr() if not isinstance(a, torch._subclasses.FakeTensor) else torch._C._is_alias_of(a, b)
+
+
+def _fake_gradients(kx, vx, qy):
+    """Metadata of (dk, dv, dq) as the binding's backward returns them (csrc/s2attn_torch.cpp, backward_impl): packed tensors, except
+    that k | v (| q) given as DISJOINT column blocks of one buffer get their gradients as the same column blocks of one new
+    buffer."""
+    ldk, ldv, ldq = _point_stride(kx), _point_stride(vx), _point_stride(qy)
+
+    def cols(t, ld):
+        first = t.storage_offset() % ld
+        return first, first + t.shape[3]
+
+    def disjoint(a, b):
+        return a[1] <= b[0] or b[1] <= a[0]
+
+    kv_fused = ldk > 0 and ldk == ldv and _same_buffer(kx, vx) and kx.storage_offset() // ldk == vx.storage_offset() // ldk
+    if kv_fused:
+        ck_, cv_ = cols(kx, ldk), cols(vx, ldk)
+        kv_fused = ck_[1] <= ldk and cv_[1] <= ldk and disjoint(ck_, cv_)
+    if not kv_fused:
+        return kx.new_empty(kx.shape), vx.new_empty(vx.shape), qy.new_empty(qy.shape)
+    all_fused = ldq == ldk and _same_buffer(qy, kx) and tuple(qy.shape[:3]) == tuple(kx.shape[:3]) and qy.storage_offset() // ldk == kx.storage_offset() // ldk
+    if all_fused:
+        cq_ = cols(qy, ldk)
+        all_fused = cq_[1] <= ldk and disjoint(cq_, ck_) and disjoint(cq_, cv_)
+    buf = kx.new_empty((kx.shape[0], kx.shape[1], kx.shape[2], ldk))
+    dk = buf.narrow(3, ck_[0], kx.shape[3])
+    dv = buf.narrow(3, cv_[0], vx.shape[3])
+    dq = buf.narrow(3, cq_[0], qy.shape[3]) if all_fused else qy.new_empty(qy.shape)
+    return dk, dv, dq
+
+
 @torch.library.register_fake("attention_kernels::backward")
 def _(kx, vx, qy, dy, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out):
-    return torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
+    return _fake_gradients(kx, vx, qy)
 
 
 @torch.library.register_fake("s2attn_kernels::backward_saved")
 def _(kx, vx, qy, dy, y, lse, quad_weights, col_idx, row_off, num_heads, nlon_in, nlat_out, nlon_out, plan=None, plan_header=None):
-    return torch.empty_like(kx), torch.empty_like(vx), torch.empty_like(qy)
+    return _fake_gradients(kx, vx, qy)
 
 
 # ---- layout ops ------------------------------------------------------------------------
@@ -134,14 +173,34 @@ def _neighborhood_s2_attention_bwd_optimized(ctx, grad_output):
 _neighborhood_s2_attention_optimized.register_autograd(_neighborhood_s2_attention_bwd_optimized, setup_context=_setup_context_attention_backward)
 
 
-def _packed_or_block(t: torch.Tensor) -> torch.Tensor:
-    """t itself when it is contiguous or a column block of a contiguous (B, nlat, nlon, width) buffer (a slice of a fused
-    q | k | v projection, which the kernels read in place), else a contiguous copy."""
+def takes_column_blocks(dtype: torch.dtype, ck: int, cv: int, nlon_in: int, nlon_out: int) -> bool:
+    """True for the shapes whose kernels read q, k, v in place out of a wider buffer and write dq, dk, dv into one
+    (fp32 heads of 32 channels on at least 64 longitudes per virtual latitude: the hybrid kernels)."""
+    return dtype == torch.float32 and ck == 32 and cv == 32 and min(nlon_in, nlon_out) >= 64
+
+
+def _is_column_block(t: torch.Tensor) -> bool:
+    """t is a column block of a contiguous (B, nlat, nlon, width) buffer: unit channel stride, one point stride of at least
+    its own width (an expanded tensor has stride 0), both offset and stride multiples of four elements."""
+    if t.dim() != 4 or t.stride(3) != 1:
+        return False
+    ld = t.stride(2)
+    return ld >= t.shape[3] and ld % 4 == 0 and t.stride(1) == t.shape[2] * ld and t.stride(0) == t.shape[1] * t.stride(1) and t.storage_offset() % 4 == 0
+
+
+def _packed_or_block(t: torch.Tensor, blocks_ok: bool) -> torch.Tensor:
+    """t itself when it is contiguous, or when it is a column block of a wider buffer (a slice of a fused q | k | v
+    projection) AND the shape is one whose kernels read such blocks in place (blocks_ok, see takes_column_blocks); a
+    contiguous copy otherwise."""
     if t.is_contiguous():
         return t
-    if t.dim() == 4 and t.stride(3) == 1 and t.stride(2) % 4 == 0 and t.stride(1) == t.shape[2] * t.stride(2) and t.stride(0) == t.shape[1] * t.stride(1) and t.storage_offset() % 4 == 0:
+    if blocks_ok and _is_column_block(t):
         return t
     return t.contiguous()
+
+
+def _blocks_ok(kw: torch.Tensor, vw: torch.Tensor, nh: int, nlon_in: int, nlon_out: int) -> bool:
+    return nh > 0 and takes_column_blocks(kw.dtype, kw.shape[3] // nh, vw.shape[3] // nh, nlon_in, nlon_out)
 
 
 # Same op, but the forward also hands its output and softmax normaliser to the backward (the reference recomputes both,
@@ -162,7 +221,8 @@ def _neighborhood_s2_attention_saved(
     plan: Optional[torch.Tensor] = None,
     plan_header: Optional[List[int]] = None,
 ) -> Tuple[torch.Tensor, torch.Tensor]:
-    return forward_lse(_packed_or_block(kw), _packed_or_block(vw), _packed_or_block(qw), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header)
+    ok = _blocks_ok(kw, vw, nh, nlon_in, nlon_out)
+    return forward_lse(_packed_or_block(kw, ok), _packed_or_block(vw, ok), _packed_or_block(qw, ok), quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out, plan, plan_header)
 
 
 @_neighborhood_s2_attention_saved.register_fake
@@ -180,8 +240,9 @@ def _setup_context_saved(ctx, inputs, output):
 
 def _neighborhood_s2_attention_bwd_saved(ctx, grad_output, grad_lse):
     col_idx, row_off, quad_weights, kw, vw, qw = ctx.saved_tensors
+    ok = _blocks_ok(kw, vw, ctx.nh, ctx.nlon_in, ctx.nlon_out)
     dkw, dvw, dqw = backward_saved(
-        _packed_or_block(kw), _packed_or_block(vw), _packed_or_block(qw), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in,
+        _packed_or_block(kw, ok), _packed_or_block(vw, ok), _packed_or_block(qw, ok), grad_output.contiguous(), ctx.y, ctx.lse, quad_weights, col_idx, row_off, ctx.nh, ctx.nlon_in,
         ctx.nlat_out, ctx.nlon_out, ctx.plan, ctx.plan_header,
     )  # fmt: skip
     return dkw, dvw, dqw, None, None, None, None, None, None, None, None, None
@@ -629,9 +690,3 @@ def backward_ring_step_upsample_pass2(
 @backward_ring_step_upsample_pass2.register_fake
 def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_norm_buf, dkx, dvx, quad_weights, col_idx, row_off, nlon_in, nlon_out_global, pscale_out, lon_lo_kx, lat_halo_start, nlat_out, nlon_out):
     return None
-
-
-def takes_column_blocks(dtype: torch.dtype, ck: int, cv: int, nlon_in: int, nlon_out: int) -> bool:
-    """True for the shapes whose kernels read q, k, v in place out of a wider buffer and write dq, dk, dv into one
-    (fp32 heads of 32 channels on at least 64 longitudes per virtual latitude: the hybrid kernels)."""
-    return dtype == torch.float32 and ck == 32 and cv == 32 and min(nlon_in, nlon_out) >= 64
