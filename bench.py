@@ -16,6 +16,8 @@ Reported alongside the throughput:
   cpu_baseline  the reference's own CPU operators (oracle/_ref, its release flags, OpenMP) and the C restatement of them (oracle/)
                 on a bounded sample of the same workload, on this machine's host cores
   other_configs op-level forward and backward times of the other four benchmark configurations
+  published_shapes  the reference's own published benchmark shapes (module level, forward and backward timed separately as there)
+  reference_signature_ms_per_step  the same step through the operators with the reference's exact signatures
 """
 
 import argparse
@@ -159,12 +161,8 @@ def time_other_config(name, device, steps=3, cpu=False):
         from oracle import cpu_attention as oracle
 
         hk, hv, hq, hg, hw, hc, hr = [t.cpu() for t in (k, v, q, dy, w, col, roff)]
-        t0 = time.perf_counter()
-        oracle.forward_f32(hk, hv, hq, hw, hc, hr, nh, fast=True)
-        t1 = time.perf_counter()
-        oracle.backward_f32(hk, hv, hq, hg, hw, hc, hr, nh, fast=True)
-        t2 = time.perf_counter()
-        res["cpu_port_fwd_ms"], res["cpu_port_bwd_ms"] = 1e3 * (t1 - t0), 1e3 * (t2 - t1)
+        res["cpu_port_fwd_ms"] = 1e3 * best_time(timed_calls(lambda: oracle.forward_f32(hk, hv, hq, hw, hc, hr, nh, fast=True), CPU_REPEAT))
+        res["cpu_port_bwd_ms"] = 1e3 * best_time(timed_calls(lambda: oracle.backward_f32(hk, hv, hq, hg, hw, hc, hr, nh, fast=True), CPU_REPEAT))
     return res
 
 
@@ -249,6 +247,106 @@ def time_ring_steps(device, nchunk=4, reps=2):
     return res
 
 
+# The reference's own published benchmark shapes (benchmarks/reference_results.csv:11-84; benchmarks/attention.py:71-112): B = 1, 64 channels, one head,
+# equiangular grids; published there for H100 / GB200 / GB300 only, so the figures beside them are context, not a baseline for this hardware.
+PUBLISHED_SHAPES = [
+    # (in_shape, out_shape, theta_cutoff, published H100 fp32 fwd ms, bwd ms, csv line)
+    ((180, 360), (180, 360), 0.017, 0.550, 1.115, 12),
+    ((180, 360), (180, 360), 0.03, 0.801, 1.781, 15),
+    ((360, 720), (360, 720), 0.017, 3.150, 7.394, 18),
+    ((360, 720), (360, 720), 0.03, 7.764, 19.431, 21),
+    ((360, 720), (180, 360), 0.017, 1.689, 3.499, 24),
+    ((360, 720), (180, 360), 0.03, 2.705, 6.049, 27),
+    ((180, 360), (360, 720), 0.03, 10.987, 19.280, 33),
+]
+
+
+def time_published_shapes(device, warmup=3, iters=20):
+    """Module-level forward and backward of the reference's published shapes, timed separately with device events around each
+    (3 warm-up + 20 iterations, upstream gradient of ones, as benchmarks/attention.py:71-112 and benchmarks/bench.py:268-323 do),
+    plus the op alone (forward_lse / backward_saved on the projected tensors) for the same shapes."""
+    from torch_harmonics_amd import NeighborhoodAttentionS2, ops
+
+    res = []
+    for ins, outs, tc, h_f, h_b, line in PUBLISHED_SHAPES:
+        torch.manual_seed(333)
+        m = NeighborhoodAttentionS2(64, ins, outs, num_heads=1, theta_cutoff=tc).to(device)
+        same = ins == outs
+        xq = torch.randn(1, 64, *outs, device=device, requires_grad=True)
+        xk = xq if same else torch.randn(1, 64, *ins, device=device, requires_grad=True)
+
+        def fwd():
+            return m(xq) if same else m(xq, xk, xk)
+
+        for _ in range(warmup):
+            o = fwd()
+            o.backward(torch.ones_like(o))
+        torch.cuda.synchronize()
+        tf = tb = 0.0
+        for _ in range(iters):
+            m.zero_grad(set_to_none=True)
+            xq.grad = None
+            if xk is not xq:
+                xk.grad = None
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+            e[0].record()
+            o = fwd()
+            e[1].record()
+            o.backward(torch.ones_like(o))
+            e[2].record()
+            torch.cuda.synchronize()
+            tf += e[0].elapsed_time(e[1])
+            tb += e[1].elapsed_time(e[2])
+        # the op alone on N(0,1) tensors of the projected shapes
+        (Hi, Wi), (Ho, Wo) = ins, outs
+        g = torch.Generator(device=device).manual_seed(333)
+        k = torch.randn(1, Hi, Wi, 64, device=device, generator=g)
+        v = torch.randn(1, Hi, Wi, 64, device=device, generator=g)
+        q = torch.randn(1, Ho, Wo, 64, device=device, generator=g) / 8.0
+        dy = torch.ones(1, Ho, Wo, 64, device=device)
+        geo = (m.quad_weights, m.psi_col_idx, m.psi_roff_idx, 1, Wi, Ho, Wo)
+        y, lse = ops.forward_lse(k, v, q, *geo)
+        ops.backward_saved(k, v, q, dy, y, lse, *geo)
+        torch.cuda.synchronize()
+        of = ob = 0.0
+        for _ in range(iters):
+            e = [torch.cuda.Event(enable_timing=True) for _ in range(3)]
+            e[0].record()
+            y, lse = ops.forward_lse(k, v, q, *geo)
+            e[1].record()
+            ops.backward_saved(k, v, q, dy, y, lse, *geo)
+            e[2].record()
+            torch.cuda.synchronize()
+            of += e[0].elapsed_time(e[1])
+            ob += e[1].elapsed_time(e[2])
+        nnz = m.psi_col_idx.numel()
+        pairs = (Wi if m.upsample else Wo) * nnz
+        res.append({
+            "shape": f"{Hi}x{Wi} -> {Ho}x{Wo}", "theta_cutoff": tc, "nnz": nnz, "pairs": pairs,
+            "module_fwd_ms": tf / iters, "module_bwd_ms": tb / iters, "op_fwd_ms": of / iters, "op_bwd_ms": ob / iters,
+            "published_h100_fwd_ms": h_f, "published_h100_bwd_ms": h_b, "published_source": f"benchmarks/reference_results.csv:{line}",
+        })  # fmt: skip
+        del m, xq, xk, k, v, q, dy, y, lse
+    return res
+
+
+CPU_REPEAT = 4  # 1 warm-up + 3 timed calls for the CPU legs that take under about 2 s
+
+
+def best_time(seconds):
+    """Minimum over the timed calls: the first call is a warm-up when there is more than one."""
+    return min(seconds[1:]) if len(seconds) > 1 else seconds[0]
+
+
+def timed_calls(f, repeat):
+    out = []
+    for _ in range(repeat):
+        t0 = time.perf_counter()
+        f()
+        out.append(time.perf_counter() - t0)
+    return out
+
+
 def cpu_sample(cfg, col, ro):
     """The bounded sample of a workload that the CPU legs time: the first four heads and every 6th output latitude (both pole
     rows included, so the reference backward's per-neighbor scratch is sized by the longest row, as in the full problem)."""
@@ -285,7 +383,7 @@ def reference_cpu_times(config_name, others):
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
     jobs, keys = [], []
 
-    def add(key, cfg, col, ro, nh, nlat_out, bwd):
+    def add(key, cfg, col, ro, nh, nlat_out, bwd, slow_bwd=False):
         (Hi, Wi), (_, Wo) = cfg["in_shape"], cfg["out_shape"]
         ck = cfg["C"] // cfg["nh"]
         w = ogeo.attention_quad_weights(Hi, Wi, cfg["grid_in"])
@@ -293,16 +391,17 @@ def reference_cpu_times(config_name, others):
         vv = {"randn": [cfg["B"], Hi, Wi, nh * ck], "seed": 2, "scale": 1.0}
         qq = {"randn": [cfg["B"], nlat_out, Wo, nh * ck], "seed": 3, "scale": 1.0 / math.sqrt(ck)}
         gg = {"randn": [cfg["B"], nlat_out, Wo, nh * ck], "seed": 4, "scale": 1.0}
-        jobs.append(dict(op="forward", args=[kk, vv, qq, w, col, ro, nh, Wi, nlat_out, Wo], discard=True))
+        # calls expected to take under about 2 s are repeated: 1 warm-up + 3 timed, the minimum is reported; the long ones run once
+        jobs.append(dict(op="forward", args=[kk, vv, qq, w, col, ro, nh, Wi, nlat_out, Wo], discard=True, repeat=CPU_REPEAT))
         keys.append((key, "fwd_ms"))
         if bwd:
-            jobs.append(dict(op="backward", args=[dict(kk), dict(vv), dict(qq), gg, w, col, ro, nh, Wi, nlat_out, Wo], discard=True))
+            jobs.append(dict(op="backward", args=[dict(kk), dict(vv), dict(qq), gg, w, col, ro, nh, Wi, nlat_out, Wo], discard=True, repeat=1 if slow_bwd else CPU_REPEAT))
             keys.append((key, "bwd_ms"))
 
     cfg = CONFIGS[config_name]
     col, ro = ogeo.neighborhood_csr(cfg["in_shape"], cfg["out_shape"], cfg["grid_in"], cfg["grid_out"], cfg["theta_cutoff"])
     smp = cpu_sample(cfg, col, ro)
-    add("sample", cfg, smp["col"], smp["ro"], smp["nh"], len(smp["rows"]), True)
+    add("sample", cfg, smp["col"], smp["ro"], smp["nh"], len(smp["rows"]), True, slow_bwd=smp["pairs"] > 5e7)
     if smp["full"]:
         add("full", cfg, col, ro, cfg["nh"], cfg["out_shape"][0], False)
     for name in others:
@@ -312,7 +411,8 @@ def reference_cpu_times(config_name, others):
     res = reference.run(jobs, threads=cores)
     out = {}
     for (key, what), r in zip(keys, res):
-        out.setdefault(key, {})[what] = 1e3 * r["seconds"][0]
+        out.setdefault(key, {})[what] = 1e3 * best_time(r["seconds"])
+        out[key][what.replace("_ms", "_runs")] = len(r["seconds"])
     return out
 
 
@@ -337,19 +437,15 @@ def cpu_baseline(cfg, mod, k, v, q, dy, ref_times=None):
     gs = dy[:, rows][..., : nh_s * cv].float().cpu().contiguous()
     w = mod.quad_weights.float().cpu()
     cores = int(os.environ.get("OMP_NUM_THREADS", os.cpu_count() or 1))
-    t0 = time.perf_counter()
-    oracle.forward_f32(ks, vs, qs, w, col_s, ro_s, nh_s, fast=True)
-    t1 = time.perf_counter()
-    oracle.backward_f32(ks, vs, qs, gs, w, col_s, ro_s, nh_s, fast=True)
-    t2 = time.perf_counter()
-    port = {"fwd_ms": 1e3 * (t1 - t0), "bwd_ms": 1e3 * (t2 - t1)}
+    slow_bwd = pairs > 5e7
+    t_f = timed_calls(lambda: oracle.forward_f32(ks, vs, qs, w, col_s, ro_s, nh_s, fast=True), CPU_REPEAT)
+    t_b = timed_calls(lambda: oracle.backward_f32(ks, vs, qs, gs, w, col_s, ro_s, nh_s, fast=True), 1 if slow_bwd else CPU_REPEAT)
+    port = {"fwd_ms": 1e3 * best_time(t_f), "bwd_ms": 1e3 * best_time(t_b)}
     # The forward alone has no scratch and is feasible in full: all heads, all latitudes of the workload (the reference backward
     # would need 2 * B * heads * nlat_out * nlon_out * max_row_len floats, 383 GB at 721x1440 with 8 heads).
     if smp["full"]:
         kf, vf, qf = k.float().cpu().contiguous(), v.float().cpu().contiguous(), q.float().cpu().contiguous()
-        t0 = time.perf_counter()
-        oracle.forward_f32(kf, vf, qf, w, col, ro, cfg["nh"], fast=True)
-        port["full_forward_ms"] = 1e3 * (time.perf_counter() - t0)
+        port["full_forward_ms"] = 1e3 * best_time(timed_calls(lambda: oracle.forward_f32(kf, vf, qf, w, col, ro, cfg["nh"], fast=True), CPU_REPEAT))
 
     timed, kind = port, "port"
     if ref_times and "sample" in ref_times:
@@ -363,7 +459,8 @@ def cpu_baseline(cfg, mod, k, v, q, dy, ref_times=None):
         "kind": kind,
         "sample": f"{nh_s} of {cfg['nh']} heads x {len(rows)} of {Ho} output latitudes (every {smp['stride']}th, both poles) = {pairs} pairs; "
         f"fwd {timed['fwd_ms']:.0f} ms + bwd {timed['bwd_ms']:.0f} ms; reference bwd scratch {smp['scratch_gb']:.1f} GB"
-        + ("; the reference's own CPU operators on N(0,1) tensors of these shapes, in a child process" if kind == "reference" else ""),
+        + f"; calls under about 2 s: 1 warm-up + {CPU_REPEAT - 1} timed, minimum; the backward of a large sample: one call"
+        + ("; the reference's own CPU operators in a child process, on the child's own N(0,1) tensors of these shapes (not the workload's smooth fields)" if kind == "reference" else ""),
         "fwd_ms": timed["fwd_ms"],
         "bwd_ms": timed["bwd_ms"],
     }
@@ -438,6 +535,20 @@ def main():
         step()
     torch.cuda.synchronize()
     ms_step = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # the operators with the reference's exact signatures (attention_kernels::forward / backward: nothing handed from the forward to
+    # the backward, which recomputes y and the softmax normaliser first), same tensors
+    def ref_step():
+        yy = ops.forward(k, v, q, wq, ci, ro, nh, Wi, Ho, Wo)
+        return yy, ops.backward(k, v, q, dy, wq, ci, ro, nh, Wi, Ho, Wo)
+
+    ref_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        ref_step()
+    torch.cuda.synchronize()
+    ms_ref_step = 1e3 * (time.perf_counter() - t0) / args.steps
 
     # ---- per-kernel durations: events on the launch stream around each launch, same K steps ----
     plan = get_plan(ci, ro, Hi, Wi, Ho, Wo)
@@ -541,6 +652,7 @@ def main():
             "kernel_ms": dom_ms,
         },
         "kernel_ms": {"fwd": t_fwd, "dq": t_dq, "dkdv": t_dkdv},
+        "reference_signature_ms_per_step": ms_ref_step,  # attention_kernels::forward + attention_kernels::backward (forward recomputed in the backward)
         "step_hbm_frac": step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBS,
         "step_matrix_frac": flops_alg / (ms_step * 1e-3) / 1e12 / matrix_peak,
         "step_fp32_valu_frac": flops_alg / (ms_step * 1e-3) / 1e12 / FP32_VALU_PEAK_TFLOPS,
@@ -579,6 +691,7 @@ def main():
             if name in out["other_configs"]:
                 out["other_configs"][name]["cpu_reference_fwd_ms"], out["other_configs"][name]["cpu_reference_bwd_ms"] = t["fwd_ms"], t["bwd_ms"]
         out["ring_steps"] = time_ring_steps(dev)
+        out["published_shapes"] = time_published_shapes(dev)
 
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(cfg, mod, k, v, q, dy, ref_times)
