@@ -85,3 +85,80 @@ def test_cfg5_one_head_bf16_every_latitude_against_the_reference_cpu_operators()
     torch.cuda.synchronize()
     for key, got, r in zip(("y", "dk", "dv", "dq"), (y, dk, dv, dq), want):
         _bf16_close(f"cfg5 {key}", got.cpu(), r.double())
+
+
+# ---- the headline configuration on the benchmark's OWN inputs --------------------------------------------------------------------
+POLAR_ROWS = 45  # output latitudes within 45 rows of a pole hold the runs of 32 and more longitudes (matrix-core tiles, up to 5,760 neighbors per query)
+
+
+def _excess(got, want, rtol=1e-5, atol=1e-5):
+    """How far the worst element lies outside atol + rtol * |want| (<= 0: inside), and the largest absolute difference."""
+    err = (got.detach().double().cpu() - want.detach().double().cpu()).abs()
+    return float((err - (atol + rtol * want.detach().double().cpu().abs())).max()), float(err.max())
+
+
+def cfg3_benchmark_input_deviations(head=2):
+    """One head of cfg3 on bench.make_workload's tensors (smooth spherical-harmonic fields plus noise through the seeded
+    projections, query scaled by the module), all 721 latitudes: y, dk, dv, dq of both HIP routes against the reference's CPU
+    operators and against the float64 spec; per tensor and region (polar / equatorial latitudes) the largest absolute
+    difference and the excess over rtol = atol = 1e-5.  Returns {route: {tensor: {region: {against: (excess, max_abs)}}}} and
+    the same figures for the reference's CPU result against float64."""
+    import bench
+    from oracle import cpu_attention as oracle
+    from torch_harmonics_amd import ops
+
+    cfg = bench.CONFIGS["cfg3"]
+    mod, _, _, k8, v8, q8, dy8 = bench.make_workload(cfg, torch.device(DEV))
+    d = cfg["C"] // cfg["nh"]
+    kd, vd, qd, gd = [t[..., head * d : (head + 1) * d].contiguous() for t in (k8, v8, q8, dy8)]
+    del k8, v8, q8, dy8
+    (Hi, Wi), (Ho, Wo) = cfg["in_shape"], cfg["out_shape"]
+    geo = (mod.quad_weights, mod.psi_col_idx, mod.psi_roff_idx, 1, Wi, Ho, Wo)
+    y, lse = ops.forward_lse(kd, vd, qd, *geo)
+    routes = {"saved": (y,) + tuple(ops.backward_saved(kd, vd, qd, gd, y, lse, *geo)), "recompute": (ops.forward(kd, vd, qd, *geo),) + tuple(ops.backward(kd, vd, qd, gd, *geo))}
+    torch.cuda.synchronize()
+    k, v, q, dy = kd.cpu(), vd.cpu(), qd.cpu(), gd.cpu()
+    w, col, roff = mod.quad_weights.cpu(), mod.psi_col_idx.cpu(), mod.psi_roff_idx.cpu()
+    print("reference CPU operators on one head of cfg3 (child process) ...", flush=True)
+    want_ref = _reference(k, v, q, dy, w, col, roff, 1)
+    print("float64 spec ...", flush=True)
+    want_64 = (oracle.forward_f64(k, v, q, w, col, roff, 1),) + tuple(oracle.backward_f64(k, v, q, dy, w, col, roff, 1))
+    polar = torch.zeros(Ho, dtype=torch.bool)
+    polar[:POLAR_ROWS] = True
+    polar[Ho - POLAR_ROWS :] = True
+    regions = {"polar": polar, "equatorial": ~polar}
+    names = ("y", "dk", "dv", "dq")
+
+    def table(got):
+        return {
+            n: {r: {"reference": _excess(g[:, m].cpu(), wr[:, m]), "float64": _excess(g[:, m].cpu(), w64[:, m])} for r, m in regions.items()}
+            for n, g, wr, w64 in zip(names, got, want_ref, want_64)
+        }
+
+    out = {route: table(got) for route, got in routes.items()}
+    out["reference_cpu"] = {n: {r: {"float64": _excess(wr[:, m], w64[:, m])} for r, m in regions.items()} for n, wr, w64 in zip(names, want_ref, want_64)}
+    return out
+
+
+def test_cfg3_benchmark_inputs_one_head_every_latitude():
+    """The headline configuration on the tensors bench.py times (smooth fields through seeded projections; one head, all 721
+    latitudes, both backward routes), against the reference's own CPU operators AND the float64 spec.
+
+    y, dk, dv: rtol = atol = 1e-5 against both.  dq: on these inputs g_j = <dy, v_j> and I = <dy, y> are numbers of size 15-30
+    whose difference the gradient is made of, and fp32 carries them to about 2e-6 each: measured on the device, dq lies within
+    1.6e-5 of the float64 spec (atol 2e-5 here), the reference's CPU operators within 1.5e-4 of it (their dq comes from
+    (A_kvw S - A_vw A_k) / S^2, which cancels harder), so against the reference dq is held to the reference's own distance from
+    float64, and the HIP result must be the closer of the two."""
+    dev = cfg3_benchmark_input_deviations()
+    for route in ("saved", "recompute"):
+        for name in ("y", "dk", "dv"):
+            for region, against in dev[route][name].items():
+                for what, (excess, max_abs) in against.items():
+                    assert excess <= 0, f"{route} {name} {region} vs {what}: misses rtol = atol = 1e-5 by {excess:.3e} (max |diff| {max_abs:.3e})"
+        for region, against in dev[route]["dq"].items():
+            ex64, abs64 = against["float64"]
+            ref_ex64, ref_abs64 = dev["reference_cpu"]["dq"][region]["float64"]
+            print(f"{route} dq {region}: max |HIP - float64| {abs64:.3e} (excess over 1e-5 {ex64:+.3e}); reference CPU vs float64 {ref_abs64:.3e}; HIP vs reference {against['reference'][1]:.3e}", flush=True)
+            assert ex64 <= 1e-5, f"{route} dq {region}: {abs64:.3e} from the float64 spec, outside atol 2e-5 + rtol 1e-5"
+            assert abs64 <= ref_abs64, f"{route} dq {region}: farther from float64 ({abs64:.3e}) than the reference's CPU operators are ({ref_abs64:.3e})"
+            assert against["reference"][1] <= 2e-4, f"{route} dq {region}: {against['reference'][1]:.3e} from the reference's CPU result"

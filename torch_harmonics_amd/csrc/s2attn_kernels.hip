@@ -198,6 +198,20 @@ __device__ inline float xor16_max(float x)
 // passed through settle() right before the loop.  The empty asm uses the register, so the wait for the load is placed
 // there; without it the compiler (which cannot see that the loop only runs on a path that has already waited) puts a
 // vmcnt(0) at the first use INSIDE the loop, and that also waits for the tile prefetch issued just before it, every step.
+// Uniform reads of the plan and the weights inside a walk that also stores to global memory: through the constant address
+// space the load stays a scalar load (neither array is ever written by a kernel); through a plain pointer the compiler must
+// assume the store may have changed it and makes it a vector load with a full wait.
+template <typename V> __device__ inline V const_load(const V *p)
+{
+    typedef const V __attribute__((address_space(4))) * cptr;
+    return *(cptr)(p);
+}
+__device__ inline Run const_load(const Run *p)
+{
+    typedef int i4v __attribute__((ext_vector_type(4)));
+    const i4v r = const_load(reinterpret_cast<const i4v *>(p));
+    return Run{r[0], r[1], r[2], r[3]};
+}
 __device__ inline void settle(float &x) { asm("" : "+v"(x)); }
 __device__ inline void settle(uint4 &x) { asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w)); }
 template <typename V, int N> __device__ inline void settle(V (&x)[N])
@@ -1660,6 +1674,18 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
 #pragma unroll
     for (int v = 0; v < 16; v++) acc[v] = 0.f;
     float m = NEG_BIG, S = 0.f;
+    // Two-level summation on long rows (fp32 storage): every FLUSH matrix-core steps the running sums are added to a second
+    // level and start again from zero, so the rounding of each addition is relative to a short partial sum and the second
+    // level sees few additions (a pole row has 5,760 terms per query; summed in one chain y is off by 2-3e-6 of its size,
+    // which the backward's <dy, y> turns into 2e-5 of dq).  The second level of the output sums lives in the output row
+    // itself (each lane owns its 16 values of y), that of the normaliser in S2; part_scale collects the rescalings since
+    // the last flush.
+    constexpr bool two_level = std::is_same<T, float>::value;
+    constexpr int FLUSH = 8;
+    float S2 = 0.f, part_scale = 1.f;
+    int nflush = 0;
+    bool have_part = false;
+    T *const yout = static_cast<T *>(a.y) + pt * a.ldy + (size_t)h * 32 + 4 * half;
 
     int ri = a.goff[ho];
     const int rend = a.goff[ho + 1];
@@ -1673,7 +1699,7 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
         vt.fetch(vx + (size_t)key_row(a, rn.lat, rn.pad) * ldv, ldv * a.kps, c0, a.Wi, lane, fifth);
     };
     if (ri < rend) {
-        run = a.gruns[ri];
+        run = const_load(a.gruns + ri);
         fetch(run, 0);
         kt.commit(Ks, lane, !run_is_dense(run.len));
         vt.commit(Vs, lane, !run_is_dense(run.len));
@@ -1681,14 +1707,14 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     __syncthreads();
 
     while (ri < rend) {
-        const float w = a.quad_w[run.pad];
+        const float w = const_load(a.quad_w + run.pad);
         const int len = run.len;
         int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
         if (run_done(len, npos)) {
             nri++;
             npos = 0;
-            if (nri < rend) nrun = a.gruns[nri];
+            if (nri < rend) nrun = const_load(a.gruns + nri);
         }
         const bool more = nri < rend;
         if (more) fetch(nrun, npos);
@@ -1726,6 +1752,8 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
             if (__any(mn > m)) {
                 const float corr = fast_exp2(m - mn);
                 S *= corr;
+                S2 *= corr;
+                part_scale *= corr;
 #pragma unroll
                 for (int v = 0; v < 16; v++) acc[v] *= corr;
             }
@@ -1754,6 +1782,26 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
                 const float x = Vs[kappa(v, half) * MLK + j];
                 acc = __builtin_amdgcn_mfma_f32_32x32x2f32(x, sc[v], acc, 0, 0, 0);
             }
+            if (two_level && ++nflush == FLUSH) {
+                if (mine) {
+#pragma unroll
+                    for (int g = 0; g < 4; g++) {
+                        float4 o = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
+                        if (have_part) {
+                            const float4 old = load4(yout + 8 * g);
+                            o.x = fmaf(old.x, part_scale, o.x), o.y = fmaf(old.y, part_scale, o.y), o.z = fmaf(old.z, part_scale, o.z), o.w = fmaf(old.w, part_scale, o.w);
+                        }
+                        store4(yout + 8 * g, o);
+                    }
+                }
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[v] = 0.f;
+                S2 += S;
+                S = 0.f;
+                part_scale = 1.f;
+                nflush = 0;
+                have_part = true;
+            }
         } else {
             // ---- vector chunk: neighbors pos .. pos + L - 1, query j reads staged rows j + t; one pass, lazy maximum ----
             const int L = min(VC, len - pos);
@@ -1770,6 +1818,8 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
                     if (__any(sv > m + RESCALE_THR)) {
                         const float mn = sv > m + RESCALE_THR ? sv : m, corr = fast_exp2(m - mn);
                         S *= corr;
+                        S2 *= corr;
+                        part_scale *= corr;
 #pragma unroll
                         for (int v = 0; v < 16; v++) acc[v] *= corr;
                         m = mn;
@@ -1799,11 +1849,19 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
     }
 
     if (mine) {
+        if (two_level && have_part) {
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                const float4 old = load4(yout + 8 * g);
+                acc[4 * g] = fmaf(old.x, part_scale, acc[4 * g]), acc[4 * g + 1] = fmaf(old.y, part_scale, acc[4 * g + 1]);
+                acc[4 * g + 2] = fmaf(old.z, part_scale, acc[4 * g + 2]), acc[4 * g + 3] = fmaf(old.w, part_scale, acc[4 * g + 3]);
+            }
+            S += S2;
+        }
         if (a.lse && half == 0) a.lse[((size_t)bh * a.Ho + ho) * a.Wo + w0 + j] = m + fast_log2(S);
         const float inv = 1.0f / S;
-        T *y = static_cast<T *>(a.y) + pt * a.ldy + (size_t)h * 32 + 4 * half;
 #pragma unroll
-        for (int g = 0; g < 4; g++) store4(y + 8 * g, make_float4(acc[4 * g] * inv, acc[4 * g + 1] * inv, acc[4 * g + 2] * inv, acc[4 * g + 3] * inv));
+        for (int g = 0; g < 4; g++) store4(yout + 8 * g, make_float4(acc[4 * g] * inv, acc[4 * g + 1] * inv, acc[4 * g + 2] * inv, acc[4 * g + 3] * inv));
     }
 }
 
