@@ -213,6 +213,7 @@ __device__ inline Run const_load(const Run *p)
     return Run{r[0], r[1], r[2], r[3]};
 }
 __device__ inline void settle(float &x) { asm("" : "+v"(x)); }
+__device__ inline void settle(unsigned &x) { asm("" : "+v"(x)); }
 __device__ inline void settle(uint4 &x) { asm("" : "+v"(x.x), "+v"(x.y), "+v"(x.z), "+v"(x.w)); }
 template <typename V, int N> __device__ inline void settle(V (&x)[N])
 {
@@ -1609,6 +1610,25 @@ template <typename T> struct Tile40 {
             raw[4] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
         }
     }
+    // The 32 rows of a split tile: lane holds rows 4 (lane / 8) + it (one commit instruction then writes rows 0, 4, .. 28 + it,
+    // whose LDS words tile the banks exactly; rows it * 8 + lane / 8 would collide two ways).
+    __device__ inline void fetch_split(const T *src, unsigned ld, int c0, int W, int lane)
+    {
+        const unsigned lane_off = 4u * (unsigned)(lane >> 3) * ld + 4u * (unsigned)(lane & 7);
+        if (c0 + MT <= W) {
+            const T *base = src + (size_t)c0 * ld;
+#pragma unroll
+            for (int it = 0; it < 4; it++) raw[it] = *reinterpret_cast<const raw_t *>(base + (size_t)it * ld + lane_off);
+            return;
+        }
+        const int colA = c0 + 4 * (lane >> 3), cb = 4 * (lane & 7);
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            int col = colA + it;
+            col -= (col >= W) ? W : 0;
+            raw[it] = *reinterpret_cast<const raw_t *>(src + (size_t)(__umul24(col, ld) + cb));
+        }
+    }
     __device__ inline void commit(float *dst, int lane, bool fifth) const
     {
         const int r0 = lane >> 3, cb = 4 * (lane & 7);
@@ -1639,6 +1659,7 @@ __device__ inline int run_stride(int len) { return run_is_dense(len) ? MT : VC; 
     const int nvalid = min(MT, (W_TILED)-w0);
 
 #include "s2attn_pair.hpp"
+#include "s2attn_split.hpp"
 
 // forward, head dim 32.  Lane (j, half) keeps channels 8g + 4 half + e (g, e < 4) of query j: that is the
 // accumulator layout of the matrix-core product, and the vector path for short runs uses the same one (each half
@@ -2036,11 +2057,13 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
 // dV^T += dY^T P.  Short runs: vector chunks of VC query rows starting at row pos, key j reads staged rows j + i.
 template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(const Args a)
 {
-    __shared__ __attribute__((aligned(16))) float Qs[MR * MLK];
-    __shared__ __attribute__((aligned(16))) float Gs[MR * MLK];
-    __shared__ __attribute__((aligned(16))) float Ls[MR];
-    __shared__ __attribute__((aligned(16))) float Is[MR];
-    __shared__ __attribute__((aligned(16))) int Rs[8 * S2_PAIR_MAX_RUNS];
+    // fp32 tiles of 40 rows for vector chunks (and the merged runs of a latitude pair behind them), or split tiles of 32 rows for
+    // matrix-core steps, in one buffer (see the forward); the statistics of the staged rows behind it
+    __shared__ __attribute__((aligned(16))) char smem[2 * SPLIT_TILE_BYTES + 2 * MR * 4];
+    float *const Qs = reinterpret_cast<float *>(smem), *const Gs = Qs + MR * MLK;
+    int *const Rs = reinterpret_cast<int *>(Gs + MR * MLK);
+    char *const Qb = smem, *const Gb = smem + SPLIT_TILE_BYTES;
+    float *const Ls = reinterpret_cast<float *>(smem + 2 * SPLIT_TILE_BYTES), *const Is = Ls + MR;
 
     S2_MFMA_IDS(a.Wi)
     const int hi = a.sitems[2 * rowsel], pair = a.sitems[2 * rowsel + 1];
@@ -2055,18 +2078,11 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     const bool mine = j < nvalid;
     const size_t pt = (size_t)key_point(a, b, hi, hi / a.kps) + (size_t)(w0 + (mine ? j : 0)) * a.kps;
 
-    float kb[16], vb[16];
-    {
-        const T *krow = static_cast<const T *>(a.k) + pt * a.ldk + (size_t)h * 32 + 4 * half;
-        const T *vrow = static_cast<const T *>(a.v) + pt * a.ldv + (size_t)h * 32 + 4 * half;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float4 x = load4(krow + 8 * g);
-            const float4 z = load4(vrow + 8 * g);
-            kb[4 * g] = x.x * LOG2E, kb[4 * g + 1] = x.y * LOG2E, kb[4 * g + 2] = x.z * LOG2E, kb[4 * g + 3] = x.w * LOG2E;
-            vb[4 * g] = z.x, vb[4 * g + 1] = z.y, vb[4 * g + 2] = z.z, vb[4 * g + 3] = z.w;
-        }
-    }
+    // k (times log2 e) and v in the form the current run needs, one set of registers each (OwnRegs, see the forward)
+    OwnRegs ko, vo;
+    bool own_split = false;
+    const T *const krow = static_cast<const T *>(a.k) + pt * a.ldk + (size_t)h * 32 + 4 * half;
+    const T *const vrow = static_cast<const T *>(a.v) + pt * a.ldv + (size_t)h * 32 + 4 * half;
     f16v dkt, dvt;
 #pragma unroll
     for (int v = 0; v < 16; v++) {
@@ -2084,16 +2100,25 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     auto fetch = [&](const Run &rn, int p) {
         int c0 = (w0 - rn.ws - rn.len + 1 + p) % a.Wo; // longitude of staged row 0
         c0 += (c0 < 0) ? a.Wo : 0;
-        const bool fifth = !run_is_dense(rn.len);
-        qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldq, ldq * a.qps, c0, a.Wo, lane, fifth);
-        gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldg, ldg * a.qps, c0, a.Wo, lane, fifth);
+        if (run_is_dense(rn.len)) {
+            qt.fetch_split(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldq, ldq * a.qps, c0, a.Wo, lane);
+            gt.fetch_split(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldg, ldg * a.qps, c0, a.Wo, lane);
+        } else {
+            qt.fetch(qy + (size_t)query_row(a, rn.lat, rn.pad) * ldq, ldq * a.qps, c0, a.Wo, lane, true);
+            gt.fetch(gy + (size_t)query_row(a, rn.lat, rn.pad) * ldg, ldg * a.qps, c0, a.Wo, lane, true);
+        }
         int col = c0 + lane; // lanes 0..39 fetch the statistics of the staged rows
         col -= (col >= a.Wo) ? a.Wo : 0;
         if (lane < MR) st = stats[(size_t)rn.lat * a.Wo + col];
     };
-    auto commit = [&](bool fifth) {
-        qt.commit(Qs, lane, fifth);
-        gt.commit(Gs, lane, fifth);
+    auto commit = [&](bool dense) {
+        if (dense) {
+            commit_split(qt, Qb, lane);
+            commit_split(gt, Gb, lane);
+        } else {
+            qt.commit(Qs, lane, true);
+            gt.commit(Gs, lane, true);
+        }
         if (lane < MR) {
             Ls[lane] = st.x;
             Is[lane] = st.y;
@@ -2102,14 +2127,23 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
     if (ri < rend) {
         run = a.sruns[ri];
         fetch(run, 0);
-        commit(!run_is_dense(run.len));
+        commit(run_is_dense(run.len));
     }
+    own_split = ri < rend && run_is_dense(run.len);
+    ko.load(krow, LOG2E, own_split);
+    vo.load(vrow, 1.0f, own_split);
     __syncthreads();
-    settle(kb);
-    settle(vb);
+    settle(ko.r);
+    settle(vo.r);
+    const int troff = tr_lane_offset(lane);
 
     while (ri < rend) {
         const int len = run.len;
+        if (run_is_dense(len) != own_split) {
+            own_split = run_is_dense(len);
+            ko.load(krow, LOG2E, own_split);
+            vo.load(vrow, 1.0f, own_split);
+        }
         int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
         if (run_done(len, npos)) {
@@ -2130,19 +2164,8 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
                 sc[v] = 0.f;
                 gc[v] = 0.f;
             }
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                const float4 x = *reinterpret_cast<const float4 *>(qq + 8 * g);
-                const float4 z = *reinterpret_cast<const float4 *>(gq + 8 * g);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.x, kb[4 * g + 0], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.x, vb[4 * g + 0], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.y, kb[4 * g + 1], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.y, vb[4 * g + 1], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.z, kb[4 * g + 2], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.z, vb[4 * g + 2], gc, 0, 0, 0);
-                sc = __builtin_amdgcn_mfma_f32_32x32x2f32(x.w, kb[4 * g + 3], sc, 0, 0, 0);
-                gc = __builtin_amdgcn_mfma_f32_32x32x2f32(z.w, vb[4 * g + 3], gc, 0, 0, 0);
-            }
+            sc = rows_times_regs(Qb + j * SPP + 32 * half, ko.terms(), sc);
+            gc = rows_times_regs(Gb + j * SPP + 32 * half, vo.terms(), gc);
             const bool edge = (r0 < MT - 1) || (r0 + MT - 1 >= len);
 #pragma unroll
             for (int g = 0; g < 4; g++) {
@@ -2162,15 +2185,21 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
                     gc[v] = p * (gc[v] - iv[e]);
                 }
             }
-#pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const float x = Qs[kappa(v, half) * MLK + j];
-                const float z = Gs[kappa(v, half) * MLK + j];
-                dkt = __builtin_amdgcn_mfma_f32_32x32x2f32(x, gc[v], dkt, 0, 0, 0);
-                dvt = __builtin_amdgcn_mfma_f32_32x32x2f32(z, sc[v], dvt, 0, 0, 0);
+            {
+                Terms3 cs;
+                split_regs(cs, gc);
+                dkt = cols_times_regs(Qb, troff, cs, dkt);
+            }
+            {
+                Terms3 ps;
+                split_regs(ps, sc);
+                dvt = cols_times_regs(Gb, troff, ps, dvt);
             }
         } else {
             const int L = min(VC, len - pos);
+            float kb[16], vb[16];
+            ko.floats(kb);
+            vo.floats(vb);
 #pragma unroll
             for (int i = 0; i < VC; i++) {
                 if (i < L) {
@@ -2197,7 +2226,7 @@ template <typename T> __global__ __launch_bounds__(64) void dkdv_mfma_kernel(con
         }
 
         __syncthreads();
-        if (more) commit(!run_is_dense(nrun.len));
+        if (more) commit(run_is_dense(nrun.len));
         __syncthreads();
         ri = nri;
         pos = npos;
