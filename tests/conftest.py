@@ -8,6 +8,10 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 
+# the modules built by the tests do not leave plan files in the user's cache directory (the cache has a test of its own)
+os.environ.setdefault("S2ATTN_CACHE_DIR", "off")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a ROCm GPU (run with -m gpu on an MI355X box)")
 

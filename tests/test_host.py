@@ -683,3 +683,51 @@ def test_projections_fed_from_and_to_nchw_match_plain_linear():
     g = torch.randn_like(o)
     for a, rr in zip(torch.autograd.grad(o, [y, w, b], g), torch.autograd.grad(r, [y, w, b], g)):
         assert torch.allclose(a, rr, atol=1e-8)
+
+
+def test_plan_blob_is_cached_on_disk(tmp_path, monkeypatch):
+    """A module's plan blob is written to $S2ATTN_CACHE_DIR by the first constructor and read back by the next one; a file that
+    does not describe the problem is ignored and replaced; "off" disables the cache."""
+    import os
+
+    from torch_harmonics_amd import NeighborhoodAttentionS2
+
+    monkeypatch.setenv("S2ATTN_CACHE_DIR", str(tmp_path))
+    kw = dict(in_channels=8, in_shape=(12, 24), out_shape=(6, 12), num_heads=2, theta_cutoff=0.5)
+    m1 = NeighborhoodAttentionS2(**kw)
+    files = sorted(os.listdir(tmp_path))
+    assert len(files) == 1 and files[0].startswith("plan_") and files[0].endswith(".npy")
+    stamp = os.stat(tmp_path / files[0]).st_mtime_ns
+    m2 = NeighborhoodAttentionS2(**kw)
+    assert torch.equal(m1.psi_plan, m2.psi_plan) and m1._psi_plan_header == m2._psi_plan_header
+    assert os.stat(tmp_path / files[0]).st_mtime_ns == stamp  # read, not rewritten
+    m3 = NeighborhoodAttentionS2(**{**kw, "theta_cutoff": 0.7})  # another psi: another file
+    assert len(os.listdir(tmp_path)) == 2 and not torch.equal(m3.psi_plan[: m1.psi_plan.numel()], m1.psi_plan)
+    (tmp_path / files[0]).write_bytes(b"not a plan")
+    m4 = NeighborhoodAttentionS2(**kw)
+    assert torch.equal(m4.psi_plan, m1.psi_plan)
+    import numpy as np
+
+    assert np.load(tmp_path / files[0]).shape == (m1.psi_plan.numel(),)  # rewritten
+    monkeypatch.setenv("S2ATTN_CACHE_DIR", "off")
+    for f in os.listdir(tmp_path):
+        os.remove(tmp_path / f)
+    NeighborhoodAttentionS2(**kw)
+    assert os.listdir(tmp_path) == []
+
+
+def test_module_constructor_time_at_the_headline_grid():
+    """721 x 1440 self-attention: psi from its structure plus the plan build stay far below a second (the reference's loop over
+    output latitudes takes seconds there)."""
+    import time
+
+    from torch_harmonics_amd import NeighborhoodAttentionS2
+    from torch_harmonics_amd.neighborhood import _neighborhood_cached, _segments_cached
+
+    _neighborhood_cached.cache_clear()
+    _segments_cached.cache_clear()
+    t0 = time.perf_counter()
+    m = NeighborhoodAttentionS2(16, (721, 1440), (721, 1440), num_heads=1, theta_cutoff=3 * math.pi / 720)
+    dt = time.perf_counter() - t0
+    print(f"constructor at 721x1440: {dt * 1e3:.0f} ms")
+    assert m.psi_col_idx.numel() == 99625 and dt < 1.0

@@ -18,7 +18,7 @@ from ._attention_utils import _check_dtypes_match, _check_extent, _check_ndim
 from ._layout import to_nchw, to_nhwc
 from .neighborhood import precompute_neighborhood_s2
 from .ops import neighborhood_s2_attention, takes_column_blocks
-from .plan import build_host_blob
+from .plan import cached_host_blob
 from .quadrature import precompute_latitudes
 
 __all__ = ["NeighborhoodAttentionS2"]
@@ -390,7 +390,9 @@ class NeighborhoodAttentionS2(nn.Module):
         # The kernels consume psi as a run-length plan (include/s2attn.h).  It is built here, on the host, from the CSR that was
         # just computed, and travels with the module as one more buffer, so no forward ever copies psi back from the device
         # (the reference re-sorts the CSR rows on the device in every call, attention_cuda_utils.cu:74-113).
-        plan = build_host_blob(col_idx, row_off, self.nlat_in, self.nlon_in, self.nlat_out, self.nlon_out)
+        # The blob is also kept on disk, keyed by what determines psi (see plan.cached_host_blob), so later processes skip the build.
+        psi_key = ("NeighborhoodAttentionS2", tuple(in_shape), tuple(out_shape), grid_in, grid_out, float(self.theta_cutoff).hex(), bool(self.upsample))
+        plan = cached_host_blob(psi_key, col_idx, row_off, self.nlat_in, self.nlon_in, self.nlat_out, self.nlon_out)
         self.register_buffer("psi_plan", plan.blob, persistent=False)
         self._psi_plan_header = list(plan.header)
 

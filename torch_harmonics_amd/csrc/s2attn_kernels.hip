@@ -1826,16 +1826,18 @@ template <typename T> __global__ __launch_bounds__(64) void fwd_mfma_kernel(cons
         } else {
             // ---- vector chunk: neighbors pos .. pos + L - 1, query j reads staged rows j + t; one pass, lazy maximum ----
             const int L = min(VC, len - pos);
+            // (LDS reads software-pipelined as in the pair path: K row of the next neighbor while this one's exponential and
+            // accumulation run, V row while its dot product does)
+            float4 x[4], z[4];
+            read_row(x, kq);
 #pragma unroll
             for (int t = 0; t < VC; t++) {
                 if (t < L) {
-                    float4 x[4], z[4];
-#pragma unroll
-                    for (int g = 0; g < 4; g++) {
-                        x[g] = *reinterpret_cast<const float4 *>(kq + t * MLK + 8 * g);
-                        z[g] = *reinterpret_cast<const float4 *>(vq + t * MLK + 8 * g);
-                    }
+                    read_row(z, vq + t * MLK);
                     const float sv = xor32_sum(dot16(qb, x));
+                    __builtin_amdgcn_sched_barrier(0);
+                    read_row(x, kq + (t + 1) * MLK); // (past the last neighbor: a row nobody uses, still inside the buffer)
+                    __builtin_amdgcn_sched_barrier(0);
                     if (__any(sv > m + RESCALE_THR)) {
                         const float mn = sv > m + RESCALE_THR ? sv : m, corr = fast_exp2(m - mn);
                         S *= corr;

@@ -133,17 +133,26 @@ __device__ inline void fwd_pair(const Args &a, float *Ks, float *Vs, int *Rs, in
         }
         const bool more = nri < rend;
         if (more) fetch(nrun, npos);
-        // One pass per band position: K row and V row are read together, the score goes straight into the accumulators.
-        // The running maximum is only a reference point of the exponentials, so it is moved lazily (see RESCALE_THR).
+        // One pass per band position, software-pipelined over the LDS reads: the K row of a position is read while the
+        // previous position's exponentials and accumulations run, its V row while its two dot products do, so a step does
+        // not begin by waiting a full LDS round trip (the same registers as reading both rows up front: a K row is dead once
+        // both scores exist).  The running maximum is only a reference point of the exponentials, so it is moved lazily
+        // (see RESCALE_THR).
+        float4 x[4], z[4];
+        read_row(x, kq);
 #pragma unroll
         for (int u = 0; u < VC; u++) {
             if (u < L) {
                 const bool inA = (unsigned)(pos + u - run.dA) < (unsigned)run.lenA, inB = (unsigned)(pos + u - run.dB) < (unsigned)run.lenB;
-                float4 x[4], z[4];
-                read_row(x, kq + u * MLK);
                 read_row(z, vq + u * MLK);
+                float scA = 0.f, scB = 0.f;
+                if (inA) scA = xor32_sum(dot16(qA, x));
+                if (inB) scB = xor32_sum(dot16(qB, x));
+                __builtin_amdgcn_sched_barrier(0);
+                read_row(x, kq + (u + 1) * MLK); // (past the last position: a row nobody uses, still inside the buffer)
+                __builtin_amdgcn_sched_barrier(0);
                 if (inA) {
-                    const float sc = xor32_sum(dot16(qA, x));
+                    const float sc = scA;
                     if (__any(sc > mA + RESCALE_THR)) {
                         const float mn = sc > mA + RESCALE_THR ? sc : mA, corr = fast_exp2(mA - mn);
                         SA *= corr;
@@ -156,7 +165,7 @@ __device__ inline void fwd_pair(const Args &a, float *Ks, float *Vs, int *Rs, in
                     axpy16(accA, p, z);
                 }
                 if (inB) {
-                    const float sc = xor32_sum(dot16(qB, x));
+                    const float sc = scB;
                     if (__any(sc > mB + RESCALE_THR)) {
                         const float mn = sc > mB + RESCALE_THR ? sc : mB, corr = fast_exp2(mB - mn);
                         SB *= corr;

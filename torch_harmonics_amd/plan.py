@@ -11,9 +11,13 @@ addresses cannot be recycled for a different psi while the entry exists, and an 
 edit of either tensor changes its version counter and misses the cache.
 """
 
+import hashlib
+import os
+import tempfile
 import threading
 from collections import OrderedDict
 
+import numpy as np
 import torch
 
 from . import _lib
@@ -87,6 +91,48 @@ def build_host_blob(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, 
     blob = torch.zeros(n, dtype=torch.int32)
     _lib.check(lib.s2attn_plan_build(*args, blob.data_ptr(), n), "s2attn_plan_build")
     return Plan(blob, blob[: _lib.PLAN_HEADER_INTS].tolist())
+
+
+def _disk_cache_dir():
+    """Directory of the on-disk plan cache: $S2ATTN_CACHE_DIR, else ~/.cache/torch_harmonics_amd; None when the variable is set to
+    an empty string or "off" (no caching)."""
+    d = os.environ.get("S2ATTN_CACHE_DIR")
+    if d is None:
+        d = os.path.join(os.path.expanduser("~"), ".cache", "torch_harmonics_amd")
+    return None if d in ("", "off") else d
+
+
+def cached_host_blob(key, col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int) -> Plan:
+    """build_host_blob with the blob kept on disk between processes.  `key` names the psi (a module passes its grids, shapes
+    and cutoff); the file name also carries the library's ABI version, the plan format and the psi's size, and a file whose
+    header does not describe this problem is ignored and rewritten.  Any I/O failure falls back to building in memory."""
+    d = _disk_cache_dir()
+    if d is None:
+        return build_host_blob(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    ident = repr((key, _lib.ABI_VERSION, _lib.PLAN_MAGIC, int(col_idx.numel()), int(row_off.numel()), nlat_in, nlon_in, nlat_out, nlon_out))
+    path = os.path.join(d, "plan_" + hashlib.sha1(ident.encode()).hexdigest() + ".npy")
+    PH = _lib.PH
+    try:
+        blob = torch.from_numpy(np.load(path, allow_pickle=False))
+        h = blob[: _lib.PLAN_HEADER_INTS].tolist()
+        ok = (
+            blob.dtype == torch.int32 and blob.dim() == 1 and len(h) == _lib.PLAN_HEADER_INTS and h[PH["MAGIC"]] == _lib.PLAN_MAGIC and h[PH["TOTAL"]] == blob.numel()
+            and (h[PH["NLAT_IN"]], h[PH["NLON_IN"]], h[PH["NLAT_OUT"]], h[PH["NLON_OUT"]]) == (nlat_in, nlon_in, nlat_out, nlon_out)
+        )  # fmt: skip
+        if ok:
+            return Plan(blob.contiguous(), h)
+    except (OSError, ValueError):
+        pass
+    plan = build_host_blob(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    try:
+        os.makedirs(d, exist_ok=True)
+        fd, tmp = tempfile.mkstemp(dir=d, suffix=".tmp")
+        with os.fdopen(fd, "wb") as f:
+            np.save(f, plan.blob.numpy(), allow_pickle=False)
+        os.replace(tmp, path)  # atomic: a concurrent reader sees the old file or the whole new one
+    except OSError:
+        pass
+    return plan
 
 
 def build_host_plan(col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in: int, nlon_in: int, nlat_out: int, nlon_out: int, with_mixed: bool = False):
