@@ -198,6 +198,20 @@ __device__ inline uint4 h16_load_piece(const char *p, bool ok)
     return r;
 }
 
+// A 16-byte piece (eight 16-bit values) times log2 e, rounded back to the storage type: the q (or k) operand of the score product
+// then yields scores in the log2 domain straight from the matrix cores.  The rounding is one more of the size the storage type
+// already made (2^-9 relative for bf16), independent per channel.
+template <typename M> __device__ inline uint4 h16_scale_log2e(uint4 x)
+{
+    unsigned u[4] = {x.x, x.y, x.z, x.w};
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        const float2 f = M::unpack2(u[i]);
+        u[i] = M::pack2(f.x * LOG2E, f.y * LOG2E);
+    }
+    return make_uint4(u[0], u[1], u[2], u[3]);
+}
+
 __device__ inline float h16_quarter_max(float x)
 {
     return xor32_max(xor16_max(x));
@@ -473,7 +487,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             const bool ok = 32 * s + 8 * qd < dr;
-            qop[s] = h16_load_piece(static_cast<const char *>(a.q) + off + 64 * s, ok);
+            qop[s] = h16_scale_log2e<M>(h16_load_piece(static_cast<const char *>(a.q) + off + 64 * s, ok));
             gop[s] = h16_load_piece(static_cast<const char *>(a.dy) + off + 64 * s, ok);
             const uint4 yv = h16_load_piece(static_cast<const char *>(a.ysaved) + off + 64 * s, ok);
             const unsigned gu[4] = {gop[s].x, gop[s].y, gop[s].z, gop[s].w}, yu[4] = {yv.x, yv.y, yv.z, yv.w};
@@ -530,11 +544,12 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
             const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
             const char *kblk[2] = {band_block<PITCH>(Ks, xw), band_block<PITCH>(Ks, xw + 16)};
             const char *vblk[2] = {band_block<PITCH>(Vs, xw), band_block<PITCH>(Vs, xw + 16)};
+            // The accumulators start at log2 w - lse and at -I, so the matrix cores hand back the exponent of p and g - I.
             f4v sc[2], gc[2];
 #pragma unroll
             for (int kb = 0; kb < 2; kb++) {
-                sc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
-                gc[kb] = f4v{0.f, 0.f, 0.f, 0.f};
+                sc[kb] = f4v{lwl, lwl, lwl, lwl};
+                gc[kb] = f4v{-I, -I, -I, -I};
 #pragma unroll
                 for (int s = 0; s < NS; s++) {
                     sc[kb] = M::mfma(h16_read_row<PITCH>(kblk[kb], s, c, qd), qop[s], sc[kb]);
@@ -546,7 +561,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 #pragma unroll
                 for (int kb = 0; kb < 2; kb++) {
 #pragma unroll
-                    for (int v = 0; v < 4; v++) gc[kb][v] = fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) * (gc[kb][v] - I);
+                    for (int v = 0; v < 4; v++) gc[kb][v] = fast_exp2(sc[kb][v]) * gc[kb][v];
                 }
             } else {
 #pragma unroll
@@ -554,8 +569,8 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 #pragma unroll
                     for (int v = 0; v < 4; v++) {
                         const unsigned t = (unsigned)(tb + 16 * kb + v);
-                        const float p = (t < (unsigned)len) ? fast_exp2(fmaf(sc[kb][v], LOG2E, lwl)) : 0.f;
-                        gc[kb][v] = p * (gc[kb][v] - I);
+                        const float p = (t < (unsigned)len) ? fast_exp2(sc[kb][v]) : 0.f;
+                        gc[kb][v] = p * gc[kb][v];
                     }
                 }
             }
@@ -616,7 +631,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             const bool ok = 32 * s + 8 * qd < dr;
-            kop[s] = h16_load_piece(static_cast<const char *>(a.k) + off + 64 * s, ok);
+            kop[s] = h16_scale_log2e<M>(h16_load_piece(static_cast<const char *>(a.k) + off + 64 * s, ok));
             vop[s] = h16_load_piece(static_cast<const char *>(a.v) + off + 64 * s, ok);
         }
     }
@@ -661,7 +676,7 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
             bd.template commit<FRESH>(Qs, Gs, tid, 0);
         else
             bd.template commit<HK>(Qs, Gs, tid, x0);
-        if (tid < (x0 == 0 ? FRESH : HK)) *reinterpret_cast<float2 *>(Qs + ((x0 + tid) & (BR - 4)) * PITCH + STAT + 8 * (tid & 3)) = st;
+        if (tid < (x0 == 0 ? FRESH : HK)) *reinterpret_cast<float2 *>(Qs + ((x0 + tid) & (BR - 4)) * PITCH + STAT + 8 * (tid & 3)) = make_float2(lw - st.x, -st.y);
     };
     if (wk.ri < wk.rend) {
         wk.run = a.sruns[wk.ri];
@@ -680,11 +695,15 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
             const int xw = HQ * wave + pos; // band row of this wavefront's position `pos`
             const char *qblk[2] = {band_block<PITCH>(Qs, xw), band_block<PITCH>(Qs, xw + 16)};
             const char *gblk[2] = {band_block<PITCH>(Gs, xw), band_block<PITCH>(Gs, xw + 16)};
+            // The accumulators start at the staged statistics (log2 w - lse of the query, -I of the query: written in that form at
+            // commit), so the matrix cores hand back the exponent of p and g - I.
             f4v sc[2], gc[2];
 #pragma unroll
             for (int qb = 0; qb < 2; qb++) {
-                sc[qb] = f4v{0.f, 0.f, 0.f, 0.f};
-                gc[qb] = f4v{0.f, 0.f, 0.f, 0.f};
+                const float4 *sp = reinterpret_cast<const float4 *>(qblk[qb] + 4 * qd * PITCH + STAT);
+                const float4 s01 = sp[0], s23 = sp[1];
+                sc[qb] = f4v{s01.x, s01.z, s23.x, s23.z};
+                gc[qb] = f4v{s01.y, s01.w, s23.y, s23.w};
 #pragma unroll
                 for (int s = 0; s < NS; s++) {
                     sc[qb] = M::mfma(h16_read_row<PITCH>(qblk[qb], s, c, qd), kop[s], sc[qb]);
@@ -695,16 +714,12 @@ template <typename T, int D, bool PAD> __global__ __launch_bounds__(64 * NW) voi
             const bool inner = pos >= HQ - 1 && pos + HK <= len; // every element of the step is a (query, key) pair of the run
 #pragma unroll
             for (int qb = 0; qb < 2; qb++) {
-                const float4 *sp = reinterpret_cast<const float4 *>(qblk[qb] + 4 * qd * PITCH + STAT);
-                const float4 s01 = sp[0], s23 = sp[1];
-                const float lv[4] = {s01.x, s01.z, s23.x, s23.z};
-                const float iv[4] = {s01.y, s01.w, s23.y, s23.w};
 #pragma unroll
                 for (int v = 0; v < 4; v++) {
-                    float p = fast_exp2(fmaf(sc[qb][v], LOG2E, lw - lv[v]));
+                    float p = fast_exp2(sc[qb][v]);
                     if (!inner) p = ((unsigned)(tb + 16 * qb + v) < (unsigned)len) ? p : 0.f; // band mask, first and last steps of a run only
                     sc[qb][v] = p;
-                    gc[qb][v] = p * (gc[qb][v] - iv[v]);
+                    gc[qb][v] = p * gc[qb][v];
                 }
             }
             const uint4 pop = make_uint4(M::pack2(sc[0][0], sc[0][1]), M::pack2(sc[0][2], sc[0][3]), M::pack2(sc[1][0], sc[1][1]), M::pack2(sc[1][2], sc[1][3]));
