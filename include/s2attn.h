@@ -18,6 +18,15 @@
  * proper multiple of nlon_in (up-sampling, "scatter" direction); the two
  * directions are told apart by the longitude counts, as in the reference
  * (attention.py:337).
+ *
+ * Accuracy, fp32 storage, against a float64 evaluation of the reference's torch loop (attention_torch.py:97-104): y, dk, dv,
+ * dq within rtol = atol = 1e-5 for heads of up to 128 channels and a query that carries the softmax scale.  Measured
+ * exceptions: dq on smooth fields (neighboring v almost equal, so the backward's g_j - <dy, y> cancels) lies within
+ * atol 2e-5 + rtol 1e-5 (1.6e-5 on values of magnitude 1 at 721 x 1440; the reference's CPU operators are 1.4e-4 from float64
+ * on the same tensors); heads wider than 128 channels and unscaled N(0,1) queries are as exact as a plain fp32 CPU evaluation
+ * of the same inputs (4.2e-5 absolute on values of magnitude 3 at 512 channels), with dv of the head-dim-32 kernels up to
+ * 1.2e-6 beyond 1e-5 on such a query.  16-bit storage: within 2e-2 of each tensor's RMS (arithmetic in fp32, operands of the
+ * matrix instructions in the storage type).
  */
 #ifndef S2ATTN_H
 #define S2ATTN_H
