@@ -169,7 +169,7 @@ def time_other_config(name, device, steps=3, cpu=False):
 def time_ring_steps(device, nchunk=4, reps=2):
     """The ring-step operators on one device (all longitude chunks of K/V folded one after the other, ms for the whole fold):
     gather direction on cfg3's tensors (B = 1, 8 heads of 32 channels folded into the batch, its grid and cutoff), up-sampling
-    361x720 -> 721x1440 with the same batch; fp32."""
+    361x720 -> 721x1440 with the same batch; fp32, and the gather direction once more with k, v, q, dy stored in bf16."""
     from torch_harmonics_amd import ops
     from torch_harmonics_amd.neighborhood import precompute_neighborhood_s2
     from torch_harmonics_amd.quadrature import precompute_latitudes
@@ -177,7 +177,12 @@ def time_ring_steps(device, nchunk=4, reps=2):
     BB, d = CONFIGS["cfg3"]["B"] * CONFIGS["cfg3"]["nh"], CONFIGS["cfg3"]["C"] // CONFIGS["cfg3"]["nh"]
     gen = torch.Generator(device=device).manual_seed(333)
     res = {}
-    for name, ins, outs, theta in (("gather", (721, 1440), (721, 1440), CONFIGS["cfg3"]["theta_cutoff"]), ("upsample", (361, 720), (721, 1440), 0.03)):
+    cases = (
+        ("gather", (721, 1440), (721, 1440), CONFIGS["cfg3"]["theta_cutoff"], torch.float32),
+        ("upsample", (361, 720), (721, 1440), 0.03, torch.float32),
+        ("gather_bf16", (721, 1440), (721, 1440), CONFIGS["cfg3"]["theta_cutoff"], torch.bfloat16),
+    )
+    for name, ins, outs, theta, dtype in cases:
         up = name == "upsample"
         (Hi, Wi), (Ho, Wo) = ins, outs
         col, roff, _ = precompute_neighborhood_s2(outs if up else ins, ins if up else outs, "equiangular", "equiangular", theta)
@@ -186,10 +191,10 @@ def time_ring_steps(device, nchunk=4, reps=2):
         split = ops.split_csr_rows(row_idx, roff, Ho)
         pairs = BB * (Wi if up else Wo) * col.numel()
         col, roff, row_idx = col.to(device), roff.to(device), row_idx.to(device)
-        k = torch.randn(BB, Hi, Wi, d, device=device, generator=gen)
-        v = torch.randn(BB, Hi, Wi, d, device=device, generator=gen)
-        q = torch.randn(BB, Ho, Wo, d, device=device, generator=gen) / math.sqrt(d)
-        dy = torch.randn(BB, Ho, Wo, d, device=device, generator=gen)
+        k = torch.randn(BB, Hi, Wi, d, device=device, generator=gen).to(dtype)
+        v = torch.randn(BB, Hi, Wi, d, device=device, generator=gen).to(dtype)
+        q = (torch.randn(BB, Ho, Wo, d, device=device, generator=gen) / math.sqrt(d)).to(dtype)
+        dy = torch.randn(BB, Ho, Wo, d, device=device, generator=gen).to(dtype)
         cw = Wi // nchunk
         parts = [(k[:, :, i * cw : (i + 1) * cw].contiguous(), v[:, :, i * cw : (i + 1) * cw].contiguous(), i * cw) for i in range(nchunk)]
         z = lambda *s: torch.zeros(*s, device=device)  # noqa: E731
@@ -213,7 +218,7 @@ def time_ring_steps(device, nchunk=4, reps=2):
                 else:
                     ops.backward_ring_step_pass1(kc, vc, q, dy, as2, qm2, integ, ak, akvw, w, col, roff, row_idx, *tail(lo))
 
-        grads = [(torch.zeros_like(kc), torch.zeros_like(vc)) for kc, vc, _ in parts]
+        grads = [(torch.zeros_like(kc, dtype=torch.float32), torch.zeros_like(vc, dtype=torch.float32)) for kc, vc, _ in parts]
 
         def pass2():
             for (kc, vc, lo), (dkc, dvc) in zip(parts, grads):
@@ -238,9 +243,9 @@ def time_ring_steps(device, nchunk=4, reps=2):
         geo = (w, col, roff, 1, Wi, Ho, Wo)
         y, lse = ops.forward_lse(k, v, q, *geo)
         t_one = run(lambda: ops.forward_lse(k, v, q, *geo))
-        err = ((y_acc / asum[..., None]) - y).abs().max().item()
+        err = ((y_acc / asum[..., None]) - y.float()).abs().max().item()
         res[name] = {
-            "grid": f"{Hi}x{Wi} -> {Ho}x{Wo}", "theta_cutoff": theta, "pairs": pairs, "chunks": nchunk, "forward_ms": t_f, "pass1_ms": t_1, "pass2_ms": t_2,
+            "grid": f"{Hi}x{Wi} -> {Ho}x{Wo}", "storage": str(dtype).replace("torch.", ""), "theta_cutoff": theta, "pairs": pairs, "chunks": nchunk, "forward_ms": t_f, "pass1_ms": t_1, "pass2_ms": t_2,
             "single_device_forward_ms": t_one, "max_abs_diff_to_single_device_y": err,
         }  # fmt: skip
         del k, v, q, dy, parts, grads, y_acc, ak, akvw, y

@@ -320,8 +320,10 @@ int s2attn_ring_backward_pass2(const void *k, const void *v, const void *q, cons
  * built once per psi by s2attn_plan_build(col_idx, row_off, nnz, nlat_in = global input latitudes, nlon_in, nlat_out =
  * local output latitudes, nlon_out = nlon_in / pscale) on host copies of the same col_idx / row_off.  A row of a staged
  * band is one input longitude, so the chunk clips rows of the band and the kernels walk only the steps of each run that
- * hold a longitude of the chunk.  Shapes: fp32 storage, ck == cv a multiple of 4 from 16 to 128, nlon_in / pscale >= 32,
- * 16-byte aligned tensors; anything else returns S2ATTN_E_UNSUPPORTED and the caller uses the entry points above.
+ * hold a longitude of the chunk.  Shapes: ck == cv a multiple of 4 from 16 to 128, nlon_in / pscale >= 32, k, v, q, dy
+ * of any storage dtype aligned to four channels (16 bytes fp32, 8 bytes bf16 / fp16: 16-bit rows are widened as they are
+ * staged, so tiles, matrix instructions and state are fp32 whatever the storage), state and dk, dv fp32 and 16-byte
+ * aligned; anything else returns S2ATTN_E_UNSUPPORTED and the caller uses the entry points above.
  * Pass 1 re-accumulates alpha_sum and qdotk_max with the forward step's operations in the forward step's order: fed the
  * same chunks in the same order the two alpha_sum are bit-identical, which the dq formula above (the forward's alpha_sum
  * with pass 1's other sums, as the reference combines them) relies on for wide heads - use the two together.
@@ -409,8 +411,8 @@ int s2attn_ring_backward_pass2_upsample(const void *k, const void *v, const void
  * The three up-sampling steps on the band-staged matrix-core kernels (same operators, same tensors and state): they take the
  * run-length plan of the local psi, built once per psi by s2attn_plan_build(col_idx, row_off, nnz, nlat_in = nlat_halo (the
  * chunk's rows, pole padding included), nlon_in, nlat_out = local output latitudes, nlon_out = nlon_out_global) on host
- * copies of the same col_idx / row_off.  Shapes as for the gather direction: fp32 storage, ck == cv a multiple of 4 from 16
- * to 128, nlon_in >= 32, 16-byte aligned tensors; anything else returns S2ATTN_E_UNSUPPORTED.  (Pass 1 of this direction
+ * copies of the same col_idx / row_off.  Shapes as for the gather direction: any storage dtype, ck == cv a multiple of 4 from 16
+ * to 128, nlon_in >= 32, tensors aligned to four channels; anything else returns S2ATTN_E_UNSUPPORTED.  (Pass 1 of this direction
  * works from the forward's final maximum, so its sums and the forward's alpha_sum are rounded differently whatever the
  * kernels; the dq formula amplifies that by |alpha_kvw| / alpha_sum, which grows with the head width: 3.5e-5 on values of
  * magnitude 1 at 128 channels.  The Python operators therefore take these entry points up to 64 channels.)

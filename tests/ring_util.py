@@ -83,7 +83,7 @@ RING_UP_CASES = [
 ]
 
 
-# up-sampling direction on grids with at least 32 input longitudes: with fp32 storage and ck == cv a multiple of 4 from 16 to 128
+# up-sampling direction on grids with at least 32 input longitudes: with ck == cv a multiple of 4 from 16 to 128
 # the three steps run on the band-staged matrix-core kernels
 RING_UP_BAND_CASES = [
     ((6, 40), (11, 80), "equiangular", "equiangular", 0.6, (2, 6, 9, 50), [0, 13, 14, 40], 0),  # ratio 2, a one-column chunk, odd window

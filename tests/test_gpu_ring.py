@@ -53,6 +53,21 @@ def test_ring_forward_step_and_pass1_on_the_band_staged_kernels(case, d, monkeyp
     assert taken and all(taken)
 
 
+@pytest.mark.parametrize("d", [16, 40, 64, 128], ids=lambda d: f"d{d}")
+@pytest.mark.parametrize("case", [RING_BAND_CASES[0], RING_BAND_CASES[2], RING_BAND_CASES[-1]], ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_band_staged_ring_steps_take_16_bit_storage(case, dtype, d, monkeypatch):
+    """k, v, q, dy in bf16 / fp16 on the band-staged kernels (rows widened at staging, fp32 state): state against the oracle fed the
+    same stored values at 1e-5 after every chunk, final results against the dense attention at the storage type's tolerance."""
+    from torch_harmonics_amd import ops
+
+    taken = []
+    real = ops._ring_takes_plan
+    monkeypatch.setattr(ops, "_ring_takes_plan", lambda *a: taken.append(real(*a)) or taken[-1])
+    _gather_direction(case, dtype, d, d, monkeypatch)
+    assert taken and all(taken)
+
+
 def _gather_direction(case, dtype, ck, cv, monkeypatch):
     from torch_harmonics_amd import ops
 
@@ -196,6 +211,20 @@ def test_upsample_ring_steps_on_the_band_staged_kernels(case, d, monkeypatch):
     real = ops._ring_takes_plan
     monkeypatch.setattr(ops, "_ring_takes_plan", lambda *a: taken.append(real(*a)) or taken[-1])
     _upsample_direction(case, torch.float32, d, d)
+    assert taken and all(taken)
+
+
+@pytest.mark.parametrize("d", [16, 40, 64], ids=lambda d: f"d{d}")
+@pytest.mark.parametrize("case", [RING_UP_BAND_CASES[0], RING_UP_BAND_CASES[-1]], ids=lambda c: f"{c[0][0]}x{c[0][1]}to{c[1][0]}x{c[1][1]}_win{c[5]}")
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+def test_band_staged_upsample_ring_steps_take_16_bit_storage(case, dtype, d, monkeypatch):
+    """The up-sampling direction's three steps on the band-staged kernels with 16-bit k, v, q, dy."""
+    from torch_harmonics_amd import ops
+
+    taken = []
+    real = ops._ring_takes_plan
+    monkeypatch.setattr(ops, "_ring_takes_plan", lambda *a: taken.append(real(*a)) or taken[-1])
+    _upsample_direction(case, dtype, d, d)
     assert taken and all(taken)
 
 

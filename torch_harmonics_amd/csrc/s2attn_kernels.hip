@@ -35,9 +35,10 @@
 
 #include "s2attn_internal.h"
 
-// This file is compiled three times (see the Makefile), so that the three groups of kernel instantiations build side by
+// This file is compiled four times (see the Makefile), so that the groups of kernel instantiations build side by
 // side: S2_PART 1 = everything but the launchers of the 16-longitude matrix-core families, 2 = the 16-bit family
-// (s2attn_h16.hpp), 3 = the fp32 family (s2attn_m32.hpp).  S2_PART 0 (the default) is the whole library in one unit.
+// (s2attn_h16.hpp), 3 = the fp32 family (s2attn_m32.hpp), 4 = its ring-step kernels for 16-bit storage.  S2_PART 0 (the
+// default) is the whole library in one unit.
 #ifndef S2_PART
 #define S2_PART 0
 #endif
@@ -2284,8 +2285,8 @@ enum Which { FWD, DQ, DKDV };
 
 template <typename T, int D, bool PAD> int launch_h16(Which which, const Args &a0, hipStream_t stream);
 template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t stream);
-template <int D, int MODE> int launch_ring_m32(const Args &a0, hipStream_t stream);
-template <int D, bool WRITE> int launch_ring_pass2_m32(const Args &a0, hipStream_t stream);
+template <int D, int MODE, typename T> int launch_ring_m32(const Args &a0, hipStream_t stream);
+template <int D, bool WRITE, typename T> int launch_ring_pass2_m32(const Args &a0, hipStream_t stream);
 
 #if S2_PART == 0 || S2_PART == 2
 // 16-bit matrix-core kernels: bf16 / fp16 storage, head dim D, equal longitude counts, 16-byte aligned tensors.  The
@@ -2368,52 +2369,52 @@ template <int D, int NS> int launch_m32(Which which, const Args &a0, hipStream_t
     return S2ATTN_OK;
 }
 #endif
-#if S2_PART == 0 || S2_PART == 3
-// one ring step (forward, or pass 1 of the backward) on the fp32 16-longitude kernels: one wavefront per 16 local output longitudes
-template <int D, int MODE> int launch_ring_m32(const Args &a0, hipStream_t stream)
+#if S2_PART == 0 || S2_PART == 3 || S2_PART == 4
+// one ring step (forward, or pass 1 of the backward) on the fp32 16-longitude kernels, tensors of storage type T: one wavefront per 16 local output longitudes
+template <int D, int MODE, typename T> int launch_ring_m32(const Args &a0, hipStream_t stream)
 {
     Args a = a0;
     a.row_first = 0;
     const long nblocks = (long)a.Ho * ((a.Wo + HQ - 1) / HQ) * a.B * a.nh;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    hipLaunchKernelGGL((ring_m32_kernel<D, MODE>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL((ring_m32_kernel<D, MODE, T>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
 // pass 2 of a ring step: one wavefront per 16 virtual columns of a column class of a chunk latitude
-template <int D, bool WRITE> int launch_ring_pass2_m32(const Args &a, hipStream_t stream)
+template <int D, bool WRITE, typename T> int launch_ring_pass2_m32(const Args &a, hipStream_t stream)
 {
     const int ntile = (a.r_nkx / a.kps + 1 + HQ - 1) / HQ + 1; // as in the kernel
     const long nblocks = (long)a.Hi * ntile * a.B;
     if (nblocks > 0x7fffffffL) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "problem needs %ld workgroups, more than one grid holds", nblocks);
-    hipLaunchKernelGGL((ring_pass2_m32_kernel<D, WRITE>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
+    hipLaunchKernelGGL((ring_pass2_m32_kernel<D, WRITE, T>), dim3((unsigned)nblocks), dim3(64), 0, stream, a);
     const hipError_t e = hipGetLastError();
     if (e != hipSuccess) return s2attn_fail(S2ATTN_E_LAUNCH, "kernel launch: %s", hipGetErrorString(e));
     return S2ATTN_OK;
 }
 #endif
 #if S2_PART == 3
-template int launch_ring_pass2_m32<16, false>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<16, true>(const Args &, hipStream_t);
-template int launch_ring_m32<16, 0>(const Args &, hipStream_t);
-template int launch_ring_m32<16, 1>(const Args &, hipStream_t);
-template int launch_ring_m32<16, 2>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<32, false>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<32, true>(const Args &, hipStream_t);
-template int launch_ring_m32<32, 0>(const Args &, hipStream_t);
-template int launch_ring_m32<32, 1>(const Args &, hipStream_t);
-template int launch_ring_m32<32, 2>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<64, false>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<64, true>(const Args &, hipStream_t);
-template int launch_ring_m32<64, 0>(const Args &, hipStream_t);
-template int launch_ring_m32<64, 1>(const Args &, hipStream_t);
-template int launch_ring_m32<64, 2>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<128, false>(const Args &, hipStream_t);
-template int launch_ring_pass2_m32<128, true>(const Args &, hipStream_t);
-template int launch_ring_m32<128, 0>(const Args &, hipStream_t);
-template int launch_ring_m32<128, 1>(const Args &, hipStream_t);
-template int launch_ring_m32<128, 2>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, false, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, true, float>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 0, float>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 1, float>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 2, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, false, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, true, float>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 0, float>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 1, float>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 2, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, false, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, true, float>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 0, float>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 1, float>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 2, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, false, float>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, true, float>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 0, float>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 1, float>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 2, float>(const Args &, hipStream_t);
 template int launch_m32<16, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<32, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<64, 1>(Which, const Args &, hipStream_t);
@@ -2421,6 +2422,48 @@ template int launch_m32<128, 1>(Which, const Args &, hipStream_t);
 template int launch_m32<128, 2>(Which, const Args &, hipStream_t);
 template int launch_m32<128, 3>(Which, const Args &, hipStream_t);
 template int launch_m32<128, 4>(Which, const Args &, hipStream_t);
+#endif
+#if S2_PART == 4
+template int launch_ring_pass2_m32<16, false, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, true, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 0, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 1, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 2, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, false, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, true, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 0, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 1, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 2, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, false, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, true, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 0, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 1, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 2, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, false, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, true, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 0, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 1, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 2, bf16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, false, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<16, true, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 0, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 1, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<16, 2, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, false, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<32, true, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 0, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 1, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<32, 2, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, false, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<64, true, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 0, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 1, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<64, 2, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, false, f16_t>(const Args &, hipStream_t);
+template int launch_ring_pass2_m32<128, true, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 0, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 1, f16_t>(const Args &, hipStream_t);
+template int launch_ring_m32<128, 2, f16_t>(const Args &, hipStream_t);
 #endif
 
 } // namespace s2
@@ -2770,11 +2813,13 @@ int ring_plan_args(Args &a, const void *k, const void *v, const void *q, const v
         return s2attn_fail(S2ATTN_E_INVALID, "plan was built for grids %dx%d -> %dx%d, the step needs %s x%d -> %dx%d (local latitudes, global longitudes)",
                            h[S2ATTN_PH_NLAT_IN], h[S2ATTN_PH_NLON_IN], h[S2ATTN_PH_NLAT_OUT], h[S2ATTN_PH_NLON_OUT], g.qps > 1 ? "the chunk's latitudes" : "all input latitudes",
                            g.nlon_in, g.nlat_out, wout);
-    if (g.dtype != S2ATTN_F32 || !m32_width(g.ck, g.cv) || g.ck > 128 || W < HK)
-        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take fp32 tensors with ck = cv a multiple of 4 from 16 to 128 on at least %d longitudes", HK);
+    if (g.dtype != S2ATTN_F32 && g.dtype != S2ATTN_BF16 && g.dtype != S2ATTN_F16) return s2attn_fail(S2ATTN_E_INVALID, "unknown dtype code %d", g.dtype);
+    if (!m32_width(g.ck, g.cv) || g.ck > 128 || W < HK)
+        return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take tensors with ck = cv a multiple of 4 from 16 to 128 on at least %d longitudes", HK);
     const void *ptrs[] = {k, v, q, dy};
+    const int need = g.dtype == S2ATTN_F32 ? 16 : 8; // four channels are loaded at a time
     for (const void *p : ptrs)
-        if (p && !aligned(p, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
+        if (p && !aligned(p, need)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take tensors aligned to four channels (%d bytes)", need);
     for (int i : {S2ATTN_PH_GATHER_OFF, S2ATTN_PH_GATHER_RUNS, S2ATTN_PH_GATHER_ORDER, S2ATTN_PH_GATHER_SPAN, S2ATTN_PH_SCATTER_OFF, S2ATTN_PH_SCATTER_RUNS, S2ATTN_PH_SCATTER_ORDER})
         if (h[i] < S2ATTN_PLAN_HEADER_INTS || h[i] > h[S2ATTN_PH_TOTAL]) return s2attn_fail(S2ATTN_E_INVALID, "plan header: offset %d of array %d lies outside the plan", h[i], i);
     const int32_t *d = plan->data;
@@ -2815,19 +2860,31 @@ int ring_geo(RingGeo &g, const s2attn_ring_up_shape *sh)
                 sh->nlon_out_global / sh->pscale_out, 1, sh->pscale_out};
     return S2ATTN_OK;
 }
-template <int MODE> int launch_ring_plan(const Args &a, hipStream_t st)
+template <int MODE, typename T> int launch_ring_plan_t(const Args &a, hipStream_t st)
 {
-    if (a.dk_ <= 16) return launch_ring_m32<16, MODE>(a, st);
-    if (a.dk_ <= 32) return launch_ring_m32<32, MODE>(a, st);
-    if (a.dk_ <= 64) return launch_ring_m32<64, MODE>(a, st);
-    return launch_ring_m32<128, MODE>(a, st);
+    if (a.dk_ <= 16) return launch_ring_m32<16, MODE, T>(a, st);
+    if (a.dk_ <= 32) return launch_ring_m32<32, MODE, T>(a, st);
+    if (a.dk_ <= 64) return launch_ring_m32<64, MODE, T>(a, st);
+    return launch_ring_m32<128, MODE, T>(a, st);
 }
-template <bool WRITE> int launch_ring_pass2_plan(const Args &a, hipStream_t st)
+template <int MODE> int launch_ring_plan(const Args &a, int dtype, hipStream_t st)
 {
-    if (a.dk_ <= 16) return launch_ring_pass2_m32<16, WRITE>(a, st);
-    if (a.dk_ <= 32) return launch_ring_pass2_m32<32, WRITE>(a, st);
-    if (a.dk_ <= 64) return launch_ring_pass2_m32<64, WRITE>(a, st);
-    return launch_ring_pass2_m32<128, WRITE>(a, st);
+    if (dtype == S2ATTN_BF16) return launch_ring_plan_t<MODE, bf16_t>(a, st);
+    if (dtype == S2ATTN_F16) return launch_ring_plan_t<MODE, f16_t>(a, st);
+    return launch_ring_plan_t<MODE, float>(a, st);
+}
+template <bool WRITE, typename T> int launch_ring_pass2_plan_t(const Args &a, hipStream_t st)
+{
+    if (a.dk_ <= 16) return launch_ring_pass2_m32<16, WRITE, T>(a, st);
+    if (a.dk_ <= 32) return launch_ring_pass2_m32<32, WRITE, T>(a, st);
+    if (a.dk_ <= 64) return launch_ring_pass2_m32<64, WRITE, T>(a, st);
+    return launch_ring_pass2_m32<128, WRITE, T>(a, st);
+}
+template <bool WRITE> int launch_ring_pass2_plan(const Args &a, int dtype, hipStream_t st)
+{
+    if (dtype == S2ATTN_BF16) return launch_ring_pass2_plan_t<WRITE, bf16_t>(a, st);
+    if (dtype == S2ATTN_F16) return launch_ring_pass2_plan_t<WRITE, f16_t>(a, st);
+    return launch_ring_pass2_plan_t<WRITE, float>(a, st);
 }
 template <typename SHAPE>
 int ring_forward_plan(const void *k, const void *v, const void *q, float *y_acc, float *alpha_sum, float *qdotk_max, const float *quad_weights,
@@ -2841,7 +2898,7 @@ int ring_forward_plan(const void *k, const void *v, const void *q, float *y_acc,
     if (!y_acc || !alpha_sum || !qdotk_max) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!aligned(y_acc, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_yacc = y_acc, a.r_asum = alpha_sum, a.r_qmax = qdotk_max;
-    return launch_ring_plan<0>(a, static_cast<hipStream_t>(stream));
+    return launch_ring_plan<0>(a, g.dtype, static_cast<hipStream_t>(stream));
 }
 template <typename SHAPE, bool WRITE>
 int ring_pass2_plan(const void *k, const void *v, const void *q, const void *dy, const float *alpha_sum, const float *qdotk_max, const float *integral_norm,
@@ -2856,7 +2913,7 @@ int ring_pass2_plan(const void *k, const void *v, const void *q, const void *dy,
     if (!aligned(dk, 16) || !aligned(dv, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_asum = const_cast<float *>(alpha_sum), a.r_qmax = const_cast<float *>(qdotk_max), a.r_integral = const_cast<float *>(integral_norm);
     a.dk = dk, a.dv = dv;
-    return launch_ring_pass2_plan<WRITE>(a, static_cast<hipStream_t>(stream));
+    return launch_ring_pass2_plan<WRITE>(a, g.dtype, static_cast<hipStream_t>(stream));
 }
 } // namespace
 
@@ -2898,7 +2955,7 @@ extern "C" int s2attn_ring_backward_pass1_plan(const void *k, const void *v, con
     if (!dy || !alpha_sum || !qdotk_max || !integral || !alpha_k || !alpha_kvw) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!aligned(alpha_k, 16) || !aligned(alpha_kvw, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_asum = alpha_sum, a.r_qmax = qdotk_max, a.r_integral = integral, a.r_ak = alpha_k, a.r_akvw = alpha_kvw;
-    return launch_ring_plan<1>(a, static_cast<hipStream_t>(stream));
+    return launch_ring_plan<1>(a, g.dtype, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int s2attn_ring_backward_pass1_upsample_plan(const void *k, const void *v, const void *q, const void *dy, const float *qdotk_max,
@@ -2913,7 +2970,7 @@ extern "C" int s2attn_ring_backward_pass1_upsample_plan(const void *k, const voi
     if (!dy || !qdotk_max || !integral || !alpha_k || !alpha_kvw) return s2attn_fail(S2ATTN_E_INVALID, "null tensor pointer");
     if (!aligned(alpha_k, 16) || !aligned(alpha_kvw, 16)) return s2attn_fail(S2ATTN_E_UNSUPPORTED, "the band-staged ring steps take 16-byte aligned tensors");
     a.r_qmax = const_cast<float *>(qdotk_max), a.r_integral = integral, a.r_ak = alpha_k, a.r_akvw = alpha_kvw;
-    return launch_ring_plan<2>(a, static_cast<hipStream_t>(stream));
+    return launch_ring_plan<2>(a, g.dtype, static_cast<hipStream_t>(stream));
 }
 
 namespace {

@@ -153,18 +153,25 @@ template <int D, int PITCH> __device__ inline void m32_accumulate(f4v (&acc)[D /
     }
 }
 
-// this lane's quarter (channels qd * D/4 ..) of one grid point's vector of dr channels; zeros from channel dr on
-template <int D> __device__ inline void m32_load_quarter(float (&op)[D / 4], const char *vec, int qd, int dr)
+// this lane's quarter (channels qd * D/4 ..) of one grid point's vector of dr channels of storage type T; zeros from channel dr on
+template <int D, typename T = float> __device__ inline void m32_load_quarter(float (&op)[D / 4], const char *vec, int qd, int dr)
 {
 #pragma unroll
     for (int i = 0; i < D / 16; i++) {
         float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (qd * (D / 4) + 4 * i < dr) x = *reinterpret_cast<const float4 *>(vec + qd * D + 16 * i);
+        if (qd * (D / 4) + 4 * i < dr) x = load4(reinterpret_cast<const T *>(vec) + qd * (D / 4) + 4 * i);
         op[4 * i + 0] = x.x;
         op[4 * i + 1] = x.y;
         op[4 * i + 2] = x.z;
         op[4 * i + 3] = x.w;
     }
+}
+
+// four consecutive channels of storage type T, widened: one 16-byte piece of an fp32 tile row
+template <typename T> __device__ inline u4v m32_piece(const char *p)
+{
+    const float4 x = load4(reinterpret_cast<const T *>(p));
+    return u4v{__float_as_uint(x.x), __float_as_uint(x.y), __float_as_uint(x.z), __float_as_uint(x.w)};
 }
 
 // ---- forward ---------------------------------------------------------------------------------------------------
@@ -565,6 +572,8 @@ template <int D, int NS> __global__ __launch_bounds__(64 * NS) void dkdv_m32_ker
 // the chunk are up to three intervals, and the walk visits only the 32-position steps inside them (a chunk of a quarter of
 // the circle costs a polar tile a quarter of its steps, an equatorial tile one step per run in the one or two chunks its
 // neighborhood touches).  Tiles without any such step leave the state untouched.
+// k, v, q, dy have storage type T (fp32, bf16 or fp16: 16-bit rows are widened when they are fetched, so the staged tiles,
+// the matrix instructions and the caller's state are fp32 whatever the storage); dk, dv of pass 2 are fp32.
 constexpr float NEG_BIG_NAT = -1.0e38f; // "no neighbor yet" for a maximum in natural units (times log2 e stays finite)
 
 struct RingWalk {
@@ -631,7 +640,7 @@ struct RingWalk {
 // Both directions: in the up-sampling direction (r_qps = nlon_out / nlon_in > 1) the plan's output latitudes are virtual
 // (real latitude * r_qps + column class), a tile's queries are the local output columns (w0 + c) * r_qps + class, input
 // latitudes are rows of the chunk as they stand and r_wlat0 turns them into quadrature-weight indices.
-template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 0) ? 4 : (D <= 32 ? 3 : (D <= 64 && MODE == 0 ? 2 : 1))) void ring_m32_kernel(const Args a)
+template <int D, int MODE, typename T> __global__ __launch_bounds__(64, (D <= 32 && MODE == 0) ? 4 : (D <= 32 ? 3 : (D <= 64 && MODE == 0 ? 2 : 1))) void ring_m32_kernel(const Args a)
 {
     constexpr int NS = 1;
     constexpr bool PASS1 = MODE != 0, FIXED = MODE == 2;
@@ -646,7 +655,7 @@ template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 
     const int hor = ho / a.r_qps, parq = ho - hor * a.r_qps;
     const int nval = min(HQ, (a.r_wo - parq + a.r_qps - 1) / a.r_qps - w0); // queries of the tile inside the local window
     if (nval <= 0) return;
-    const unsigned ldb = drt * 4; // bytes between two grid points
+    const unsigned ldb = drt * sizeof(T); // bytes between two grid points
     const char *kx = static_cast<const char *>(a.k) + (size_t)b * a.r_nlat * a.r_nkx * ldb;
     const char *vx = static_cast<const char *>(a.v) + (size_t)b * a.r_nlat * a.r_nkx * ldb;
     const bool mine = c < nval;
@@ -670,8 +679,8 @@ template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 
     if (!wk.advance()) return; // nothing of this tile's neighborhood is in the chunk
 
     float qop[D / 4], gop[PASS1 ? D / 4 : 1];
-    m32_load_quarter<D>(qop, static_cast<const char *>(a.q) + pt * ldb, qd, dr);
-    if constexpr (PASS1) m32_load_quarter<D>(gop, static_cast<const char *>(a.dy) + pt * ldb, qd, dr);
+    m32_load_quarter<D, T>(qop, static_cast<const char *>(a.q) + pt * ldb, qd, dr);
+    if constexpr (PASS1) m32_load_quarter<D, T>(gop, static_cast<const char *>(a.dy) + pt * ldb, qd, dr);
     // forward: Y^T; pass 1: alpha_k^T (acc) and alpha_kvw^T (acc2): register v of block cb is channel 16 cb + 4 qd + v of column c
     float *const acc_state = PASS1 ? a.r_ak : a.r_yacc;
     f4v acc[NCB], acc2[PASS1 ? NCB : 1];
@@ -696,8 +705,8 @@ template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 
 
     Tile kt, vt;
     const int r0 = lane / Tile::CPR;
-    const unsigned pc = 16u * (lane % Tile::CPR);
-    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
+    const unsigned pc = 4u * sizeof(T) * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's four channels of a staged row exist
     const unsigned colb = ldb * a.kps;                 // bytes between two virtual columns
     auto fetch = [&]() { // the rows of the step the walk stands at; rows beyond the interval are staged as zeros
         const size_t base = ((size_t)wk.rl * a.r_nkx + (size_t)((wk.vca + wk.pos - wk.ua) * a.kps + wk.par - a.r_lon_lo)) * ldb + pc;
@@ -708,8 +717,8 @@ template <int D, int MODE> __global__ __launch_bounds__(64, (D <= 32 && MODE == 
             kt.raw[it] = u4v{0u, 0u, 0u, 0u};
             vt.raw[it] = u4v{0u, 0u, 0u, 0u};
             if (row < nrows && piece_ok) {
-                kt.raw[it] = *reinterpret_cast<const u4v *>(kx + base + (size_t)row * colb);
-                vt.raw[it] = *reinterpret_cast<const u4v *>(vx + base + (size_t)row * colb);
+                kt.raw[it] = m32_piece<T>(kx + base + (size_t)row * colb);
+                vt.raw[it] = m32_piece<T>(vx + base + (size_t)row * colb);
             }
         }
     };
@@ -883,7 +892,7 @@ struct RingWalk2 {
 // WRITE = false (gather direction): dk, dv are added to.  WRITE = true (up-sampling direction: r_qps > 1, the plan's output
 // latitudes are virtual, a staged row of virtual column j is the local query column j * r_qps + class): every element of
 // the chunk's dk, dv is written, zeros where no query sees the key.
-template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(const Args a)
+template <int D, bool WRITE, typename T> __global__ __launch_bounds__(64) void ring_pass2_m32_kernel(const Args a)
 {
     typedef FTile<D> Tile;
     constexpr int PITCH = Tile::PITCH, NCB = D / 16;
@@ -922,15 +931,15 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
     char *lds = m32_lds<m32_lds_bytes<D, 1>(true), 1>();
     char *Qs = lds, *Gs = Qs + HK * PITCH;
     float *Ls = reinterpret_cast<float *>(Gs + HK * PITCH), *Is = Ls + HK;
-    const unsigned ldb = drt * 4; // bytes between two grid points
+    const unsigned ldb = drt * sizeof(T); // bytes between two grid points
     const int Hor = a.Ho / a.r_qps; // real local output latitudes
     const size_t sbase = (size_t)b * Hor * a.r_wo;
     const char *qy = static_cast<const char *>(a.q) + sbase * ldb;
     const char *gy = static_cast<const char *>(a.dy) + sbase * ldb;
 
     float kop[D / 4], vop[D / 4]; // this lane's quarter of key c
-    m32_load_quarter<D>(kop, static_cast<const char *>(a.k) + pt * ldb, qd, dr);
-    m32_load_quarter<D>(vop, static_cast<const char *>(a.v) + pt * ldb, qd, dr);
+    m32_load_quarter<D, T>(kop, static_cast<const char *>(a.k) + pt * ldb, qd, dr);
+    m32_load_quarter<D, T>(vop, static_cast<const char *>(a.v) + pt * ldb, qd, dr);
     f4v dkt[NCB], dvt[NCB];
 #pragma unroll
     for (int cb = 0; cb < NCB; cb++) {
@@ -942,8 +951,8 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
     Tile qt, gt;
     float2 st = make_float2(0.f, 0.f);
     const int r0 = lane / Tile::CPR;
-    const unsigned pc = 16u * (lane % Tile::CPR);
-    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's 16-byte piece of a staged row exists
+    const unsigned pc = 4u * sizeof(T) * (lane % Tile::CPR);
+    const bool piece_ok = 4 * (lane % Tile::CPR) < dr; // this lane's four channels of a staged row exist
     RingWalk2 wk;
     wk.W = a.Wi, wk.w0 = w0, wk.qps = a.r_qps, wk.wo = a.r_wo;
     wk.start(a.sruns, ri, rend);
@@ -962,8 +971,8 @@ template <int D, bool WRITE> __global__ __launch_bounds__(64) void ring_pass2_m3
                 int cr = wk.col + row; // wraps only when the window is the whole circle
                 cr -= (cr >= a.Wi) ? a.Wi : 0;
                 const size_t o = (lat + (size_t)cr * a.r_qps) * ldb + pc;
-                qt.raw[it] = *reinterpret_cast<const u4v *>(qy + o);
-                gt.raw[it] = *reinterpret_cast<const u4v *>(gy + o);
+                qt.raw[it] = m32_piece<T>(qy + o);
+                gt.raw[it] = m32_piece<T>(gy + o);
             }
         }
         if (lane < HK) { // lanes 0..31 fetch the statistics of the staged rows: (log2-sum-exp, integral_norm)

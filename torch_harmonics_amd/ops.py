@@ -319,9 +319,10 @@ def _ring_takes_plan(kx, vx, qy, nlon_in, pscale, max_ck=128) -> bool:
     alpha_sum are then bit-identical; the state buffers are fresh torch allocations, 16-byte aligned like every tensor).
     The up-sampling direction stops at 64 channels (max_ck): its pass 1 works from the forward's FINAL maximum, so its sums and
     the forward's alpha_sum are rounded differently whatever the kernels, and the dq formula that combines them amplifies that
-    by |alpha_kvw| / alpha_sum, which grows with the head width (3.5e-5 on values of magnitude 1 at 128 channels)."""
+    by |alpha_kvw| / alpha_sum, which grows with the head width (3.5e-5 on values of magnitude 1 at 128 channels).
+    Any storage dtype: 16-bit rows are widened as they are staged, tiles, matrix instructions and state are fp32."""
     ck, cv = kx.shape[3], vx.shape[3]
-    if qy.dtype != torch.float32 or ck != cv or ck % 4 or not 16 <= ck <= max_ck or nlon_in // pscale < 32:
+    if qy.dtype not in _DTYPE_CODE or ck != cv or ck % 4 or not 16 <= ck <= max_ck or nlon_in // pscale < 32:
         return False
     return True
 
