@@ -612,6 +612,46 @@ def test_reference_operator_names_and_schemas_are_registered():
         assert dk.shape == k.shape and dv.shape == v.shape and dq.shape == q.shape
 
 
+def test_ring_and_autograd_operators_carry_the_reference_names_and_argument_lists():
+    """attention_kernels::forward_ring_step ... backward_ring_step_upsample_pass2, split_csr_rows (attention_interface.cpp:136-189)
+    and the autograd-carrying _neighborhood_s2_attention_optimized (attention_optimized.py:230) exist under the reference's names
+    with its argument names, order and written-to arguments (Python fragments of the namespace; ints are SymInt there)."""
+    ring_tail = "Tensor quad_weights, Tensor col_idx, Tensor row_off, Tensor row_idx, int nlon_in, int pscale, int lon_lo_kx, int lat_halo_start, int nlat_out, int nlon_out, int n_long_rows, int max_row_len, int mid_row_len"
+    up_tail = "Tensor quad_weights, Tensor col_idx, Tensor row_off, int nlon_in, int nlon_out_global, int pscale_out, int lon_lo_kx, int lat_halo_start, int nlat_out, int nlon_out"
+    want = {
+        "split_csr_rows": ("Tensor row_idx, Tensor row_off, int nlat_out", "(int, int, int)"),
+        "forward_ring_step": ("Tensor kx, Tensor vx, Tensor qy, Tensor! y_acc, Tensor! alpha_sum_buf, Tensor! qdotk_max_buf, " + ring_tail, "()"),
+        "backward_ring_step_pass1": (
+            "Tensor kx, Tensor vx, Tensor qy, Tensor dy, Tensor! alpha_sum_buf, Tensor! qdotk_max_buf, Tensor! integral_buf, Tensor! alpha_k_buf, Tensor! alpha_kvw_buf, " + ring_tail,
+            "()",
+        ),
+        "backward_ring_step_pass2": (
+            "Tensor kx, Tensor vx, Tensor qy, Tensor dy, Tensor alpha_sum_buf, Tensor qdotk_max_buf, Tensor integral_norm_buf, Tensor! dkx, Tensor! dvx, " + ring_tail,
+            "()",
+        ),
+        "forward_ring_step_upsample": ("Tensor kx, Tensor vx, Tensor qy, Tensor! y_acc, Tensor! alpha_sum_buf, Tensor! qdotk_max_buf, " + up_tail, "()"),
+        "backward_ring_step_upsample_pass1": (
+            "Tensor kx, Tensor vx, Tensor qy, Tensor dy, Tensor qdotk_max_buf, Tensor! integral_buf, Tensor! alpha_k_buf, Tensor! alpha_kvw_buf, " + up_tail,
+            "()",
+        ),
+        "backward_ring_step_upsample_pass2": (
+            "Tensor kx, Tensor vx, Tensor qy, Tensor dy, Tensor alpha_sum_buf, Tensor qdotk_max_buf, Tensor integral_norm_buf, Tensor! dkx, Tensor! dvx, " + up_tail,
+            "()",
+        ),
+        "_neighborhood_s2_attention_optimized": (
+            "Tensor kw, Tensor vw, Tensor qw, Tensor quad_weights, Tensor col_idx, Tensor row_off, int nh, int nlon_in, int nlat_out, int nlon_out",
+            "Tensor",
+        ),
+    }
+    for name, (args, ret) in want.items():
+        schema = getattr(torch.ops.attention_kernels, name).default._schema
+        got = ", ".join(("Tensor!" if a.alias_info is not None and a.alias_info.is_write else str(a.type).replace("SymInt", "int")) + " " + a.name for a in schema.arguments)
+        assert got == args, f"{name}: {got}"
+        rets = [str(r.type).replace("SymInt", "int") for r in schema.returns]
+        assert (("(" + ", ".join(rets) + ")") if len(rets) != 1 else rets[0]) == ret, name
+    assert torch.ops.attention_kernels.split_csr_rows(torch.tensor([1, 0, 2], dtype=torch.int32), torch.tensor([0, 3, 3000, 3001]), 3) == (1, 2997, 3)
+
+
 def test_point_strides_are_validated_on_the_host():
     """A tensor may be a column block of a wider buffer (point stride > packed row); strides must cover the packed row and be
     multiples of 4 elements."""

@@ -6,8 +6,12 @@ Operator set and signatures follow the reference:
   attention_kernels::permute_to_nhwc / _nchw    85-119), registered for the CUDA dispatch key by the C++ binding
                                                 csrc/s2attn_torch.cpp; fake and autograd rules here, as in
                                                 attention_optimized.py:230-322 and attention/_layout.py:76-103
-  s2attn::_neighborhood_s2_attention_optimized  the autograd-carrying op
-                                                (attention_optimized.py:230-322)
+  attention_kernels::_neighborhood_s2_attention_optimized
+                                                the autograd-carrying op, a Python fragment of the namespace the C++
+                                                binding defines, as in the reference (attention_optimized.py:230-322)
+  attention_kernels::forward_ring_step ...      the six ring-step operators and split_csr_rows under the reference's names
+                                                and argument lists (attention_interface.cpp:136-189)
+  s2attn::_neighborhood_s2_attention_saved      the same attention with y and the normaliser handed to the backward
 Argument order is (k, v, q, ...), outputs of backward are (dk, dv, dq), as there.
 
 Both directions are served: nlon_in a multiple of nlon_out (self-attention, down-sampling; psi keyed by output latitude) and
@@ -141,7 +145,7 @@ torch.library.register_autograd("attention_kernels::permute_to_nchw", lambda ctx
 # ---- the autograd-carrying attention op ---------------------------------------------------
 
 
-@torch.library.custom_op("s2attn::_neighborhood_s2_attention_optimized", mutates_args=())
+@torch.library.custom_op("attention_kernels::_neighborhood_s2_attention_optimized", mutates_args=())
 def _neighborhood_s2_attention_optimized(
     kw: torch.Tensor,
     vw: torch.Tensor,
@@ -260,7 +264,7 @@ def neighborhood_s2_attention(kw, vw, qw, quad_weights, col_idx, row_off, nh, nl
 # Autocast: k, v, q are brought to the active autocast dtype and the op re-entered with autocast off;
 # quad_weights and the index tensors pass through (attention_optimized.py:310-322).
 def _make_autocast_impl(device_type: str):
-    @torch.library.impl("s2attn::_neighborhood_s2_attention_optimized", f"Autocast{device_type.upper()}")
+    @torch.library.impl("attention_kernels::_neighborhood_s2_attention_optimized", f"Autocast{device_type.upper()}")
     def _(kw, vw, qw, quad_weights, col_idx, row_off, nh, nlon_in, nlat_out, nlon_out):
         cast_dtype = torch.get_autocast_dtype(device_type)
         with torch.amp.autocast(device_type, enabled=False):
@@ -306,6 +310,13 @@ def split_csr_rows(row_idx: torch.Tensor, row_off: torch.Tensor, nlat_out: int):
     short = (lens < min_long).nonzero()
     n_long = int(short[0]) if short.numel() else int(nlat_out)
     return n_long, (max_rlen if n_long else 0), (int(lens[n_long]) if n_long < nlat_out else 0)
+
+
+# the reference's operator of the same name and schema (attention_interface.cpp:136): a set-up-time host computation, not
+# pt2-compliant and without a fake kernel there either
+_ring_fragment = torch.library.Library("attention_kernels", "FRAGMENT")
+_ring_fragment.define("split_csr_rows(Tensor row_idx, Tensor row_off, int nlat_out) -> (int, int, int)")
+_ring_fragment.impl("split_csr_rows", split_csr_rows, "CompositeExplicitAutograd")
 
 
 def _ring_shape(kx, vx, qy, nlon_in, pscale, lon_lo_kx, lat_halo_start, nlat_out, nlon_out) -> _lib.RingShapeStruct:
@@ -358,7 +369,7 @@ def _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, row_id
         raise RuntimeError(f"row_off must have {nrows + 1} entries" + ("" if row_idx is None else f" and row_idx {nrows}"))
 
 
-@torch.library.custom_op("s2attn::forward_ring_step", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
+@torch.library.custom_op("attention_kernels::forward_ring_step", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
 def forward_ring_step(
     kx: torch.Tensor,
     vx: torch.Tensor,
@@ -409,7 +420,7 @@ def _(kx, vx, qy, y_acc, alpha_sum_buf, qdotk_max_buf, quad_weights, col_idx, ro
 
 
 @torch.library.custom_op(
-    "s2attn::backward_ring_step_pass1", mutates_args=("alpha_sum_buf", "qdotk_max_buf", "integral_buf", "alpha_k_buf", "alpha_kvw_buf")
+    "attention_kernels::backward_ring_step_pass1", mutates_args=("alpha_sum_buf", "qdotk_max_buf", "integral_buf", "alpha_k_buf", "alpha_kvw_buf")
 )
 def backward_ring_step_pass1(
     kx: torch.Tensor,
@@ -471,7 +482,7 @@ def _(kx, vx, qy, dy, alpha_sum_buf, qdotk_max_buf, integral_buf, alpha_k_buf, a
 _RING_PASS2_FROM_CSR = False
 
 
-@torch.library.custom_op("s2attn::backward_ring_step_pass2", mutates_args=("dkx", "dvx"))
+@torch.library.custom_op("attention_kernels::backward_ring_step_pass2", mutates_args=("dkx", "dvx"))
 def backward_ring_step_pass2(
     kx: torch.Tensor,
     vx: torch.Tensor,
@@ -537,7 +548,7 @@ def _ring_up_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, nla
     _ring_validate(kx, vx, qy, dy, state, quad_weights, col_idx, row_off, None, nlat_out, nlon_out, nrows=kx.shape[1])
 
 
-@torch.library.custom_op("s2attn::forward_ring_step_upsample", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
+@torch.library.custom_op("attention_kernels::forward_ring_step_upsample", mutates_args=("y_acc", "alpha_sum_buf", "qdotk_max_buf"))
 def forward_ring_step_upsample(
     kx: torch.Tensor,
     vx: torch.Tensor,
@@ -585,7 +596,7 @@ def _(kx, vx, qy, y_acc, alpha_sum_buf, qdotk_max_buf, quad_weights, col_idx, ro
     return None
 
 
-@torch.library.custom_op("s2attn::backward_ring_step_upsample_pass1", mutates_args=("integral_buf", "alpha_k_buf", "alpha_kvw_buf"))
+@torch.library.custom_op("attention_kernels::backward_ring_step_upsample_pass1", mutates_args=("integral_buf", "alpha_k_buf", "alpha_kvw_buf"))
 def backward_ring_step_upsample_pass1(
     kx: torch.Tensor,
     vx: torch.Tensor,
@@ -635,7 +646,7 @@ def _(kx, vx, qy, dy, qdotk_max_buf, integral_buf, alpha_k_buf, alpha_kvw_buf, q
     return None
 
 
-@torch.library.custom_op("s2attn::backward_ring_step_upsample_pass2", mutates_args=("dkx", "dvx"))
+@torch.library.custom_op("attention_kernels::backward_ring_step_upsample_pass2", mutates_args=("dkx", "dvx"))
 def backward_ring_step_upsample_pass2(
     kx: torch.Tensor,
     vx: torch.Tensor,
