@@ -124,14 +124,22 @@ def cached_host_blob(key, col_idx: torch.Tensor, row_off: torch.Tensor, nlat_in:
     except (OSError, ValueError):
         pass
     plan = build_host_blob(col_idx, row_off, nlat_in, nlon_in, nlat_out, nlon_out)
+    tmp = None
     try:
         os.makedirs(d, exist_ok=True)
         fd, tmp = tempfile.mkstemp(dir=d, suffix=".tmp")
         with os.fdopen(fd, "wb") as f:
             np.save(f, plan.blob.numpy(), allow_pickle=False)
         os.replace(tmp, path)  # atomic: a concurrent reader sees the old file or the whole new one
+        tmp = None
     except OSError:
         pass
+    finally:
+        if tmp is not None:  # a write that failed half way leaves nothing behind
+            try:
+                os.unlink(tmp)
+            except OSError:
+                pass
     return plan
 
 
