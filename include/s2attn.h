@@ -103,7 +103,7 @@ int s2attn_abi_version(void);
  * s2attn_plan_build   fills blob_out[blob_ints] (host memory; blob_ints as returned by s2attn_plan_size).
  */
 #define S2ATTN_PLAN_HEADER_INTS 32
-#define S2ATTN_PLAN_MAGIC 0x53324132 /* "S2A2" */
+#define S2ATTN_PLAN_MAGIC 0x53324133 /* "S2A3" */
 enum {
     S2ATTN_PH_MAGIC = 0,
     S2ATTN_PH_TOTAL = 1, /* ints in the blob */

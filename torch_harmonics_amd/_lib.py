@@ -25,7 +25,7 @@ _int = ctypes.c_int
 
 
 PLAN_HEADER_INTS = 32
-PLAN_MAGIC = 0x53324132
+PLAN_MAGIC = 0x53324133
 # index of each field in the plan header (include/s2attn.h, S2ATTN_PH_*)
 PH = dict(
     MAGIC=0, TOTAL=1, NVOUT=2, NVIN=3, NRUNS=4, GATHER_NDENSE=5, SCATTER_NDENSE=6,

@@ -145,9 +145,14 @@ int cost_class(int64_t c)
 // Two work lists (matrix-core-heavy and vector-heavy units, each most work first) merged in proportion to their work.
 // The kernels that treat long runs on the matrix cores and short runs on the vector ALU take this order: both kinds of
 // workgroups then sit side by side on a SIMD for the whole launch instead of one kind after the other (measured 6-7 %
-// on 721x1440 grids).  The long-run list is held back a little (its share of work handed out <= 0.7 of the other's):
-// measured best between 0.5 and 0.8, 1.5-2 % of the step over equal shares.
-template <typename Emit> void merge_by_share(const std::vector<int64_t> &cd_, const std::vector<int64_t> &cv_, Emit emit)
+// on 721x1440 grids).  `hold` bounds the long-run list's share of work handed out relative to the other list's.  Gather
+// grouping (forward, dq pass): 0.7, the long-run list held back a little (measured best between 0.5 and 0.8, 1.5-2 % of
+// the step over equal shares).  Scatter grouping (dk/dv pass): 1.2 - its long-run steps run on the bf16 matrix
+// instructions and cost less than the model's common weight says, so they are handed out a little ahead (dk/dv pass at
+// 721x1440 self-attention 4.47 -> 4.38 ms, 4.60 -> 4.45 on unstructured inputs; 2.0 gives the same there but costs the
+// 721x1440 -> 360x720 down-sampling 5 %; the dq pass loses 3 % with values above 1).
+constexpr double HOLD_GATHER = 0.7, HOLD_SCATTER = 1.2;
+template <typename Emit> void merge_by_share(const std::vector<int64_t> &cd_, const std::vector<int64_t> &cv_, double hold, Emit emit)
 {
     double wd = 0, wv = 0;
     for (int64_t c : cd_) wd += (double)c;
@@ -155,7 +160,7 @@ template <typename Emit> void merge_by_share(const std::vector<int64_t> &cd_, co
     size_t i = 0, j = 0;
     double cd = 0, cv = 0;
     while (i < cd_.size() || j < cv_.size()) {
-        const bool take_dense = j >= cv_.size() || (i < cd_.size() && cd * wv <= 0.7 * cv * wd);
+        const bool take_dense = j >= cv_.size() || (i < cd_.size() && cd * wv <= hold * cv * wd);
         if (take_dense) {
             cd += (double)cd_[i];
             emit(true, i++);
@@ -166,7 +171,7 @@ template <typename Emit> void merge_by_share(const std::vector<int64_t> &cd_, co
     }
 }
 
-int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order, int32_t *mixed)
+int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order, int32_t *mixed, double hold)
 {
     const int n = (int)cost.size();
     std::vector<int32_t> dense, vec;
@@ -179,7 +184,7 @@ int32_t order_rows(const std::vector<RowCost> &cost, int32_t *order, int32_t *mi
     for (int32_t r : dense) cd.push_back(cost[r].dense);
     for (int32_t r : vec) cv.push_back(cost[r].vector);
     int32_t *out = mixed;
-    merge_by_share(cd, cv, [&](bool d, size_t k) { *out++ = d ? dense[k] : vec[k]; });
+    merge_by_share(cd, cv, hold, [&](bool d, size_t k) { *out++ = d ? dense[k] : vec[k]; });
     return (int32_t)dense.size();
 }
 
@@ -272,7 +277,7 @@ void build_items(const int32_t *off, const int32_t *runs, int ngroups, int W, bo
     std::vector<int64_t> cd, cv;
     for (const Unit &u : dense) cd.push_back(u.c);
     for (const Unit &u : vec) cv.push_back(u.c);
-    merge_by_share(cd, cv, [&](bool d, size_t k) {
+    merge_by_share(cd, cv, scatter ? HOLD_SCATTER : HOLD_GATHER, [&](bool d, size_t k) {
         const Unit &u = d ? dense[k] : vec[k];
         items->push_back(u.lat);
         items->push_back(u.pair);
@@ -340,8 +345,8 @@ int build_blob(const int64_t *col_idx, const int64_t *row_off, int64_t nnz, int 
         gspan[2 * r + 1] = n_;
     }
     std::vector<int32_t> gorder(nvout), gmixed(nvout), sorder(nvin), smixed(nvin);
-    const int32_t gnd = order_rows(gcost, gorder.data(), gmixed.data());
-    const int32_t snd = order_rows(scost, sorder.data(), smixed.data());
+    const int32_t gnd = order_rows(gcost, gorder.data(), gmixed.data(), HOLD_GATHER);
+    const int32_t snd = order_rows(scost, sorder.data(), smixed.data(), HOLD_SCATTER);
     std::vector<int32_t> gitems, gpoff, gpruns, sitems, spoff, spruns;
     build_items(goff.data(), gruns.data(), nvout, W, false, gcost, &gitems, &gpoff, &gpruns);
     build_items(soff.data(), sruns.data(), nvin, W, true, scost, &sitems, &spoff, &spruns);
