@@ -317,6 +317,29 @@ def test_product_neighborhood_equals_oracle(ins, outs, gi, go, tc):
     assert torch.equal(row, torch.repeat_interleave(torch.arange(outs[0]), roff[1:] - roff[:-1]))
 
 
+def test_product_neighborhood_equals_oracle_on_random_small_grids():
+    """Degenerate and odd cases of the arc construction: one to five latitudes, one to four longitudes, cutoffs from nothing to
+    beyond the sphere, every grid kind, longitude ratios 1-4 in both directions; element-equal to the oracle's psi."""
+    import random
+
+    rng = random.Random(2024)
+    grids = ["equiangular", "legendre-gauss", "lobatto"]
+    checked = 0
+    for _ in range(150):
+        Hi, Ho = rng.choice([2, 3, 4, 5, 7, 8, 12, 16, 23, 32]), rng.choice([2, 3, 4, 5, 7, 8, 12, 16, 23, 32])
+        ratio, small = rng.choice([1, 1, 2, 3, 4]), rng.choice([1, 2, 3, 4, 6, 8, 16, 24, 33, 48])
+        big = (Hi, small * ratio), (Ho, small)
+        gi, go = rng.choice(grids), rng.choice(grids)
+        tc = rng.choice([None, 1e-6, 0.01, 0.05, 0.1, 0.3, 0.7, 1.5, 3.0, 3.2, 7.0, math.pi * rng.random()])
+        args = (big[0], big[1], gi, go) if rng.random() < 0.5 else (big[1], big[0], go, gi)  # psi is always built with nlon_in a multiple of nlon_out or the reverse
+        want_col, want_off = ogeo.neighborhood_csr(*args, tc)
+        col, off, row = precompute_neighborhood_s2(*args, tc)
+        assert torch.equal(col, want_col) and torch.equal(off, want_off), (args, tc)
+        assert torch.equal(row, torch.repeat_interleave(torch.arange(off.numel() - 1), off[1:] - off[:-1]))
+        checked += 1
+    assert checked == 150
+
+
 @pytest.mark.parametrize(
     "ins,outs,gi,go,tc,nnz,lens",
     [
