@@ -26,8 +26,9 @@
  * on the same tensors); heads wider than 128 channels and unscaled N(0,1) queries are as exact as a plain fp32 CPU evaluation
  * of the same inputs (4.2e-5 absolute on values of magnitude 3 at 512 channels), with dv of the head-dim-32 kernels up to
  * 1.2e-6 beyond 1e-5 on such a query; heads of 64 and more channels with neighborhoods of a few points, one of them dominant:
- * dq up to 5e-6 beyond 1e-5 on values of magnitude 30-70, as far as a plain fp32 CPU evaluation is off there.  16-bit storage: within 2e-2 of each tensor's RMS (arithmetic in fp32, operands of the
- * matrix instructions in the storage type).
+ * dq up to 5e-6 beyond 1e-5 on values of magnitude 30-70, as far as a plain fp32 CPU evaluation is off there.  16-bit storage (arithmetic in fp32, P and dS enter the
+ * matrix instructions in the storage type): fp16 within 2e-2 |x| + 2e-2 RMS per element; bf16 the same on typical problems, single
+ * elements of dq (wide heads) and dk (sums over many queries of both signs) up to 0.2 RMS off in a sweep of random problems.
  */
 #ifndef S2ATTN_H
 #define S2ATTN_H
