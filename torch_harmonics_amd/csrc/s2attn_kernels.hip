@@ -1909,8 +1909,11 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     const size_t pt = (size_t)query_point(a, b, ho, ho / a.qps) + (size_t)(w0 + (mine ? j : 0)) * a.qps;
     const size_t sidx = ((size_t)bh * a.Ho + ho) * a.Wo + w0 + (mine ? j : 0);
 
+    // The loads of this point's q, dy and y rows are issued here; what is computed from them (I = <dy, y>, which waits for
+    // them) comes after the first tile's loads have been issued too, so that the wavefront starts with one memory round trip
+    // instead of two in a row.
     float qb[16], gb[16];
-    float I = 0.f;
+    float4 yv[4];
     {
         const T *qrow = static_cast<const T *>(a.q) + pt * a.ldq + (size_t)h * 32 + 4 * half;
         const T *grow = static_cast<const T *>(a.dy) + pt * a.ldg + (size_t)h * 32 + 4 * half;
@@ -1919,15 +1922,10 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
         for (int g = 0; g < 4; g++) {
             const float4 x = load4(qrow + 8 * g);
             const float4 z = load4(grow + 8 * g);
-            const float4 yv = load4(yrow + 8 * g);
-            qb[4 * g] = x.x * LOG2E, qb[4 * g + 1] = x.y * LOG2E, qb[4 * g + 2] = x.z * LOG2E, qb[4 * g + 3] = x.w * LOG2E;
+            yv[g] = load4(yrow + 8 * g);
+            qb[4 * g] = x.x, qb[4 * g + 1] = x.y, qb[4 * g + 2] = x.z, qb[4 * g + 3] = x.w;
             gb[4 * g] = z.x, gb[4 * g + 1] = z.y, gb[4 * g + 2] = z.z, gb[4 * g + 3] = z.w;
-            I = fmaf(z.x, yv.x, I);
-            I = fmaf(z.y, yv.y, I);
-            I = fmaf(z.z, yv.z, I);
-            I = fmaf(z.w, yv.w, I);
         }
-        I = xor32_sum(I);
     }
     float lse = a.lse[sidx];
     f16v dqt;
@@ -1948,6 +1946,20 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     if (ri < rend) {
         run = a.gruns[ri];
         fetch(run, 0);
+    }
+    __builtin_amdgcn_sched_barrier(0);
+    float I = 0.f;
+#pragma unroll
+    for (int g = 0; g < 4; g++) {
+        I = fmaf(gb[4 * g], yv[g].x, I);
+        I = fmaf(gb[4 * g + 1], yv[g].y, I);
+        I = fmaf(gb[4 * g + 2], yv[g].z, I);
+        I = fmaf(gb[4 * g + 3], yv[g].w, I);
+    }
+    I = xor32_sum(I);
+#pragma unroll
+    for (int v = 0; v < 16; v++) qb[v] *= LOG2E;
+    if (ri < rend) {
         kt.commit(Ks, lane, !run_is_dense(run.len));
         vt.commit(Vs, lane, !run_is_dense(run.len));
     }
@@ -1956,18 +1968,31 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
     settle(gb);
     settle(lse);
 
+    // Run descriptors and quadrature weights are read a run ahead of their use (`ahead` is the run after `run`, `w` arrives
+    // with the run it belongs to): a scalar load at the top of the loop would be waited for right there, in front of the
+    // addresses of the next tile's loads, on every short run.
+    Run ahead = run;
+    float w = 0.f;
+    if (ri < rend) w = a.quad_w[run.pad];
+    if (ri + 1 < rend) ahead = a.gruns[ri + 1];
     while (ri < rend) {
-        const float w = a.quad_w[run.pad];
         const int len = run.len;
         int nri = ri, npos = pos + run_stride(len);
         Run nrun = run;
-        if (run_done(len, npos)) {
+        const bool adv = run_done(len, npos);
+        if (adv) {
             nri++;
             npos = 0;
-            if (nri < rend) nrun = a.gruns[nri];
+            if (nri < rend) nrun = ahead;
         }
         const bool more = nri < rend;
         if (more) fetch(nrun, npos);
+        Run ahead2 = ahead;
+        float wn = w;
+        if (adv && more) {
+            wn = a.quad_w[nrun.pad];
+            if (nri + 1 < rend) ahead2 = a.gruns[nri + 1];
+        }
 
         const float *kq = Ks + j * MLK + 4 * half;
         const float *vq = Vs + j * MLK + 4 * half;
@@ -2040,6 +2065,8 @@ template <typename T> __global__ __launch_bounds__(64) void dq_saved_mfma_kernel
         ri = nri;
         pos = npos;
         run = nrun;
+        ahead = ahead2;
+        w = wn;
     }
 
     // (stored after the walk: a global store ahead of the loop would turn the loop's scalar loads of runs and weights,
