@@ -98,7 +98,10 @@ def _disk_cache_dir():
     an empty string or "off" (no caching)."""
     d = os.environ.get("S2ATTN_CACHE_DIR")
     if d is None:
-        d = os.path.join(os.path.expanduser("~"), ".cache", "torch_harmonics_amd")
+        home = os.path.expanduser("~")
+        if not os.path.isabs(home):  # no home directory known: no default cache (never a directory named "~" under the working directory)
+            return None
+        d = os.path.join(home, ".cache", "torch_harmonics_amd")
     return None if d in ("", "off") else d
 
 
